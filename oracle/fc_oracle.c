@@ -1,0 +1,371 @@
+/*
+ * fc_oracle.c — epilogues, repack, weight compression, mat-vec and MLP of the CPU oracle.
+ * TEST INFRASTRUCTURE ONLY (see fc_oracle.h).
+ *
+ * Built with -ffp-contract=off: every multiply and add below rounds separately, exactly as
+ * the reference's separate AVX-512 mul/add instructions do; fused operations are written
+ * out as fmaf() where the reference uses an fmadd instruction.
+ */
+#include "fc_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* ------------------------------------------------------------------------------------ */
+/* bf16: include/bf16.hpp:91-102 (round_to_nearest_even) for normal numbers, which is also
+ * what vcvtne2ps2bf16 (include/kernels_amx.hpp:654) produces; the instruction additionally
+ * treats fp32 denormals as zero and quiets NaNs, which the bit formula alone would not. */
+uint16_t orc_f32_to_bf16(float x) {
+    uint32_t u = f2u(x);
+    if ((u & 0x7f800000u) == 0x7f800000u && (u & 0x007fffffu)) return (uint16_t)((u >> 16) | 0x0040u);
+    if ((u & 0x7f800000u) == 0) return (uint16_t)((u >> 16) & 0x8000u);
+    uint32_t bias = 0x00007fffu + ((u >> 16) & 1u);
+    return (uint16_t)((u + bias) >> 16);
+}
+/* include/bf16.hpp:70-76 */
+float orc_bf16_to_f32(uint16_t b) { return u2f((uint32_t)b << 16); }
+void orc_f32_to_bf16_n(const float* s, uint16_t* d, size_t n) { for (size_t i = 0; i < n; i++) d[i] = orc_f32_to_bf16(s[i]); }
+void orc_bf16_to_f32_n(const uint16_t* s, float* d, size_t n) { for (size_t i = 0; i < n; i++) d[i] = orc_bf16_to_f32(s[i]); }
+
+/* ------------------------------------------------------------------------------------ */
+/* include/kernels_amx.hpp:242-289 — oneDNN's gelu_erf minimax polynomial.
+ * x*0.5*(1 + x*P(x^2)), Horner with fused multiply-adds, then three selects. */
+float orc_gelu(float x) {
+    static const uint32_t coef[15] = {
+        0x1f1c83fdu, 0xa3198977u, 0x268a7927u, 0xa998c963u, 0x2c67ddb2u, 0xaf013b2cu, 0x315d4a4fu, 0xb3969b11u,
+        0x35a776e9u, 0xb79b0914u, 0x3970b255u, 0xbb1b7399u, 0x3ca3621fu, 0xbe082bc7u, 0x3f4c4228u};
+    const float x2 = x * x;
+    const float x_pos = u2f(f2u(x) & 0x7fffffffu);
+    const float x_half = x * 0.5f;
+    float poly = u2f(coef[0]);
+    for (int i = 1; i < 15; i++) poly = fmaf(poly, x2, u2f(coef[i]));
+    poly = fmaf(poly, x, 1.0f);
+    poly = poly * x_half;
+    /* cmpnlt: "not (x < -5)" is true for NaN, so NaN stays NaN */
+    if (x < u2f(0xc0a00000u)) x = 0.0f;
+    /* cmpnle: "not (|x| <= 5)" */
+    if (!(x_pos <= u2f(0x40a00000u))) poly = x;
+    if (x_pos <= u2f(0x33800000u)) poly = x_half;
+    return poly;
+}
+void orc_gelu_n(const float* s, float* d, size_t n) { for (size_t i = 0; i < n; i++) d[i] = orc_gelu(s[i]); }
+
+/* vcvtps2dq under the default MXCSR (round to nearest even; out of range or NaN gives the
+ * "integer indefinite" 0x80000000), then vpmovsdb signed saturation
+ * (include/kernels_amx.hpp:658-661). */
+static inline int8_t cvt_f32_to_s8_sat(float r) {
+    int32_t d;
+    if (!(r >= -2147483648.0f && r < 2147483648.0f)) d = INT32_MIN;
+    else d = (int32_t)nearbyintf(r);
+    if (d > 127) d = 127;
+    if (d < -128) d = -128;
+    return (int8_t)d;
+}
+
+/* include/kernels_amx.hpp:586-672 — BiasGeluStore::operator(): per element
+ *   [cvt i32->f32] [x deq] [+ bias[n]] [gelu] [x q[n]]  then store as bf16 / int8 / fp32.
+ * Extension (not in the reference): deq_per_oc[n] replaces the per-tensor deq_scale, same
+ * position in the chain, still one rounded multiply. */
+static inline void pp_store(float r, int n, const orc_pp* pp, void* crow) {
+    if (pp->steps & ORC_PP_DEQUANT) r = r * (pp->deq_per_oc ? pp->deq_per_oc[n] : pp->deq_scale);
+    if (pp->steps & ORC_PP_BIAS) r = r + pp->bias[n];
+    if (pp->steps & ORC_PP_GELU) r = orc_gelu(r);
+    if (pp->steps & ORC_PP_QUANT) r = r * (pp->q_per_oc ? pp->q_per_oc[n] : pp->q_scale);
+    switch (pp->out_dtype) {
+    case ORC_BF16: ((uint16_t*)crow)[n] = orc_f32_to_bf16(r); break;
+    case ORC_I8: ((int8_t*)crow)[n] = cvt_f32_to_s8_sat(r); break;
+    default: ((float*)crow)[n] = r; break;
+    }
+}
+
+void orc_pp_f32(const float* acc, int64_t ldacc, int M, int N, const orc_pp* pp, void* C, int64_t ldc_bytes) {
+#pragma omp parallel for schedule(static)
+    for (int m = 0; m < M; m++) {
+        void* crow = (char*)C + (size_t)m * ldc_bytes;
+        for (int n = 0; n < N; n++) pp_store(acc[(size_t)m * ldacc + n], n, pp, crow);
+    }
+}
+
+void orc_pp_i32(const int32_t* acc, int64_t ldacc, int M, int N, const orc_pp* pp, void* C, int64_t ldc_bytes) {
+#pragma omp parallel for schedule(static)
+    for (int m = 0; m < M; m++) {
+        void* crow = (char*)C + (size_t)m * ldc_bytes;
+        /* vcvtdq2ps: int32 -> fp32, round to nearest even (include/kernels_amx.hpp:631-634) */
+        for (int n = 0; n < N; n++) pp_store((float)acc[(size_t)m * ldacc + n], n, pp, crow);
+    }
+}
+
+/* ------------------------------------------------------------------------------------ */
+/* include/kernels_amx.hpp:761-816 (repackB_1x2) with kpack_tile_B0B1 (:293-454) and the
+ * 16x16 dword transposes (:114-238).  Closed form of where element (k, n) lands:
+ *   g = 4/elesz (elements per 32-bit group), kStep = 64/elesz,
+ *   panel row n/32, each panel K_pad*32 elements;
+ *   offset = kb*(kStep*32) + ((n%32)/16)*(kStep*16) + (krel/g)*(16*g) + (n%16)*g + krel%g,
+ *   with kb = k/kStep, krel = k%kStep for full blocks; in the K-tail block the rows are
+ *   bottom-aligned (krel = k - (K - kStep)) under zero rows (:326-338, :415-425, :793-800). */
+size_t orc_repack_amx_bytes(int elesz, int K, int N) {
+    const int kStep = 64 / elesz;
+    const size_t Kp = (size_t)(K + kStep - 1) / kStep * kStep;
+    const size_t Npan = (size_t)(N + 31) / 32;
+    return Npan * Kp * 32 * elesz;
+}
+
+void orc_repack_amx(int elesz, const void* B, int64_t ldb_bytes, int K, int N, int transpose, void* out) {
+    const int g = 4 / elesz, kStep = 64 / elesz;
+    const int Kp = (K + kStep - 1) / kStep * kStep;
+    const int Kbody = K - (K % kStep);
+    memset(out, 0, orc_repack_amx_bytes(elesz, K, N));
+    for (int n = 0; n < N; n++) {
+        for (int k = 0; k < K; k++) {
+            int kb, krel;
+            if (k < Kbody) { kb = k / kStep; krel = k % kStep; }
+            else { kb = Kbody / kStep; krel = k - (K - kStep); }
+            size_t off = (size_t)(n / 32) * ((size_t)Kp * 32) + (size_t)kb * (kStep * 32) +
+                         (size_t)((n % 32) / 16) * (kStep * 16) + (size_t)(krel / g) * (16 * g) +
+                         (size_t)(n % 16) * g + (krel % g);
+            const char* src = transpose ? (const char*)B + (size_t)n * ldb_bytes + (size_t)k * elesz
+                                        : (const char*)B + (size_t)k * ldb_bytes + (size_t)n * elesz;
+            memcpy((char*)out + off * elesz, src, elesz);
+        }
+    }
+}
+
+/* This project's device layout (no counterpart in the reference): the unit an MFMA consumes
+ * as its B operand — 64 lanes x 16 bytes — is contiguous, units are ordered panel-major
+ * then K, exactly the idea of include/kernels_amx.hpp:456-463 applied to gfx950. */
+size_t orc_repack_mfma_bytes(int elesz, int K, int N) {
+    const int kalign = 128 / elesz;
+    const size_t Kp = (size_t)(K + kalign - 1) / kalign * kalign;
+    const size_t Npan = (size_t)(N + 31) / 32;
+    return Npan * Kp * 32 * elesz;
+}
+
+void orc_repack_mfma(int elesz, const void* B, int64_t ldb_bytes, int K, int N, int transpose, void* out) {
+    const int KS = 32 / elesz;   /* k per 1 KiB fragment: bf16 16, int8 32 */
+    const int half = KS / 2;     /* k per lane */
+    const int kalign = 128 / elesz;
+    const int Kp = (K + kalign - 1) / kalign * kalign;
+    memset(out, 0, orc_repack_mfma_bytes(elesz, K, N));
+    for (int n = 0; n < N; n++) {
+        for (int k = 0; k < K; k++) {
+            const int lane = (n % 32) + 32 * ((k % KS) / half);
+            size_t off_bytes = ((size_t)(n / 32) * (Kp / KS) + (size_t)(k / KS)) * 1024 + (size_t)lane * 16 +
+                               (size_t)(k % half) * elesz;
+            const char* src = transpose ? (const char*)B + (size_t)n * ldb_bytes + (size_t)k * elesz
+                                        : (const char*)B + (size_t)k * ldb_bytes + (size_t)n * elesz;
+            memcpy((char*)out + off_bytes, src, elesz);
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------------------ */
+/* include/kernels_amx.hpp:1363-1377 with get_min_max (:465-488) and bf16_to_i8_tensor
+ * (:508-523): scale = 127/max|w| over the whole matrix, q = sat8(rne(w*scale)). */
+float orc_quantize_weights(const uint16_t* W, int64_t ldw, int rows, int cols, int8_t* Wq, int64_t ldq,
+                           float* quant_scale) {
+    float mx = -__FLT_MAX__, mn = __FLT_MAX__;
+    for (int r = 0; r < rows; r++)
+        for (int c = 0; c < cols; c++) {
+            float v = orc_bf16_to_f32(W[(size_t)r * ldw + c]);
+            if (v > mx) mx = v;
+            if (v < mn) mn = v;
+        }
+    float amax = fabsf(mx) > fabsf(mn) ? fabsf(mx) : fabsf(mn);
+    const float q = 127 / amax;
+    const float dq = amax / 127;
+    for (int r = 0; r < rows; r++)
+        for (int c = 0; c < cols; c++)
+            Wq[(size_t)r * ldq + c] = cvt_f32_to_s8_sat(orc_bf16_to_f32(W[(size_t)r * ldw + c]) * q);
+    if (quant_scale) *quant_scale = q;
+    return dq;
+}
+
+/* weight_compression/fc16m.cpp:451-502 (matmul16m_Wint8B) and include/kernels_amx.hpp:1381-1441:
+ * int8 weights are converted to bf16 exactly (|w| <= 128 needs 8 significant bits;
+ * include/kernels_amx.hpp:490-506, fc16m.cpp:309-333) and fed to the same tdpbf16ps chain, the
+ * scale is applied to the fp32 result afterwards (fc16m.cpp:496-500 per tensor; here per
+ * output channel, one rounded multiply), then rounded to bf16. */
+void orc_gemv_w8(const uint16_t* x, int64_t ldx, const int8_t* Wq, int64_t ldw, int transW, const float* scale,
+                 uint16_t* y, int64_t ldy, float* acc_out, int M, int K, int N, int nthreads) {
+    const int rows = transW ? N : K, cols = transW ? K : N;
+    uint16_t* Wb = (uint16_t*)malloc((size_t)rows * cols * sizeof(uint16_t));
+    float* acc = (float*)malloc((size_t)M * N * sizeof(float));
+    if (!Wb || !acc) abort();
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < rows; r++)
+        for (int c = 0; c < cols; c++) Wb[(size_t)r * cols + c] = orc_f32_to_bf16((float)Wq[(size_t)r * ldw + c]);
+    orc_gemm_bf16(x, ldx, Wb, cols, transW, acc, N, M, K, N, nthreads);
+    for (int m = 0; m < M; m++)
+        for (int n = 0; n < N; n++) y[(size_t)m * ldy + n] = orc_f32_to_bf16(acc[(size_t)m * N + n] * scale[n]);
+    if (acc_out) memcpy(acc_out, acc, (size_t)M * N * sizeof(float));
+    free(Wb);
+    free(acc);
+}
+
+/* ------------------------------------------------------------------------------------ */
+/* include/kernels_amx.hpp:854-1042 — MatmulVector: the same tdpbf16ps chain with a
+ * one-column B.  Full 16-row groups read the K tail left-aligned at Kbody (B zero padded
+ * below, :874-880); the last group of rows reads it right-aligned at K-32 (B zero padded
+ * above, :866-872) — the tail products then sit at different slots of the tile, which
+ * changes which of the two partial sums they join when K is odd.  The reference's dispatch
+ * is wrong for more than four K tiles (:939-953); this follows the intended product. */
+void orc_matvec_bf16(const uint16_t* A, int64_t lda, const uint16_t* b, float* c, int M, int K) {
+    const int Ktail = K & 31, Kbody = K - Ktail;
+    int Mtail = M & 15, Mbody = M - Mtail;
+    if (Ktail && Mtail == 0) { Mtail = 16; Mbody -= 16; }
+    for (int m = 0; m < M; m++) {
+        const uint16_t* a = A + (size_t)m * lda;
+        float acc = 0.0f;
+        for (int kb = 0; kb < Kbody; kb += 32) {
+            float p0 = 0.0f, p1 = 0.0f;
+            for (int p = 0; p < 32; p += 2) {
+                p0 += orc_bf16_to_f32(a[kb + p]) * orc_bf16_to_f32(b[kb + p]);
+                p1 += orc_bf16_to_f32(a[kb + p + 1]) * orc_bf16_to_f32(b[kb + p + 1]);
+            }
+            acc += (p0 + p1);
+        }
+        if (Ktail) {
+            const int t0 = (m < Mbody) ? Kbody : K - 32;
+            float p0 = 0.0f, p1 = 0.0f;
+            for (int k = Kbody; k < K; k++) {
+                float pr = orc_bf16_to_f32(a[k]) * orc_bf16_to_f32(b[k]);
+                if ((k - t0) & 1) p1 += pr; else p0 += pr;
+            }
+            acc += (p0 + p1);
+        }
+        c[m] = acc;
+    }
+}
+
+/* include/kernels_amx.hpp:1529-1618 — GemAvB: vdpbf16ps on k pairs, pair i of each 32-block
+ * goes to accumulator i&1 (:1595-1610), the two are added at the end (:1612).  vdpbf16ps
+ * adds the odd element's product first, then the even one, each with one rounding. */
+void orc_gemavb_bf16(const uint16_t* A, int64_t lda, const uint16_t* b, float* c, int M, int K) {
+    for (int m = 0; m < M; m++) {
+        const uint16_t* a = A + (size_t)m * lda;
+        float acc[2] = {0.0f, 0.0f};
+        for (int k = 0; k < K; k += 2) {
+            const int which = (k >> 1) & 1;
+            float odd = (k + 1 < K) ? orc_bf16_to_f32(a[k + 1]) * orc_bf16_to_f32(b[k + 1]) : 0.0f;
+            float even = orc_bf16_to_f32(a[k]) * orc_bf16_to_f32(b[k]);
+            float t = acc[which] + odd;
+            acc[which] = t + even;
+        }
+        c[m] = acc[0] + acc[1];
+    }
+}
+
+void orc_matvec_i8(const int8_t* A, int64_t lda, const int8_t* b, int32_t* c, int M, int K) {
+    for (int m = 0; m < M; m++) {
+        int32_t acc = 0;
+        for (int k = 0; k < K; k++) acc += (int32_t)A[(size_t)m * lda + k] * (int32_t)b[k];
+        c[m] = acc;
+    }
+}
+
+/* ------------------------------------------------------------------------------------ */
+/* tests/amx-mlp.cpp:383-448 — exp_ps_avx512: clamp, n = floor(x*log2e + 0.5),
+ * r = x - n*ln2 (fused), degree-5 polynomial (fused), times 2^(n-1), times 2. */
+float orc_exp_poly(float x) {
+    const float ln_flt_min = u2f(0xc2aeac50u), ln_flt_max = u2f(0x42b17218u);
+    const float log2ef = u2f(0x3fb8aa3bu), ln2f = u2f(0x3f317218u);
+    const float p1 = u2f(0x3f7ffffbu), p2 = u2f(0x3efffee3u), p3 = u2f(0x3e2aad40u), p4 = u2f(0x3d2b9d0du),
+                p5 = u2f(0x3c07cfceu);
+    const int zero = x < ln_flt_min;
+    float s = x;
+    s = (s < ln_flt_max) ? s : ln_flt_max; /* vminps(src, max): returns max unless src < max */
+    s = (s > ln_flt_min) ? s : ln_flt_min;
+    float aux1 = s;
+    s = s * log2ef;
+    s = s + 0.5f;
+    s = floorf(s);
+    aux1 = fmaf(-s, ln2f, aux1);
+    s = s - 1.0f;
+    int32_t e = (int32_t)nearbyintf(s);
+    e = (int32_t)((uint32_t)(e + 127) << 23);
+    float aux2 = zero ? 0.0f : u2f((uint32_t)e);
+    s = p5;
+    s = fmaf(s, aux1, p4);
+    s = fmaf(s, aux1, p3);
+    s = fmaf(s, aux1, p2);
+    s = fmaf(s, aux1, p1);
+    s = fmaf(s, aux1, 1.0f);
+    s = s * aux2;
+    s = s * 2.0f;
+    return s;
+}
+
+/* tests/amx-mlp.cpp:450-456 — silu(x) = x * rcp(1 + exp(-x)).  The reference's rcp is
+ * vrcp14ps (relative error < 2^-14, Intel-specific bits); here it is the correctly rounded
+ * reciprocal.  See the pinning note in fc_oracle.h. */
+float orc_silu(float x) {
+    float e = orc_exp_poly(0.0f - x);
+    float sig = 1.0f / (1.0f + e);
+    return x * sig;
+}
+
+/* tests/amx-mlp.cpp:720-734 — runGateUp epilogue: bf16( silu(gate) * up ) */
+void orc_silu_mul_bf16(const float* gate, const float* up, uint16_t* h, size_t n) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; i++) h[i] = orc_f32_to_bf16(orc_silu(gate[i]) * up[i]);
+}
+
+/* tests/amx-mlp.cpp:648-704 with the partition at :546-593 — down_proj.  With split-K the K
+ * blocks of 256 are cut into a first half of ceil(nblk/2) blocks and the rest; each half is
+ * accumulated on its own (first block starts from zero, later blocks accumulate into the
+ * fp32 C, :199-334), the halves are added (:676-677) and rounded to bf16 (:678). */
+void orc_mlp_down(const uint16_t* h, const uint16_t* w_down, uint16_t* y, int M, int Kout, int N, int split_k,
+                  int nthreads) {
+    float* p0 = (float*)malloc((size_t)M * Kout * sizeof(float));
+    float* p1 = NULL;
+    if (!p0) abort();
+    int n_first = N;
+    if (split_k && (N % 256) == 0 && N >= 512) {
+        const int nblk = N / 256;
+        n_first = ((nblk + 1) / 2) * 256;
+    }
+    orc_gemm_bf16(h, N, w_down, N, 1, p0, Kout, M, n_first, Kout, nthreads);
+    if (n_first < N) {
+        p1 = (float*)malloc((size_t)M * Kout * sizeof(float));
+        if (!p1) abort();
+        orc_gemm_bf16(h + n_first, N, w_down + n_first, N, 1, p1, Kout, M, N - n_first, Kout, nthreads);
+    }
+    for (size_t i = 0; i < (size_t)M * Kout; i++) y[i] = orc_f32_to_bf16(p1 ? (p0[i] + p1[i]) : p0[i]);
+    free(p0);
+    free(p1);
+}
+
+/* tests/amx-mlp.cpp:740-784 (MLP::setup / run) and :788-841 (mlp_ref):
+ *   h = bf16(silu(x·Wg^T) * (x·Wu^T)),  y = bf16(h·Wd^T) */
+void orc_mlp(const uint16_t* x, const uint16_t* w_gate, const uint16_t* w_up, const uint16_t* w_down,
+             uint16_t* h_out, uint16_t* y, int M, int K, int N, int split_k, int nthreads) {
+    float* g = (float*)malloc((size_t)M * N * sizeof(float));
+    float* u = (float*)malloc((size_t)M * N * sizeof(float));
+    uint16_t* h = h_out ? h_out : (uint16_t*)malloc((size_t)M * N * sizeof(uint16_t));
+    if (!g || !u || !h) abort();
+    orc_gemm_bf16(x, K, w_gate, K, 1, g, N, M, K, N, nthreads);
+    orc_gemm_bf16(x, K, w_up, K, 1, u, N, M, K, N, nthreads);
+    orc_silu_mul_bf16(g, u, h, (size_t)M * N);
+    orc_mlp_down(h, w_down, y, M, K, N, split_k, nthreads);
+    free(g);
+    free(u);
+    if (!h_out) free(h);
+}
+
+/* include/misc.hpp:521-535 */
+void orc_splitter(int n, int team, int tid, int* n_start, int* n_end) {
+    if (team <= 1 || n == 0) { *n_start = 0; *n_end = n; return; }
+    int n1 = (n + team - 1) / team;
+    int n2 = n1 - 1;
+    int T1 = n - n2 * team;
+    int len = tid < T1 ? n1 : n2;
+    *n_start = tid <= T1 ? tid * n1 : T1 * n1 + (tid - T1) * n2;
+    *n_end = *n_start + len;
+}
