@@ -1,0 +1,152 @@
+/*
+ * mm_amx_amd.h — C ABI of the MI355X (gfx950) fully-connected GEMM path.
+ *
+ * Plain C, device pointers and sizes only; every call is asynchronous on the HIP stream
+ * passed in (NULL = the default stream) and returns 0 on success or a negative MMX_E_* code,
+ * with a per-thread message available from mmx_last_error().  Nothing is thrown across this
+ * boundary.  No entry point allocates or frees device memory.
+ *
+ * The reference (usstq/mm_amx) has no FFI boundary of its own: its interface is a set of
+ * C++ templates in include/kernels_amx.hpp.  Each entry point below names the reference
+ * interface it stands in for; the C++ classes with the reference's names are layered on
+ * top of this ABI in include/mm_amx_amd/kernels_gfx950.hpp.
+ */
+#ifndef MM_AMX_AMD_H
+#define MM_AMX_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types */
+enum { MMX_F32 = 0, MMX_BF16 = 1, MMX_I8 = 2, MMX_I32 = 3 };
+
+/* error codes */
+enum {
+    MMX_OK = 0,
+    MMX_E_INVALID = -1,     /* bad argument (shape, alignment, null pointer, unknown dtype) */
+    MMX_E_UNSUPPORTED = -2, /* valid request this build has no kernel for */
+    MMX_E_HIP = -3,         /* a HIP runtime call failed */
+    MMX_E_DEVICE = -4       /* no gfx950 device */
+};
+
+/* Post-op steps: the values of amx_kernel::PP::Steps (include/kernels_amx.hpp:540-550),
+ * plus MMX_PP_SILU_GATE for the fused gate/up epilogue of tests/amx-mlp.cpp:707-737. */
+enum {
+    MMX_PP_NONE = 0,
+    MMX_PP_DEQUANT = 1,
+    MMX_PP_BIAS = 2,
+    MMX_PP_GELU = 4,
+    MMX_PP_QUANT = 8,
+    MMX_PP_SILU_GATE = 16
+};
+
+/*
+ * Epilogue descriptor — the data members of amx_kernel::PP::BiasGeluStore<D, steps>
+ * (include/kernels_amx.hpp:552-583) as plain data, because a host functor cannot be called
+ * per 32x32 block from a GPU kernel.  Applied per element, in this order, each step one
+ * correctly rounded fp32 operation (no fused multiply-add across steps):
+ *     r = float(acc)                          (int32 accumulators only, round-to-nearest-even)
+ *     r = r * deq                             MMX_PP_DEQUANT   deq = deq_scale_per_oc[n] if set, else deq_scale
+ *     r = r + bias[n]                         MMX_PP_BIAS
+ *     r = gelu_erf_minimax(r)                 MMX_PP_GELU      (include/kernels_amx.hpp:242-289)
+ *     r = r * q                               MMX_PP_QUANT     q = q_scale_per_oc[n] if set, else q_scale
+ *     store: MMX_F32 as is; MMX_BF16 round-to-nearest-even; MMX_I8 round-to-nearest-even then
+ *            saturate to [-128,127]; MMX_I32 (only with steps == 0 on int8 inputs) raw accumulator.
+ * With MMX_PP_SILU_GATE the packed weights hold gate and up projections in alternating
+ * 32-column panels (see mmx_repack_gate_up) and the output has half as many columns:
+ *     C[m, c] = bf16( silu(acc_gate[m, c]) * acc_up[m, c] )   (DEQUANT/BIAS/GELU/QUANT must be off)
+ * deq_scale_per_oc is an extension: the reference has a per-tensor dequant scale only.
+ */
+typedef struct mmx_epilogue {
+    uint32_t steps;
+    int32_t out_dtype;
+    void* C;            /* device, [M, n1-n0 columns starting at column n0 of the full C row] */
+    int64_t ldc_bytes;  /* row stride of C in bytes; C points at row 0, column 0 of the FULL matrix */
+    const float* bias;  /* device [N] */
+    float deq_scale;
+    const float* deq_scale_per_oc; /* device [N] or NULL */
+    float q_scale;
+    const float* q_scale_per_oc;   /* device [N] or NULL */
+} mmx_epilogue;
+
+/* message for the last failing call made by this thread ("" if none) */
+const char* mmx_last_error(void);
+
+/* Selects `device`, checks that it is a gfx950, raises kernel LDS limits.  Idempotent.
+ * Stands in for initXTILE() (include/misc.hpp:376-396), the reference's one-time set-up. */
+int mmx_init(int device);
+
+/* ---- weight repack: amx_kernel::repackB_1x2 (include/kernels_amx.hpp:761-816) --------------
+ * B is [K, N] (transpose = 0) or [N, K] (transpose = 1, the torch nn.Linear.weight layout),
+ * row stride ldb_bytes, dtype MMX_BF16 or MMX_I8.  The result is in MFMA-fragment order:
+ *     packed[panel = n/32][kstep = k/KS][lane 0..63][16 bytes],  KS = 16 (bf16) / 32 (int8),
+ *     lane = n%32 + 32*((k%KS)/(KS/2)),  byte offset in the lane = (k%(KS/2))*sizeof(T),
+ * zero padded in K up to a multiple of 128 bytes per column and in N up to a multiple of 32. */
+size_t mmx_packed_b_bytes(int dtype, int K, int N);
+int mmx_repack_b(int dtype, const void* B, int64_t ldb_bytes, int K, int N, int transpose, void* packed,
+                 void* stream);
+
+/* MLP::setup (tests/amx-mlp.cpp:752-766): interleaves W_gate and W_up (both [N, K] bf16,
+ * torch layout) into one packed matrix of 2N columns, alternating 32-column panels
+ * (gate panel p, up panel p), for use with MMX_PP_SILU_GATE.  N % 32 == 0. */
+int mmx_repack_gate_up(const void* w_gate, const void* w_up, int64_t ldw_bytes, int K, int N, void* packed,
+                       void* stream);
+
+/* Weight compression of amx_kernel::Matmul<bf16,int8,float> (include/kernels_amx.hpp:1363-1377,
+ * 465-523): per-tensor symmetric quantisation of a bf16 matrix [rows, cols] to int8, scale
+ * 127/max|w|.  scales_out (device, 2 floats) receives {quant_scale, dequant_scale};
+ * absmax_scratch is a device uint32 the call uses as scratch. */
+int mmx_quantize_weights(const void* W, int64_t ldw_bytes, int rows, int cols, void* Wq, int64_t ldq_bytes,
+                         float* scales_out, uint32_t* absmax_scratch, void* stream);
+
+/* int8 packed weights -> bf16 packed weights (exact), the on-the-fly dequant of
+ * include/kernels_amx.hpp:490-506 done once for the large-M weight-compressed path. */
+int mmx_dequant_packed(const void* packed_i8, int K, int N, void* packed_bf16, void* stream);
+
+/* ---- C[:, n0:n1] = PP( A · B[:, n0:n1] ): amx_kernel::Matmul<TA,TB,TC>::operator()
+ * (include/kernels_amx.hpp:1169-1314; int8-weight specialisation :1319-1516) -----------------
+ * a_dtype/b_dtype: (BF16,BF16), (I8,I8), or (BF16,I8) = bf16 activations on int8-compressed
+ * weights, dequantised in registers (M <= 32 only; larger M goes through mmx_dequant_packed).
+ * A is [M, K] row-major with row stride lda_bytes; Bpacked comes from mmx_repack_b for the
+ * FULL [K, N]; n0 % 32 == 0, 0 <= n0 < n1 <= N.  M <= 32 takes the bandwidth-bound decode
+ * kernel (the M<=16 paths of the reference and weight_compression/fc16m.cpp:451-502), larger
+ * M the MFMA tile kernel. */
+int mmx_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* Bpacked, int M, int K,
+             int N, int n0, int n1, const mmx_epilogue* ep, void* stream);
+
+/* ---- c[M] = A[M, K] · b[K]: amx_kernel::MatmulVector::operator() (include/kernels_amx.hpp:959)
+ * and amx_kernel::GemAvB::operator() (:1534).  dtype MMX_BF16 (c fp32) or MMX_I8 (c int32). */
+int mmx_matvec(int dtype, const void* A, int64_t lda_bytes, const void* b, void* c, int M, int K, void* stream);
+
+/* ---- fused Llama MLP: AMX_MLP::MLP::run (tests/amx-mlp.cpp:778-783) ---------------------------
+ * x [M, K] bf16; w_gate_up from mmx_repack_gate_up (K x 2N); w_down from mmx_repack_b of the
+ * [K, N] torch down_proj weight with transpose = 1 (so it is an N x K "B"); h is caller
+ * scratch [M, N] bf16; y [M, K] bf16.  Two launches on `stream`: gate/up GEMM with the SiLU*up
+ * epilogue, then down GEMM. */
+int mmx_mlp(const void* x, int64_t ldx_bytes, const void* w_gate_up, const void* w_down, void* h, int64_t ldh_bytes,
+            void* y, int64_t ldy_bytes, int M, int K, int N, void* stream);
+
+/* ---- introspection / tuning (no reference counterpart) --------------------------------------- */
+/* Force the MFMA tile shape ("256x256", "256x192", "128x256", "128x128", "" = automatic). */
+int mmx_set_tile(const char* shape);
+/* Name of the kernel variant the last mmx_gemm call of this thread launched. */
+const char* mmx_last_kernel(void);
+/* Sets a kernel option.  "load_mode": how the MFMA tile kernel brings A and B tiles into LDS —
+ * 0 through registers (default; always used when M/K tails or alignment need masking),
+ * 1 global_load_lds through the compiler builtin, 2 global_load_lds issued from inline asm. */
+int mmx_set_option(const char* name, int value);
+/* HIP-event timing of `iters` back-to-back launches of the given gemm on `stream`, launch i
+ * using the packed weights Bpacked_rot[i % n_rot] (rotate over several copies so that a
+ * bandwidth-bound shape is not served from cache); returns the average milliseconds per launch
+ * in *ms_out.  Other arguments as for mmx_gemm.  Blocks until the last launch has finished. */
+int mmx_time_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* const* Bpacked_rot, int n_rot,
+                  int M, int K, int N, int n0, int n1, const mmx_epilogue* ep, void* stream, int iters, float* ms_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

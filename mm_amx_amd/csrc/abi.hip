@@ -1,0 +1,267 @@
+// C ABI of the gfx950 FC-GEMM path: argument validation, dispatch, error reporting.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "common.hpp"
+
+namespace mmx {
+
+static thread_local char g_err[512] = "";
+static thread_local char g_kernel[128] = "";
+static int g_cus = 0;
+
+int set_error(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_hip(hipError_t e, const char* what) {
+    if (e == hipSuccess) return MMX_OK;
+    return set_error(MMX_E_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+void note_kernel(const char* name) {
+    strncpy(g_kernel, name, sizeof g_kernel - 1);
+    g_kernel[sizeof g_kernel - 1] = 0;
+}
+
+int num_cus() { return g_cus > 0 ? g_cus : 256; }
+
+int launch_gemm_tiles_bf16(const void* A, int64_t lda, const void* Bp, int M, int K, int N, int n0, int n1,
+                           const Epilogue& ep, hipStream_t st);
+int launch_gemm_tiles_i8(const void* A, int64_t lda, const void* Bp, int M, int K, int N, int n0, int n1,
+                         const Epilogue& ep, hipStream_t st);
+int launch_skinny(bool w8, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
+                  const Epilogue& ep, hipStream_t st);
+int launch_repack(int elesz, const void* B, int64_t ldb, int K, int N, int transpose, void* out, hipStream_t st);
+int launch_repack_gate_up(const void* wg, const void* wu, int64_t ldw, int K, int N, void* out, hipStream_t st);
+int launch_quantize(const void* W, int64_t ldw, int rows, int cols, void* Wq, int64_t ldq, float* scales_out,
+                    uint32_t* scratch, hipStream_t st);
+int launch_dequant_packed(const void* in, int K, int N, void* out, hipStream_t st);
+int launch_matvec(bool i8, const void* A, int64_t lda, const void* b, void* c, int M, int K, hipStream_t st);
+
+struct TileCfg {
+    int bm, bn;
+};
+static TileCfg g_forced = {0, 0};
+static int g_load_mode = 0;
+TileCfg forced_tile() { return g_forced; }
+int load_mode() { return g_load_mode; }
+
+static int elesz_of(int dtype) { return dtype == MMX_BF16 ? 2 : dtype == MMX_I8 ? 1 : 0; }
+
+static int out_size(int dtype) {
+    switch (dtype) {
+    case MMX_F32: case MMX_I32: return 4;
+    case MMX_BF16: return 2;
+    case MMX_I8: return 1;
+    default: return 0;
+    }
+}
+
+static int make_epilogue(const mmx_epilogue* in, int a_dtype, int b_dtype, int n0, Epilogue* out) {
+    if (!in) return set_error(MMX_E_INVALID, "epilogue descriptor is NULL");
+    if (!in->C) return set_error(MMX_E_INVALID, "epilogue: output pointer C is NULL");
+    const int sz = out_size(in->out_dtype);
+    if (!sz) return set_error(MMX_E_INVALID, "epilogue: unknown output dtype %d", in->out_dtype);
+    const uint32_t known = MMX_PP_DEQUANT | MMX_PP_BIAS | MMX_PP_GELU | MMX_PP_QUANT | MMX_PP_SILU_GATE;
+    if (in->steps & ~known) return set_error(MMX_E_INVALID, "epilogue: unknown step bits 0x%x", in->steps);
+    // the setters of BiasGeluStore assert that their step is enabled (include/kernels_amx.hpp:561-583);
+    // here the converse is enforced: an enabled step must have its operand
+    if ((in->steps & MMX_PP_BIAS) && !in->bias) return set_error(MMX_E_INVALID, "epilogue: BIAS step without a bias pointer");
+    if (in->steps & MMX_PP_SILU_GATE) {
+        if (in->steps != MMX_PP_SILU_GATE) return set_error(MMX_E_INVALID, "epilogue: SILU_GATE excludes every other step");
+        if (in->out_dtype != MMX_BF16 && in->out_dtype != MMX_F32)
+            return set_error(MMX_E_INVALID, "epilogue: SILU_GATE stores bf16 or fp32");
+        if (a_dtype != MMX_BF16) return set_error(MMX_E_INVALID, "epilogue: SILU_GATE needs bf16 activations");
+        if (n0 % 64) return set_error(MMX_E_INVALID, "epilogue: SILU_GATE needs n0 %% 64 == 0");
+    }
+    if (in->out_dtype == MMX_I32 && !(a_dtype == MMX_I8 && b_dtype == MMX_I8 && in->steps == 0))
+        return set_error(MMX_E_INVALID, "epilogue: int32 output is the raw accumulator of an int8 GEMM (steps must be 0)");
+    if (in->ldc_bytes % sz) return set_error(MMX_E_INVALID, "epilogue: ldc_bytes %lld is not a multiple of the element size", (long long)in->ldc_bytes);
+    if (reinterpret_cast<uintptr_t>(in->C) % sz) return set_error(MMX_E_INVALID, "epilogue: C is not aligned to its element size");
+    out->steps = in->steps;
+    out->out_dtype = in->out_dtype;
+    out->C = static_cast<char*>(in->C);
+    out->ldc = in->ldc_bytes;
+    out->bias = in->bias;
+    out->deq = in->deq_scale;
+    out->deq_oc = in->deq_scale_per_oc;
+    out->q = in->q_scale;
+    out->q_oc = in->q_scale_per_oc;
+    out->c_vec_ok = ((reinterpret_cast<uintptr_t>(in->C) & 15) == 0) && ((in->ldc_bytes & 15) == 0);
+    return MMX_OK;
+}
+
+static int gemm_dispatch(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* Bpacked, int M, int K,
+                         int N, int n0, int n1, const mmx_epilogue* ep_in, hipStream_t st) {
+    if (!A || !Bpacked) return set_error(MMX_E_INVALID, "mmx_gemm: NULL operand");
+    if (M <= 0 || K <= 0 || N <= 0) return set_error(MMX_E_INVALID, "mmx_gemm: M, K, N must be positive (got %d, %d, %d)", M, K, N);
+    const bool bf = a_dtype == MMX_BF16 && b_dtype == MMX_BF16;
+    const bool i8 = a_dtype == MMX_I8 && b_dtype == MMX_I8;
+    const bool w8 = a_dtype == MMX_BF16 && b_dtype == MMX_I8;
+    if (!bf && !i8 && !w8) return set_error(MMX_E_INVALID, "mmx_gemm: dtype pair (%d, %d) not supported", a_dtype, b_dtype);
+    if (n0 < 0 || n1 > N || n0 >= n1) return set_error(MMX_E_INVALID, "mmx_gemm: column range [%d, %d) outside [0, %d)", n0, n1, N);
+    // the reference splits N in units of 32 (main.cpp:461-471)
+    if (n0 % 32) return set_error(MMX_E_INVALID, "mmx_gemm: n0 = %d must be a multiple of 32", n0);
+    const int esa = elesz_of(a_dtype);
+    if (lda_bytes < (int64_t)K * esa) return set_error(MMX_E_INVALID, "mmx_gemm: lda_bytes %lld smaller than a row of A", (long long)lda_bytes);
+    if (lda_bytes % esa || reinterpret_cast<uintptr_t>(A) % esa) return set_error(MMX_E_INVALID, "mmx_gemm: A is not aligned to its element size");
+    if (reinterpret_cast<uintptr_t>(Bpacked) & 15) return set_error(MMX_E_INVALID, "mmx_gemm: packed weights must be 16-byte aligned");
+    Epilogue ep;
+    int rc = make_epilogue(ep_in, a_dtype, b_dtype, n0, &ep);
+    if (rc) return rc;
+    if ((ep.steps & MMX_PP_SILU_GATE) && ((n1 - n0) % 64)) return set_error(MMX_E_INVALID, "mmx_gemm: SILU_GATE needs (n1 - n0) %% 64 == 0");
+    if (M <= 32 && !i8) return launch_skinny(w8, A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st);
+    if (w8) return set_error(MMX_E_UNSUPPORTED, "mmx_gemm: bf16 x int8-weight with M > 32: convert the weights with mmx_dequant_packed and call the bf16 GEMM");
+    return i8 ? launch_gemm_tiles_i8(A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st)
+              : launch_gemm_tiles_bf16(A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st);
+}
+
+}  // namespace mmx
+
+using namespace mmx;
+
+extern "C" {
+
+const char* mmx_last_error(void) { return g_err; }
+const char* mmx_last_kernel(void) { return g_kernel; }
+
+int mmx_init(int device) {
+    int count = 0;
+    int rc = check_hip(hipGetDeviceCount(&count), "hipGetDeviceCount");
+    if (rc) return rc;
+    if (device < 0 || device >= count) return set_error(MMX_E_DEVICE, "mmx_init: device %d of %d", device, count);
+    rc = check_hip(hipSetDevice(device), "hipSetDevice");
+    if (rc) return rc;
+    hipDeviceProp_t prop;
+    rc = check_hip(hipGetDeviceProperties(&prop, device), "hipGetDeviceProperties");
+    if (rc) return rc;
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return set_error(MMX_E_DEVICE, "mmx_init: device %d is %s, this library holds gfx950 code only", device, prop.gcnArchName);
+    g_cus = prop.multiProcessorCount;
+    return MMX_OK;
+}
+
+size_t mmx_packed_b_bytes(int dtype, int K, int N) {
+    const int es = elesz_of(dtype);
+    if (!es || K <= 0 || N <= 0) return 0;
+    const size_t kpad_bytes = ((size_t)K * es + 127) / 128 * 128;
+    return (size_t)((N + 31) / 32) * 32 * kpad_bytes;
+}
+
+int mmx_repack_b(int dtype, const void* B, int64_t ldb_bytes, int K, int N, int transpose, void* packed, void* stream) {
+    const int es = elesz_of(dtype);
+    if (!es) return set_error(MMX_E_INVALID, "mmx_repack_b: dtype %d is neither bf16 nor int8", dtype);
+    if (!B || !packed) return set_error(MMX_E_INVALID, "mmx_repack_b: NULL pointer");
+    if (K <= 0 || N <= 0) return set_error(MMX_E_INVALID, "mmx_repack_b: K and N must be positive");
+    const int64_t min_ld = (int64_t)(transpose ? K : N) * es;
+    if (ldb_bytes < min_ld || ldb_bytes % es) return set_error(MMX_E_INVALID, "mmx_repack_b: ldb_bytes %lld too small or misaligned", (long long)ldb_bytes);
+    if (reinterpret_cast<uintptr_t>(packed) & 15) return set_error(MMX_E_INVALID, "mmx_repack_b: packed buffer must be 16-byte aligned");
+    return launch_repack(es, B, ldb_bytes, K, N, transpose, packed, static_cast<hipStream_t>(stream));
+}
+
+int mmx_repack_gate_up(const void* w_gate, const void* w_up, int64_t ldw_bytes, int K, int N, void* packed, void* stream) {
+    if (!w_gate || !w_up || !packed) return set_error(MMX_E_INVALID, "mmx_repack_gate_up: NULL pointer");
+    // AMX_MLP::Linear::setup asserts N % 32 == 0 (tests/amx-mlp.cpp:552)
+    if (K <= 0 || N <= 0 || N % 32) return set_error(MMX_E_INVALID, "mmx_repack_gate_up: N = %d must be a positive multiple of 32", N);
+    if (ldw_bytes < (int64_t)K * 2 || ldw_bytes % 2) return set_error(MMX_E_INVALID, "mmx_repack_gate_up: ldw_bytes too small or odd");
+    if (reinterpret_cast<uintptr_t>(packed) & 15) return set_error(MMX_E_INVALID, "mmx_repack_gate_up: packed buffer must be 16-byte aligned");
+    return launch_repack_gate_up(w_gate, w_up, ldw_bytes, K, N, packed, static_cast<hipStream_t>(stream));
+}
+
+int mmx_quantize_weights(const void* W, int64_t ldw_bytes, int rows, int cols, void* Wq, int64_t ldq_bytes, float* scales_out,
+                         uint32_t* absmax_scratch, void* stream) {
+    if (!W || !Wq || !scales_out || !absmax_scratch) return set_error(MMX_E_INVALID, "mmx_quantize_weights: NULL pointer");
+    if (rows <= 0 || cols <= 0 || ldw_bytes < (int64_t)cols * 2 || ldq_bytes < cols)
+        return set_error(MMX_E_INVALID, "mmx_quantize_weights: bad shape or stride");
+    return launch_quantize(W, ldw_bytes, rows, cols, Wq, ldq_bytes, scales_out, absmax_scratch, static_cast<hipStream_t>(stream));
+}
+
+int mmx_dequant_packed(const void* packed_i8, int K, int N, void* packed_bf16, void* stream) {
+    if (!packed_i8 || !packed_bf16 || K <= 0 || N <= 0) return set_error(MMX_E_INVALID, "mmx_dequant_packed: bad argument");
+    if ((reinterpret_cast<uintptr_t>(packed_i8) | reinterpret_cast<uintptr_t>(packed_bf16)) & 15)
+        return set_error(MMX_E_INVALID, "mmx_dequant_packed: buffers must be 16-byte aligned");
+    return launch_dequant_packed(packed_i8, K, N, packed_bf16, static_cast<hipStream_t>(stream));
+}
+
+int mmx_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* Bpacked, int M, int K, int N, int n0,
+             int n1, const mmx_epilogue* ep, void* stream) {
+    return gemm_dispatch(a_dtype, b_dtype, A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, static_cast<hipStream_t>(stream));
+}
+
+int mmx_matvec(int dtype, const void* A, int64_t lda_bytes, const void* b, void* c, int M, int K, void* stream) {
+    const int es = elesz_of(dtype);
+    if (!es) return set_error(MMX_E_INVALID, "mmx_matvec: dtype %d is neither bf16 nor int8", dtype);
+    if (!A || !b || !c || M <= 0 || K <= 0) return set_error(MMX_E_INVALID, "mmx_matvec: bad argument");
+    if (lda_bytes < (int64_t)K * es) return set_error(MMX_E_INVALID, "mmx_matvec: lda_bytes smaller than a row of A");
+    return launch_matvec(dtype == MMX_I8, A, lda_bytes, b, c, M, K, static_cast<hipStream_t>(stream));
+}
+
+int mmx_mlp(const void* x, int64_t ldx_bytes, const void* w_gate_up, const void* w_down, void* h, int64_t ldh_bytes, void* y,
+            int64_t ldy_bytes, int M, int K, int N, void* stream) {
+    if (!x || !w_gate_up || !w_down || !h || !y) return set_error(MMX_E_INVALID, "mmx_mlp: NULL pointer");
+    if (N % 32) return set_error(MMX_E_INVALID, "mmx_mlp: N = %d must be a multiple of 32", N);
+    mmx_epilogue e1;
+    memset(&e1, 0, sizeof e1);
+    e1.steps = MMX_PP_SILU_GATE;
+    e1.out_dtype = MMX_BF16;
+    e1.C = h;
+    e1.ldc_bytes = ldh_bytes;
+    int rc = mmx_gemm(MMX_BF16, MMX_BF16, x, ldx_bytes, w_gate_up, M, K, 2 * N, 0, 2 * N, &e1, stream);
+    if (rc) return rc;
+    mmx_epilogue e2;
+    memset(&e2, 0, sizeof e2);
+    e2.steps = MMX_PP_NONE;
+    e2.out_dtype = MMX_BF16;
+    e2.C = y;
+    e2.ldc_bytes = ldy_bytes;
+    return mmx_gemm(MMX_BF16, MMX_BF16, h, ldh_bytes, w_down, M, N, K, 0, K, &e2, stream);
+}
+
+int mmx_set_tile(const char* shape) {
+    if (!shape || !*shape) { g_forced = {0, 0}; return MMX_OK; }
+    int bm = 0, bn = 0;
+    if (sscanf(shape, "%dx%d", &bm, &bn) != 2) return set_error(MMX_E_INVALID, "mmx_set_tile: cannot parse '%s'", shape);
+    if (!((bm == 256 && (bn == 256 || bn == 192)) || (bm == 128 && (bn == 256 || bn == 128))))
+        return set_error(MMX_E_INVALID, "mmx_set_tile: no kernel for %dx%d", bm, bn);
+    g_forced = {bm, bn};
+    return MMX_OK;
+}
+
+int mmx_set_option(const char* name, int value) {
+    if (name && !strcmp(name, "load_mode")) {
+        if (value < 0 || value > 2) return set_error(MMX_E_INVALID, "mmx_set_option: load_mode is 0, 1 or 2");
+        g_load_mode = value;
+        return MMX_OK;
+    }
+    return set_error(MMX_E_INVALID, "mmx_set_option: unknown option");
+}
+
+int mmx_time_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* const* Bpacked_rot, int n_rot, int M,
+                  int K, int N, int n0, int n1, const mmx_epilogue* ep, void* stream, int iters, float* ms_out) {
+    if (!Bpacked_rot || n_rot <= 0 || iters <= 0 || !ms_out) return set_error(MMX_E_INVALID, "mmx_time_gemm: bad argument");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipEvent_t e0, e1;
+    int rc = check_hip(hipEventCreate(&e0), "hipEventCreate");
+    if (rc) return rc;
+    rc = check_hip(hipEventCreate(&e1), "hipEventCreate");
+    if (rc) { hipEventDestroy(e0); return rc; }
+    rc = check_hip(hipEventRecord(e0, st), "hipEventRecord");
+    for (int i = 0; i < iters && !rc; i++)
+        rc = gemm_dispatch(a_dtype, b_dtype, A, lda_bytes, Bpacked_rot[i % n_rot], M, K, N, n0, n1, ep, st);
+    if (!rc) rc = check_hip(hipEventRecord(e1, st), "hipEventRecord");
+    if (!rc) rc = check_hip(hipEventSynchronize(e1), "hipEventSynchronize");
+    float ms = 0.0f;
+    if (!rc) rc = check_hip(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime");
+    hipEventDestroy(e0);
+    hipEventDestroy(e1);
+    if (!rc) *ms_out = ms / iters;
+    return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,126 @@
+// Shared device/host helpers of the gfx950 FC-GEMM kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mm_amx_amd.h"
+
+namespace mmx {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+typedef __attribute__((__vector_size__(4 * sizeof(int)))) int i32x4;
+typedef __attribute__((__vector_size__(16 * sizeof(int)))) int i32x16;
+// 16 raw bytes as a first-class vector value (unlike HIP's uint4 struct it stays in registers when
+// held in small arrays)
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// error plumbing (host)
+int set_error(int code, const char* fmt, ...);
+int check_hip(hipError_t e, const char* what);
+void note_kernel(const char* name);
+int num_cus();
+
+struct Epilogue {
+    uint32_t steps;
+    int out_dtype;
+    char* C;
+    int64_t ldc;  // bytes
+    const float* bias;
+    float deq;
+    const float* deq_oc;
+    float q;
+    const float* q_oc;
+    int c_vec_ok;  // C and ldc are 16-byte aligned
+};
+
+// ---- element-wise epilogue arithmetic -----------------------------------------------------
+// All device code is compiled with -ffp-contract=off: a*b+c below never fuses unless written
+// as fmaf(), which keeps the rounding sequence of the reference's AVX-512 post-op
+// (include/kernels_amx.hpp:628-664).
+
+__device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// include/kernels_amx.hpp:242-289 — the gelu_erf minimax polynomial, same coefficient bits,
+// same Horner chain of fused multiply-adds, same three selects.
+__device__ __forceinline__ float gelu_erf_minimax(float x) {
+    const float x2 = x * x;
+    const float x_pos = u2f(f2u(x) & 0x7fffffffu);
+    const float x_half = x * 0.5f;
+    float p = u2f(0x1f1c83fdu);
+    p = __builtin_fmaf(p, x2, u2f(0xa3198977u));
+    p = __builtin_fmaf(p, x2, u2f(0x268a7927u));
+    p = __builtin_fmaf(p, x2, u2f(0xa998c963u));
+    p = __builtin_fmaf(p, x2, u2f(0x2c67ddb2u));
+    p = __builtin_fmaf(p, x2, u2f(0xaf013b2cu));
+    p = __builtin_fmaf(p, x2, u2f(0x315d4a4fu));
+    p = __builtin_fmaf(p, x2, u2f(0xb3969b11u));
+    p = __builtin_fmaf(p, x2, u2f(0x35a776e9u));
+    p = __builtin_fmaf(p, x2, u2f(0xb79b0914u));
+    p = __builtin_fmaf(p, x2, u2f(0x3970b255u));
+    p = __builtin_fmaf(p, x2, u2f(0xbb1b7399u));
+    p = __builtin_fmaf(p, x2, u2f(0x3ca3621fu));
+    p = __builtin_fmaf(p, x2, u2f(0xbe082bc7u));
+    p = __builtin_fmaf(p, x2, u2f(0x3f4c4228u));
+    p = __builtin_fmaf(p, x, 1.0f);
+    p = p * x_half;
+    if (x < -5.0f) x = 0.0f;             // zone 1 (NaN keeps x)
+    if (!(x_pos <= 5.0f)) p = x;         // zones 1 and 5 (and NaN)
+    if (x_pos <= u2f(0x33800000u)) p = x_half;  // zone 3
+    return p;
+}
+
+// tests/amx-mlp.cpp:383-448 — exp_ps_avx512, operation for operation.
+__device__ __forceinline__ float exp_poly(float x) {
+    const float ln_flt_min = u2f(0xc2aeac50u), ln_flt_max = u2f(0x42b17218u);
+    const bool zero = x < ln_flt_min;
+    float s = (x < ln_flt_max) ? x : ln_flt_max;
+    s = (s > ln_flt_min) ? s : ln_flt_min;
+    float r = s;
+    s = s * u2f(0x3fb8aa3bu);
+    s = s + 0.5f;
+    s = __builtin_floorf(s);
+    r = __builtin_fmaf(-s, u2f(0x3f317218u), r);
+    s = s - 1.0f;
+    int e = (int)__builtin_rintf(s);
+    e = (int)((uint32_t)(e + 127) << 23);
+    const float two_n = zero ? 0.0f : u2f((uint32_t)e);
+    s = u2f(0x3c07cfceu);
+    s = __builtin_fmaf(s, r, u2f(0x3d2b9d0du));
+    s = __builtin_fmaf(s, r, u2f(0x3e2aad40u));
+    s = __builtin_fmaf(s, r, u2f(0x3efffee3u));
+    s = __builtin_fmaf(s, r, u2f(0x3f7ffffbu));
+    s = __builtin_fmaf(s, r, 1.0f);
+    s = s * two_n;
+    s = s * 2.0f;
+    return s;
+}
+
+// tests/amx-mlp.cpp:450-456 — x * 1/(1+exp(-x)); the reciprocal is the correctly rounded one
+// (the reference's vrcp14ps approximation is an x86 instruction with no GPU counterpart).
+__device__ __forceinline__ float silu(float x) {
+    const float e = exp_poly(0.0f - x);
+    const float sig = 1.0f / (1.0f + e);
+    return x * sig;
+}
+
+// fp32 -> bf16, round to nearest even (vcvtne2ps2bf16, include/kernels_amx.hpp:654)
+__device__ __forceinline__ uint16_t to_bf16(float x) {
+    __bf16 b = (__bf16)x;
+    return __builtin_bit_cast(uint16_t, b);
+}
+__device__ __forceinline__ float from_bf16(uint16_t b) { return u2f((uint32_t)b << 16); }
+
+// vcvtps2dq (round to nearest even; NaN / out of int32 range -> 0x80000000) followed by
+// vpmovsdb signed saturation (include/kernels_amx.hpp:658-661)
+__device__ __forceinline__ int8_t to_s8_sat(float r) {
+    float t = __builtin_rintf(r);
+    if (!(r >= -2147483648.0f && r < 2147483648.0f)) t = -128.0f;
+    t = __builtin_fminf(__builtin_fmaxf(t, -128.0f), 127.0f);
+    return (int8_t)(int)t;
+}
+
+}  // namespace mmx

@@ -1,0 +1,436 @@
+// MFMA tile GEMM for gfx950: C[:, n0:n1] = PP(A · Bpacked[:, n0:n1]).
+//
+// Stands in for the large-M paths of amx_kernel::Matmul::operator()
+// (include/kernels_amx.hpp:1255-1313): the AMX 2x2 register blocking of 16x16 tiles becomes a
+// 2x2 grid of wavefronts, each owning a (BM/2)x(BN/2) block of 32x32 MFMA accumulators; the
+// per-32x32-block post-op through an L1 scratch tile (:1290-1294) becomes an epilogue applied
+// to the accumulators in registers and staged through LDS only to make the stores row-contiguous.
+//
+// Data movement per k-iteration (128 bytes of K per row: 64 bf16 or 128 int8):
+//   A  [BM rows x 128 B]  row-major in HBM -> LDS rows of 128 B, 16-byte chunks XOR-swizzled by
+//      (row & 7) so that the 32 rows an MFMA operand needs hit all LDS banks;
+//   B  [BN/32 panels x 4 fragments x 1 KiB] already in MFMA operand order in HBM -> copied
+//      verbatim, every ds_read_b128 of a fragment is lane-contiguous.
+// Two LDS stages; loads of stage k+1 are in flight while stage k is multiplied.  Three load modes:
+//   MODE 0  global -> VGPR -> LDS (16-byte loads, rows past M clamped to the last row);
+//   MODE 1  global_load_lds_dwordx4 (HBM -> LDS without passing through VGPRs) through the
+//           compiler builtin; the compiler then waits for ALL outstanding LDS reads before each
+//           group of MFMAs (it counts the LDS-DMA as an out-of-order event);
+//   MODE 2  the same instruction issued from inline asm, so that the compiler's in-order
+//           accounting of ds_read results stays exact; its completion is awaited explicitly
+//           (s_waitcnt vmcnt(0) before the workgroup barrier);
+//   MODE 3  global -> VGPR -> LDS with per-element masking: the general path for K tails
+//           (K*sizeof(T) not a multiple of 128) and for A rows that are not 16-byte aligned.
+//           Rows past M and elements past K are read as zero, never touched in memory.
+#pragma once
+#include "common.hpp"
+
+namespace mmx {
+
+template <typename TIn>
+struct Mfma;
+template <>
+struct Mfma<__bf16> {
+    using frag = bf16x8;
+    using accv = f32x16;
+    static __device__ __forceinline__ accv run(frag a, frag b, accv c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float to_f32(float v) { return v; }
+};
+template <>
+struct Mfma<int8_t> {
+    using frag = i32x4;
+    using accv = i32x16;
+    static __device__ __forceinline__ accv run(frag a, frag b, accv c) {
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+    }
+    // vcvtdq2ps, round to nearest even (include/kernels_amx.hpp:631-634)
+    static __device__ __forceinline__ float to_f32(int v) { return (float)v; }
+};
+
+struct GemmArgs {
+    const char* A;
+    int64_t lda;           // bytes
+    const char* Bp;        // packed weights
+    int64_t panel_stride;  // bytes per 32-column panel = nk * 4096
+    int M;
+    int kbytes;   // valid bytes per row of A
+    int nk;       // k-iterations of 128 bytes
+    int npanels;  // 32-column panels in Bp
+    int n0, n1;
+    int tiles_m, total_tiles, tiles_per_xcd;
+    int a_vec_ok;  // A and lda 16-byte aligned
+    Epilogue ep;
+};
+
+template <typename TOut>
+__device__ __forceinline__ TOut cvt_out(float r);
+template <>
+__device__ __forceinline__ float cvt_out<float>(float r) { return r; }
+template <>
+__device__ __forceinline__ uint16_t cvt_out<uint16_t>(float r) { return to_bf16(r); }
+template <>
+__device__ __forceinline__ int8_t cvt_out<int8_t>(float r) { return to_s8_sat(r); }
+template <>
+__device__ __forceinline__ int32_t cvt_out<int32_t>(float r) { return (int32_t)r; }
+
+__device__ __forceinline__ u32x4 load_a_chunk_masked(const char* rowptr, int kbyte, int kbytes, bool vec_ok) {
+    u32x4 v = u32x4{0u, 0u, 0u, 0u};
+    if (kbyte >= kbytes) return v;
+    if (vec_ok && kbyte + 16 <= kbytes) return *reinterpret_cast<const u32x4*>(rowptr + kbyte);
+    uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int b = 0; b < 16; b++) {
+        if (kbyte + b < kbytes) w[b >> 2] |= (uint32_t)(uint8_t)rowptr[kbyte + b] << (8 * (b & 3));
+    }
+    return u32x4{w[0], w[1], w[2], w[3]};
+}
+
+// 16 bytes per lane from global memory straight into LDS at lds_wave_base + lane*16
+// (lds_wave_base must be uniform across the wavefront: it travels in M0).
+template <int MODE>
+__device__ __forceinline__ void lds_dma16(const char* src, char* lds_wave_base) {
+    if constexpr (MODE == 1) {
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+    } else {
+        const uint32_t m0 = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_wave_base);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0), "v"(src) : "memory");
+    }
+}
+template <int MODE>
+__device__ __forceinline__ void lds_dma_wait() {
+    if constexpr (MODE == 1) __builtin_amdgcn_s_waitcnt(0);
+    if constexpr (MODE == 2) asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+}
+
+template <typename TIn, int BM, int BN, int MODE, typename TOut>
+__global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs g) {
+    using MF = Mfma<TIn>;
+    using frag = typename MF::frag;
+    using accv = typename MF::accv;
+    constexpr int WM = BM / 2, WN = BN / 2;
+    constexpr int MI = WM / 32, NJ = WN / 32;
+    constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+    constexpr int A_IT = BM / 32, B_IT = BN / 32;  // 16-byte chunks per thread per stage
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, g32 = lane >> 5;
+
+    // XCD-aware tile order: workgroup ids go round-robin over the 8 XCDs, so give each XCD a
+    // contiguous run of tiles (m fastest): tiles that share a B panel run on one L2.
+    const int L = (blockIdx.x & 7) * g.tiles_per_xcd + (blockIdx.x >> 3);
+    if (L >= g.total_tiles) return;
+    const int tn = L / g.tiles_m, tm = L % g.tiles_m;
+    const int m0 = tm * BM;
+    const int ntile0 = g.n0 + tn * BN;
+    const int panel0 = ntile0 >> 5;
+
+    accv acc[MI][NJ];
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0;
+
+    constexpr bool DIRECT = (MODE == 1 || MODE == 2);
+    u32x4 ra[DIRECT ? 1 : A_IT], rb[DIRECT ? 1 : B_IT];
+
+    auto fetch = [&](int kt, int stage) {
+        char* sA = smem + stage * STAGE;
+        char* sB = sA + A_BYTES;
+#pragma unroll
+        for (int it = 0; it < A_IT; it++) {
+            const int c = it * 256 + tid;
+            const int row = c >> 3, slot = c & 7;
+            const int chunk = slot ^ (row & 7);
+            int grow = m0 + row;
+            if constexpr (MODE != 3) {
+                grow = grow < g.M ? grow : g.M - 1;
+                const char* src = g.A + (int64_t)grow * g.lda + kt * 128 + chunk * 16;
+                if constexpr (DIRECT) lds_dma16<MODE>(src, sA + (it * 256 + wave * 64) * 16);
+                else ra[it] = *reinterpret_cast<const u32x4*>(src);
+            } else {
+                ra[it] = u32x4{0u, 0u, 0u, 0u};
+                if (grow < g.M)
+                    ra[it] = load_a_chunk_masked(g.A + (int64_t)grow * g.lda, kt * 128 + chunk * 16, g.kbytes,
+                                                 g.a_vec_ok);
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < B_IT; it++) {
+            // 256 chunks = one panel's 4 KiB of this k-iteration.  A tile may reach past the last
+            // panel of the packed weights: re-read the last panel instead (those columns are never
+            // stored), which keeps the loop free of branches.
+            int panel = panel0 + it;
+            panel = panel < g.npanels ? panel : g.npanels - 1;
+            const char* src = g.Bp + (int64_t)panel * g.panel_stride + (int64_t)kt * 4096 + tid * 16;
+            if constexpr (DIRECT) {
+                lds_dma16<MODE>(src, sB + (it * 256 + wave * 64) * 16);
+            } else {
+                rb[it] = *reinterpret_cast<const u32x4*>(src);
+            }
+        }
+    };
+    auto commit = [&](int stage) {
+        if constexpr (!DIRECT) {
+            char* sA = smem + stage * STAGE;
+            char* sB = sA + A_BYTES;
+#pragma unroll
+            for (int it = 0; it < A_IT; it++) *reinterpret_cast<u32x4*>(sA + (it * 256 + tid) * 16) = ra[it];
+#pragma unroll
+            for (int it = 0; it < B_IT; it++) *reinterpret_cast<u32x4*>(sB + (it * 256 + tid) * 16) = rb[it];
+        }
+    };
+
+    // Fragment registers are double buffered: the ds_reads of k-step s+1 are issued before the
+    // MFMAs of k-step s, so LDS latency is covered by matrix work even with one wave per SIMD.
+    frag fa[2][MI], fb[2][NJ];
+    auto read_frags = [&](int stage, int s, frag (&a)[MI], frag (&b)[NJ]) {
+        const char* sA = smem + stage * STAGE + (wm * WM + l32) * 128;
+        const char* sB = smem + stage * STAGE + A_BYTES + (wn * NJ * 4) * 1024 + lane * 16;
+        const int slot = (2 * s + g32) ^ (l32 & 7);
+#pragma unroll
+        for (int i = 0; i < MI; i++) a[i] = *reinterpret_cast<const frag*>(sA + i * 32 * 128 + slot * 16);
+#pragma unroll
+        for (int j = 0; j < NJ; j++) b[j] = *reinterpret_cast<const frag*>(sB + (j * 4 + s) * 1024);
+    };
+    auto mma = [&](const frag (&a)[MI], const frag (&b)[NJ]) {
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int j = 0; j < NJ; j++) acc[i][j] = MF::run(a[i], b[j], acc[i][j]);
+    };
+
+    fetch(0, 0);
+    commit(0);
+    lds_dma_wait<MODE>();
+    __syncthreads();
+    read_frags(0, 0, fa[0], fb[0]);
+
+    // Scheduling groups: within each region issue the LDS reads of the next k-step first, then
+    // the MFMAs of the current one (mask 0x100 = DS read, 0x008 = MFMA).
+#define MMX_READS_THEN_MFMA()                                          \
+    __builtin_amdgcn_sched_group_barrier(0x100, MI + NJ, 0);           \
+    __builtin_amdgcn_sched_group_barrier(0x008, MI * NJ, 0);           \
+    __builtin_amdgcn_sched_barrier(0)
+
+    for (int kt = 0; kt < g.nk; kt++) {
+        const int stage = kt & 1;
+        // the last iteration re-fetches its own stage into the idle buffer: harmless, and it keeps
+        // the loop body free of branches so that the schedule below is one straight block
+        const int kt_next = (kt + 1 < g.nk) ? kt + 1 : kt;
+        fetch(kt_next, stage ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(stage, 1, fa[1], fb[1]);
+        mma(fa[0], fb[0]);
+        MMX_READS_THEN_MFMA();
+        read_frags(stage, 2, fa[0], fb[0]);
+        mma(fa[1], fb[1]);
+        MMX_READS_THEN_MFMA();
+        read_frags(stage, 3, fa[1], fb[1]);
+        mma(fa[0], fb[0]);
+        MMX_READS_THEN_MFMA();
+        // Everything this wave reads from the current stage is now in registers, and the next
+        // stage has had three k-steps to land: synchronise here, then start reading the next
+        // stage while the last k-step of this one is multiplied.
+        commit(stage ^ 1);
+        lds_dma_wait<MODE>();
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(stage ^ 1, 0, fa[0], fb[0]);
+        mma(fa[1], fb[1]);
+        MMX_READS_THEN_MFMA();
+    }
+#undef MMX_READS_THEN_MFMA
+    __syncthreads();
+
+    // ---- epilogue: registers -> post-op -> LDS (per-wave staging band) -> row-contiguous stores
+    const Epilogue& ep = g.ep;
+    const bool silu_gate = (ep.steps & MMX_PP_SILU_GATE) != 0;
+    constexpr int SZ = sizeof(TOut);
+    constexpr int SROW = WN * SZ + 16;  // staging row stride, padded
+    char* stg = smem + wave * (32 * SROW);
+    const int out_n1 = silu_gate ? (g.n1 >> 1) : g.n1;
+    const int out_col_base = silu_gate ? ((ntile0 + wn * WN) >> 1) : (ntile0 + wn * WN);
+    const int wn_out = silu_gate ? WN / 2 : WN;
+
+#pragma unroll
+    for (int i = 0; i < MI; i++) {
+        __syncthreads();
+        if (silu_gate) {
+            if constexpr (NJ % 2 == 0) {
+#pragma unroll
+                for (int j = 0; j < NJ; j += 2) {
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        const float gt = MF::to_f32(acc[i][j][v]);
+                        const float up = MF::to_f32(acc[i][j + 1][v]);
+                        const float r = silu(gt) * up;
+                        const int row = 8 * (v >> 2) + 4 * g32 + (v & 3);
+                        *reinterpret_cast<TOut*>(stg + row * SROW + ((j >> 1) * 32 + l32) * SZ) = cvt_out<TOut>(r);
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                const int ncol = ntile0 + wn * WN + 32 * j + l32;
+                const bool col_ok = ncol < g.n1;
+                float r[16];
+#pragma unroll
+                for (int v = 0; v < 16; v++) r[v] = MF::to_f32(acc[i][j][v]);
+                if (ep.steps & MMX_PP_DEQUANT) {
+                    const float d = ep.deq_oc ? (col_ok ? ep.deq_oc[ncol] : 0.0f) : ep.deq;
+#pragma unroll
+                    for (int v = 0; v < 16; v++) r[v] = r[v] * d;
+                }
+                if (ep.steps & MMX_PP_BIAS) {
+                    const float bv = col_ok ? ep.bias[ncol] : 0.0f;
+#pragma unroll
+                    for (int v = 0; v < 16; v++) r[v] = r[v] + bv;
+                }
+                if (ep.steps & MMX_PP_GELU) {
+#pragma unroll
+                    for (int v = 0; v < 16; v++) r[v] = gelu_erf_minimax(r[v]);
+                }
+                if (ep.steps & MMX_PP_QUANT) {
+                    const float qv = ep.q_oc ? (col_ok ? ep.q_oc[ncol] : 0.0f) : ep.q;
+#pragma unroll
+                    for (int v = 0; v < 16; v++) r[v] = r[v] * qv;
+                }
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int row = 8 * (v >> 2) + 4 * g32 + (v & 3);
+                    TOut o;
+                    if constexpr (sizeof(TOut) == 4 && !__is_same(TOut, float)) {
+                        o = (TOut)acc[i][j][v];  // raw int32 accumulator
+                    } else {
+                        o = cvt_out<TOut>(r[v]);
+                    }
+                    *reinterpret_cast<TOut*>(stg + row * SROW + (j * 32 + l32) * SZ) = o;
+                }
+            }
+        }
+        __syncthreads();
+        const int ppr = wn_out * SZ / 16;  // 16-byte pieces per staged row
+        const int per_piece = 16 / SZ;
+        for (int idx = lane; idx < 32 * ppr; idx += 64) {
+            const int row = idx / ppr, piece = idx - row * ppr;
+            const int grow = m0 + wm * WM + 32 * i + row;
+            const int col0 = out_col_base + piece * per_piece;
+            if (grow < g.M && col0 < out_n1) {
+                const char* src = stg + row * SROW + piece * 16;
+                char* dst = ep.C + (int64_t)grow * ep.ldc + (int64_t)col0 * SZ;
+                if (ep.c_vec_ok && col0 + per_piece <= out_n1) {
+                    *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(src);
+                } else {
+                    for (int e = 0; e < per_piece; e++)
+                        if (col0 + e < out_n1)
+                            reinterpret_cast<TOut*>(dst)[e] = reinterpret_cast<const TOut*>(src)[e];
+                }
+            }
+        }
+    }
+}
+
+// ---- host side ---------------------------------------------------------------------------------
+
+struct TileCfg {
+    int bm, bn;
+};
+TileCfg forced_tile();
+int load_mode();
+
+// Pick the tile that minimises (rounds over the CUs) x (work per tile) / (per-tile efficiency).
+static inline TileCfg choose_tile(int M, int Ncols, bool need_pairs) {
+    const TileCfg f = forced_tile();
+    if (f.bm) return f;
+    static const struct { int bm, bn; float eff; int per_cu; } cand[] = {
+        {256, 256, 1.00f, 1}, {256, 192, 0.97f, 1}, {128, 256, 0.90f, 1}, {128, 128, 0.80f, 2}};
+    const int cus = num_cus();
+    float best = 1e30f;
+    TileCfg pick = {128, 128};
+    for (const auto& c : cand) {
+        if (need_pairs && (c.bn % 128) != 0) continue;
+        const int tiles = ((M + c.bm - 1) / c.bm) * ((Ncols + c.bn - 1) / c.bn);
+        const int slots = cus * c.per_cu;
+        const int rounds = (tiles + slots - 1) / slots;
+        const float t = (float)rounds * c.per_cu * (float)(c.bm * c.bn) / c.eff;
+        if (t < best) { best = t; pick = {c.bm, c.bn}; }
+    }
+    return pick;
+}
+
+template <typename TIn, int BM, int BN, int MODE, typename TOut>
+static int launch_cfg(const GemmArgs& g, int grid, hipStream_t st, const char* name) {
+    constexpr int lds = 2 * (BM + BN) * 128;
+    auto kern = gemm_kernel<TIn, BM, BN, MODE, TOut>;
+    static bool attr_done = false;  // one flag per instantiation
+    if (!attr_done) {
+        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+                           "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+        if (rc) return rc;
+        attr_done = true;
+    }
+    note_kernel(name);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, g);
+    return check_hip(hipGetLastError(), name);
+}
+
+#define MMX_LAUNCH(TIn, BM, BN, MODE, TOut) \
+    launch_cfg<TIn, BM, BN, MODE, TOut>(g, grid, st, "gemm_" #TIn "_" #BM "x" #BN "_mode" #MODE "_" #TOut)
+#define MMX_LAUNCH_MODES(TIn, BM, BN, TOut)                                  \
+    (mode == 2 ? MMX_LAUNCH(TIn, BM, BN, 2, TOut)                            \
+               : mode == 1 ? MMX_LAUNCH(TIn, BM, BN, 1, TOut) : MMX_LAUNCH(TIn, BM, BN, 0, TOut))
+
+template <typename TIn, typename TOut>
+static int launch_tiles(const GemmArgs& g, TileCfg t, int mode, int grid, hipStream_t st) {
+    if (mode == 3) return MMX_LAUNCH(TIn, 128, 128, 3, TOut);  // the masked path exists for one tile shape
+    if (t.bm == 256 && t.bn == 256) return MMX_LAUNCH_MODES(TIn, 256, 256, TOut);
+    if (t.bm == 256 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 256, 192, TOut);
+    if (t.bm == 128 && t.bn == 256) return MMX_LAUNCH_MODES(TIn, 128, 256, TOut);
+    if (t.bm == 128 && t.bn == 128) return MMX_LAUNCH_MODES(TIn, 128, 128, TOut);
+    return set_error(MMX_E_UNSUPPORTED, "no MFMA tile kernel for %dx%d", t.bm, t.bn);
+}
+
+// Fills the launch geometry; returns the grid size (or a negative error code).
+static inline int prepare_gemm(GemmArgs& g, TileCfg& t, int& mode, int elesz, const void* A, int64_t lda, const void* Bp,
+                               int M, int K, int N, int n0, int n1, const Epilogue& ep) {
+    g.A = static_cast<const char*>(A);
+    g.lda = lda;
+    g.Bp = static_cast<const char*>(Bp);
+    g.M = M;
+    g.kbytes = K * elesz;
+    g.nk = (g.kbytes + 127) / 128;
+    g.panel_stride = (int64_t)g.nk * 4096;
+    g.npanels = (N + 31) / 32;
+    g.n0 = n0;
+    g.n1 = n1;
+    g.a_vec_ok = ((reinterpret_cast<uintptr_t>(A) & 15) == 0) && ((lda & 15) == 0);
+    g.ep = ep;
+    const bool pairs = (ep.steps & MMX_PP_SILU_GATE) != 0;
+    // the unmasked loads need aligned rows and a K that fills whole k-iterations
+    const bool fast_ok = g.a_vec_ok && (g.kbytes % 128 == 0);
+    mode = fast_ok ? load_mode() : 3;
+    t = choose_tile(M, n1 - n0, pairs);
+    if (mode == 3) t = {128, 128};
+    if (pairs && (t.bn % 128) != 0)
+        return set_error(MMX_E_INVALID, "SILU_GATE needs a tile width that is a multiple of 128");
+    g.tiles_m = (M + t.bm - 1) / t.bm;
+    const int tiles_n = (n1 - n0 + t.bn - 1) / t.bn;
+    g.total_tiles = g.tiles_m * tiles_n;
+    g.tiles_per_xcd = (g.total_tiles + 7) / 8;
+    return g.tiles_per_xcd * 8;
+}
+
+}  // namespace mmx

@@ -1,0 +1,218 @@
+// One-off weight preparation kernels: repack to MFMA-fragment order, gate/up interleave,
+// per-tensor int8 weight compression, packed int8 -> packed bf16.
+//
+// Stands in for amx_kernel::repackB_1x2 (include/kernels_amx.hpp:761-816), MLP::setup's gate/up
+// interleave (tests/amx-mlp.cpp:758-765) and the weight compression inside
+// amx_kernel::Matmul<bf16,int8,float> (include/kernels_amx.hpp:1363-1377, 465-523).
+// These move bytes once per weight matrix; they are written for clarity, each thread producing one
+// 16-byte lane slot of the packed result.
+#include "common.hpp"
+
+namespace mmx {
+
+// Packed layout: [panel = n/32][f = k/KS][lane][16 B], KS = 32/ES elements, lane = n%32 + 32*((k%KS)/(KS/2)).
+template <int ES>
+__global__ void repack_kernel(const char* __restrict__ B, int64_t ldb, int K, int N, int transpose,
+                              char* __restrict__ out, int nfrag, int64_t total_slots) {
+    constexpr int HALF = 16 / ES;  // elements per lane slot
+    const int64_t slot = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (slot >= total_slots) return;
+    const int lane = (int)(slot & 63);
+    const int64_t pf = slot >> 6;
+    const int f = (int)(pf % nfrag);
+    const int panel = (int)(pf / nfrag);
+    const int n = panel * 32 + (lane & 31);
+    const int k0 = f * (2 * HALF) + (lane >> 5) * HALF;
+    alignas(16) char buf[16];
+#pragma unroll
+    for (int e = 0; e < HALF; e++) {
+        const int k = k0 + e;
+        const bool ok = (n < N) && (k < K);
+        const char* src = transpose ? B + (int64_t)n * ldb + (int64_t)k * ES : B + (int64_t)k * ldb + (int64_t)n * ES;
+        if (ES == 2) {
+            reinterpret_cast<uint16_t*>(buf)[e] = ok ? *reinterpret_cast<const uint16_t*>(src) : (uint16_t)0;
+        } else {
+            buf[e] = ok ? *src : (char)0;
+        }
+    }
+    *reinterpret_cast<uint4*>(out + slot * 16) = *reinterpret_cast<const uint4*>(buf);
+}
+
+int launch_repack(int elesz, const void* B, int64_t ldb, int K, int N, int transpose, void* out, hipStream_t st) {
+    const int kpad_bytes = (K * elesz + 127) / 128 * 128;
+    const int nfrag = kpad_bytes / 32;
+    const int64_t npanels = (N + 31) / 32;
+    const int64_t slots = npanels * nfrag * 64;
+    const int threads = 256;
+    const int64_t blocks = (slots + threads - 1) / threads;
+    if (blocks > 0x7fffffff) return set_error(MMX_E_INVALID, "weight matrix too large to repack in one launch");
+    if (elesz == 2)
+        hipLaunchKernelGGL((repack_kernel<2>), dim3((unsigned)blocks), dim3(threads), 0, st,
+                           static_cast<const char*>(B), ldb, K, N, transpose, static_cast<char*>(out), nfrag, slots);
+    else
+        hipLaunchKernelGGL((repack_kernel<1>), dim3((unsigned)blocks), dim3(threads), 0, st,
+                           static_cast<const char*>(B), ldb, K, N, transpose, static_cast<char*>(out), nfrag, slots);
+    return check_hip(hipGetLastError(), "repack_kernel launch");
+}
+
+// gate and up ([N, K] bf16 each) -> one packed matrix of 2N columns: panel 2p = gate columns
+// [32p, 32p+32), panel 2p+1 = up columns [32p, 32p+32).
+__global__ void repack_gate_up_kernel(const char* __restrict__ Wg, const char* __restrict__ Wu, int64_t ldw, int K,
+                                      int N, char* __restrict__ out, int nfrag, int64_t total_slots) {
+    const int64_t slot = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (slot >= total_slots) return;
+    const int lane = (int)(slot & 63);
+    const int64_t pf = slot >> 6;
+    const int f = (int)(pf % nfrag);
+    const int panel = (int)(pf / nfrag);
+    const char* W = (panel & 1) ? Wu : Wg;
+    const int n = (panel >> 1) * 32 + (lane & 31);
+    const int k0 = f * 16 + (lane >> 5) * 8;
+    alignas(16) uint16_t buf[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const int k = k0 + e;
+        buf[e] = (n < N && k < K) ? *reinterpret_cast<const uint16_t*>(W + (int64_t)n * ldw + (int64_t)k * 2) : (uint16_t)0;
+    }
+    *reinterpret_cast<uint4*>(out + slot * 16) = *reinterpret_cast<const uint4*>(buf);
+}
+
+int launch_repack_gate_up(const void* wg, const void* wu, int64_t ldw, int K, int N, void* out, hipStream_t st) {
+    const int nfrag = ((K * 2 + 127) / 128 * 128) / 32;
+    const int64_t slots = (int64_t)(2 * N / 32) * nfrag * 64;
+    const int threads = 256;
+    const int64_t blocks = (slots + threads - 1) / threads;
+    if (blocks > 0x7fffffff) return set_error(MMX_E_INVALID, "weight matrix too large to repack in one launch");
+    hipLaunchKernelGGL(repack_gate_up_kernel, dim3((unsigned)blocks), dim3(threads), 0, st, static_cast<const char*>(wg),
+                       static_cast<const char*>(wu), ldw, K, N, static_cast<char*>(out), nfrag, slots);
+    return check_hip(hipGetLastError(), "repack_gate_up_kernel launch");
+}
+
+// ---- per-tensor weight compression ---------------------------------------------------------------
+__global__ void zero_u32_kernel(uint32_t* p) { *p = 0u; }
+
+// max |w| over the matrix: the bit pattern of a non-negative float orders like an unsigned integer
+__global__ void absmax_kernel(const char* __restrict__ W, int64_t ldw, int rows, int cols, uint32_t* out) {
+    uint32_t m = 0;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < (int64_t)rows * cols;
+         i += (int64_t)gridDim.x * blockDim.x) {
+        const int r = (int)(i / cols), c = (int)(i % cols);
+        const uint32_t bits = (uint32_t)(*reinterpret_cast<const uint16_t*>(W + (int64_t)r * ldw + (int64_t)c * 2)) << 16;
+        const uint32_t a = bits & 0x7fffffffu;
+        if (a <= 0x7f800000u && a > m) m = a;  // NaNs do not take part, as with vmaxps/vminps accumulators
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        const uint32_t o = __shfl_xor(m, off);
+        m = o > m ? o : m;
+    }
+    if ((threadIdx.x & 63) == 0) atomicMax(out, m);
+}
+
+// q = sat8(rne(w * (127/max))) (include/kernels_amx.hpp:508-523); scales_out = {127/max, max/127}
+__global__ void quantize_kernel(const char* __restrict__ W, int64_t ldw, int rows, int cols, char* __restrict__ Wq,
+                                int64_t ldq, const uint32_t* absmax_bits, float* scales_out) {
+    const float amax = u2f(*absmax_bits);
+    const float q = 127 / amax;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        scales_out[0] = q;
+        scales_out[1] = amax / 127;
+    }
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < (int64_t)rows * cols;
+         i += (int64_t)gridDim.x * blockDim.x) {
+        const int r = (int)(i / cols), c = (int)(i % cols);
+        const float w = from_bf16(*reinterpret_cast<const uint16_t*>(W + (int64_t)r * ldw + (int64_t)c * 2));
+        Wq[(int64_t)r * ldq + c] = (char)to_s8_sat(w * q);
+    }
+}
+
+int launch_quantize(const void* W, int64_t ldw, int rows, int cols, void* Wq, int64_t ldq, float* scales_out,
+                    uint32_t* scratch, hipStream_t st) {
+    const int64_t n = (int64_t)rows * cols;
+    int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(1), 0, st, scratch);
+    hipLaunchKernelGGL(absmax_kernel, dim3(blocks), dim3(256), 0, st, static_cast<const char*>(W), ldw, rows, cols, scratch);
+    hipLaunchKernelGGL(quantize_kernel, dim3(blocks), dim3(256), 0, st, static_cast<const char*>(W), ldw, rows, cols,
+                       static_cast<char*>(Wq), ldq, scratch, scales_out);
+    return check_hip(hipGetLastError(), "quantize kernels launch");
+}
+
+// ---- packed int8 -> packed bf16 (exact) -------------------------------------------------------------
+// int8 slot (panel, f, lane): 16 consecutive k of column n -> bf16 fragments 2f and 2f+1 ... the
+// 16 k's starting at 32f + 16g split into two runs of 8: run h goes to bf16 fragment 2f+g,
+// lane (n%32) + 32*h.
+__global__ void dequant_packed_kernel(const char* __restrict__ in, char* __restrict__ out, int nfrag8, int nfrag16,
+                                      int64_t total_slots) {
+    const int64_t slot = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (slot >= total_slots) return;
+    const int lane = (int)(slot & 63);
+    const int64_t pf = slot >> 6;
+    const int f = (int)(pf % nfrag8);
+    const int64_t panel = pf / nfrag8;
+    const uint4 v = *reinterpret_cast<const uint4*>(in + slot * 16);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    const int g = lane >> 5, l32 = lane & 31;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        alignas(16) uint16_t o[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int b = h * 8 + e;
+            o[e] = to_bf16((float)(int8_t)((w[b >> 2] >> (8 * (b & 3))) & 0xff));
+        }
+        // the bf16 layout pads K to 64, the int8 one to 128: fragments past the bf16 padding hold only zeros
+        if (2 * f + g < nfrag16) {
+            const int64_t of = (panel * nfrag16 + 2 * f + g) * 64 + l32 + 32 * h;
+            *reinterpret_cast<uint4*>(out + of * 16) = *reinterpret_cast<const uint4*>(o);
+        }
+    }
+}
+
+int launch_dequant_packed(const void* in, int K, int N, void* out, hipStream_t st) {
+    const int nfrag8 = ((K + 127) / 128 * 128) / 32;
+    const int nfrag16 = ((K + 63) / 64 * 64) / 16;
+    const int64_t slots = (int64_t)((N + 31) / 32) * nfrag8 * 64;
+    const int64_t blocks = (slots + 255) / 256;
+    if (blocks > 0x7fffffff) return set_error(MMX_E_INVALID, "weight matrix too large");
+    hipLaunchKernelGGL(dequant_packed_kernel, dim3((unsigned)blocks), dim3(256), 0, st, static_cast<const char*>(in),
+                       static_cast<char*>(out), nfrag8, nfrag16, slots);
+    return check_hip(hipGetLastError(), "dequant_packed_kernel launch");
+}
+
+// ---- c[M] = A[M,K] · b[K] ---------------------------------------------------------------------------
+// amx_kernel::MatmulVector (include/kernels_amx.hpp:833-1043) and GemAvB (:1529-1618): one
+// wavefront per row of A, lanes stride over K, wave reduction.
+template <bool I8>
+__global__ void matvec_kernel(const char* __restrict__ A, int64_t lda, const char* __restrict__ b, void* c, int M, int K) {
+    const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= M) return;
+    const char* a = A + (int64_t)row * lda;
+    if (I8) {
+        int acc = 0;
+        for (int k = lane; k < K; k += 64) acc += (int)(int8_t)a[k] * (int)(int8_t)b[k];
+        for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+        if (lane == 0) static_cast<int*>(c)[row] = acc;
+    } else {
+        float acc = 0.0f;
+        for (int k = lane; k < K; k += 64)
+            acc = __builtin_fmaf(from_bf16(reinterpret_cast<const uint16_t*>(a)[k]),
+                                 from_bf16(reinterpret_cast<const uint16_t*>(b)[k]), acc);
+        for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+        if (lane == 0) static_cast<float*>(c)[row] = acc;
+    }
+}
+
+int launch_matvec(bool i8, const void* A, int64_t lda, const void* b, void* c, int M, int K, hipStream_t st) {
+    const int rows_per_block = 4;
+    const int blocks = (M + rows_per_block - 1) / rows_per_block;
+    if (i8)
+        hipLaunchKernelGGL((matvec_kernel<true>), dim3(blocks), dim3(256), 0, st, static_cast<const char*>(A), lda,
+                           static_cast<const char*>(b), c, M, K);
+    else
+        hipLaunchKernelGGL((matvec_kernel<false>), dim3(blocks), dim3(256), 0, st, static_cast<const char*>(A), lda,
+                           static_cast<const char*>(b), c, M, K);
+    return check_hip(hipGetLastError(), "matvec_kernel launch");
+}
+
+}  // namespace mmx

@@ -1,0 +1,191 @@
+// Decode-regime FC (M <= 32): y = PP(x · W[:, n0:n1]) over bf16 or int8-compressed weights.
+//
+// Stands in for the M<=16 / M<=32 branches of amx_kernel::Matmul (include/kernels_amx.hpp:1216-1253,
+// 1297-1302), for Matmul<bf16,int8,float> at small M (:1381-1441) and for matmul16m_Wint8B
+// (weight_compression/fc16m.cpp:451-502).  The kernel is a weight stream: every byte of W is read
+// exactly once, in 1 KiB lane-contiguous fragments of the same packed layout the tile GEMM uses.
+// The few activations ride in the other MFMA operand (32 columns, only M of them live), so the
+// matrix core does the multiply-accumulate while the vector ALU only converts int8 -> bf16
+// (exact: |w| <= 128 has at most 8 significant bits, as in include/kernels_amx.hpp:490-506).
+// K is split across the 8 wavefronts of a workgroup; partial 32x32 blocks are summed through LDS.
+#include "common.hpp"
+
+namespace mmx {
+
+struct SkinnyArgs {
+    const char* x;
+    int64_t ldx;  // bytes
+    const char* Wp;
+    int64_t panel_stride;  // bytes
+    int M, K;
+    int nfrag;    // 1 KiB fragments per panel
+    int npanels;  // panels in Wp
+    int n0, n1;
+    int x_vec_ok;
+    Epilogue ep;
+};
+
+__device__ __forceinline__ bf16x8 load_x8(const char* xrow, int k0, int K, bool live, bool vec_ok) {
+    bf16x8 v;
+#pragma unroll
+    for (int e = 0; e < 8; e++) v[e] = (__bf16)0.0f;
+    if (!live || k0 >= K) return v;
+    if (vec_ok && k0 + 8 <= K) return *reinterpret_cast<const bf16x8*>(xrow + (int64_t)k0 * 2);
+    const __bf16* p = reinterpret_cast<const __bf16*>(xrow);
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+        if (k0 + e < K) v[e] = p[k0 + e];
+    return v;
+}
+
+// 8 int8 (two dwords) -> 8 bf16, exact
+__device__ __forceinline__ bf16x8 s8x8_to_bf16(uint32_t lo, uint32_t hi) {
+    bf16x8 r;
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+        r[b] = (__bf16)(float)(int8_t)((lo >> (8 * b)) & 0xff);
+        r[4 + b] = (__bf16)(float)(int8_t)((hi >> (8 * b)) & 0xff);
+    }
+    return r;
+}
+
+__device__ __forceinline__ void store_out(const Epilogue& ep, int m, int n, float r) {
+    char* row = ep.C + (int64_t)m * ep.ldc;
+    switch (ep.out_dtype) {
+    case MMX_BF16: reinterpret_cast<uint16_t*>(row)[n] = to_bf16(r); break;
+    case MMX_I8: reinterpret_cast<int8_t*>(row)[n] = to_s8_sat(r); break;
+    default: reinterpret_cast<float*>(row)[n] = r; break;
+    }
+}
+
+template <bool W8, int NP>
+__global__ __launch_bounds__(512) void skinny_kernel(const SkinnyArgs s) {
+    constexpr int U = 4;  // fragments in flight per wave
+    __shared__ float red[8][NP][16][64];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, g32 = lane >> 5;
+    const int panel_first = (s.n0 >> 5) + blockIdx.x * NP;
+    const int panel_end = (s.n1 + 31) >> 5;
+
+    f32x16 acc[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[p][v] = 0.0f;
+
+    const int per_wave = (s.nfrag + 7) / 8;
+    const int f_begin = wave * per_wave;
+    const int f_end = (f_begin + per_wave) < s.nfrag ? (f_begin + per_wave) : s.nfrag;
+    const bool live = l32 < s.M;
+    const char* xrow = s.x + (int64_t)(live ? l32 : 0) * s.ldx;
+
+    for (int f0 = f_begin; f0 < f_end; f0 += U) {
+        u32x4 w[NP][U];
+        bf16x8 xa[U], xb[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int f = f0 + u;
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                const int panel = panel_first + p;
+                w[p][u] = u32x4{0u, 0u, 0u, 0u};
+                if (f < f_end && panel < panel_end && panel < s.npanels)
+                    w[p][u] = *reinterpret_cast<const u32x4*>(s.Wp + (int64_t)panel * s.panel_stride +
+                                                              (int64_t)f * 1024 + lane * 16);
+            }
+            if constexpr (W8) {
+                const int k0 = 32 * f + 16 * g32;
+                xa[u] = load_x8(xrow, k0, s.K, live && f < f_end, s.x_vec_ok);
+                xb[u] = load_x8(xrow, k0 + 8, s.K, live && f < f_end, s.x_vec_ok);
+            } else {
+                xa[u] = load_x8(xrow, 16 * f + 8 * g32, s.K, live && f < f_end, s.x_vec_ok);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                if constexpr (W8) {
+                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(w[p][u].x, w[p][u].y), xa[u], acc[p], 0, 0, 0);
+                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(w[p][u].z, w[p][u].w), xb[u], acc[p], 0, 0, 0);
+                } else {
+                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w[p][u]), xa[u], acc[p], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int p = 0; p < NP; p++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) red[wave][p][v][lane] = acc[p][v];
+    __syncthreads();
+
+    const Epilogue& ep = s.ep;
+    for (int idx = tid; idx < 16 * 64; idx += 512) {
+        const int v = idx >> 6, ln = idx & 63;
+        const int m = ln & 31;
+        if (m >= s.M) continue;
+        const int nloc = 8 * (v >> 2) + 4 * (ln >> 5) + (v & 3);
+        float sum[NP];
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            float t = 0.0f;
+#pragma unroll
+            for (int w8 = 0; w8 < 8; w8++) t += red[w8][p][v][ln];
+            sum[p] = t;
+        }
+        if (ep.steps & MMX_PP_SILU_GATE) {
+            if constexpr (NP == 2) {
+                const int n = ((panel_first >> 1) << 5) + nloc;  // output column (half width)
+                if (n < (s.n1 >> 1)) store_out(ep, m, n, silu(sum[0]) * sum[1]);
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                const int n = ((panel_first + p) << 5) + nloc;
+                if (n >= s.n1) continue;
+                float r = sum[p];
+                if (ep.steps & MMX_PP_DEQUANT) r = r * (ep.deq_oc ? ep.deq_oc[n] : ep.deq);
+                if (ep.steps & MMX_PP_BIAS) r = r + ep.bias[n];
+                if (ep.steps & MMX_PP_GELU) r = gelu_erf_minimax(r);
+                if (ep.steps & MMX_PP_QUANT) r = r * (ep.q_oc ? ep.q_oc[n] : ep.q);
+                store_out(ep, m, n, r);
+            }
+        }
+    }
+}
+
+int launch_skinny(bool w8, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
+                  const Epilogue& ep, hipStream_t st) {
+    SkinnyArgs s;
+    s.x = static_cast<const char*>(x);
+    s.ldx = ldx;
+    s.Wp = static_cast<const char*>(Wp);
+    s.M = M;
+    s.K = K;
+    const int kbytes_pad = ((K * (w8 ? 1 : 2)) + 127) / 128 * 128;
+    s.nfrag = kbytes_pad / 32;  // 32 bytes of K per column per fragment
+    s.panel_stride = (int64_t)s.nfrag * 1024;
+    s.npanels = (N + 31) / 32;
+    s.n0 = n0;
+    s.n1 = n1;
+    s.x_vec_ok = ((reinterpret_cast<uintptr_t>(x) & 15) == 0) && ((ldx & 15) == 0);
+    s.ep = ep;
+    const int panels = ((n1 + 31) >> 5) - (n0 >> 5);
+    const bool pairs = (ep.steps & MMX_PP_SILU_GATE) != 0;
+    if (pairs) {
+        if (panels & 1) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
+        note_kernel(w8 ? "skinny_w8_gateup" : "skinny_bf16_gateup");
+        if (w8) hipLaunchKernelGGL((skinny_kernel<true, 2>), dim3(panels / 2), dim3(512), 0, st, s);
+        else hipLaunchKernelGGL((skinny_kernel<false, 2>), dim3(panels / 2), dim3(512), 0, st, s);
+    } else {
+        note_kernel(w8 ? "skinny_w8" : "skinny_bf16");
+        if (w8) hipLaunchKernelGGL((skinny_kernel<true, 1>), dim3(panels), dim3(512), 0, st, s);
+        else hipLaunchKernelGGL((skinny_kernel<false, 1>), dim3(panels), dim3(512), 0, st, s);
+    }
+    return check_hip(hipGetLastError(), "skinny_kernel launch");
+}
+
+}  // namespace mmx

@@ -1,0 +1,369 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU oracle on the same
+seeded inputs.  Integer results bit-exact; floating point within relative Frobenius error 1e-3
+with >= 99.9 % of the elements within one bf16 ulp."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import bf16_to_f32, check_float_parity, dev, dev_bf16, host_bits
+
+pytestmark = pytest.mark.gpu
+
+import mm_amx_amd as mx  # noqa: E402
+from mm_amx_amd import workloads as wl  # noqa: E402
+
+# main.cpp:715-735 (K tails, N=5, M=2, M and N tails), the two N=10752 shapes cut to N=192
+FC_SHAPES = [(16, 65, 32), (16, 66, 32), (16, 67, 32), (16, 68, 32), (16, 69, 32), (32, 64, 5), (128, 96, 16),
+             (2, 2560, 192), (2, 337, 271), (22, 2560, 192), (704, 320, 256), (705, 320, 257), (720, 320, 273),
+             (735, 320, 271), (735, 321, 271), (735, 337, 271), (2, 320, 256)]
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    mx.init(0)
+    mx.set_tile("")
+    mx.set_option("load_mode", 0)
+    yield
+    mx.set_tile("")
+    mx.set_option("load_mode", 0)
+
+
+def rand_bf16(rng, shape, std):
+    return wl.f32_to_bf16_bits((rng.standard_normal(shape) * std).astype(np.float32))
+
+
+# ---- weight repack ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("dt", ["bf16", "int8"])
+@pytest.mark.parametrize("shape", [(64, 32), (70, 45), (256, 96), (129, 33), (4096, 64)])
+def test_repack_matches_layout_spec(po, dt, shape):
+    K, N = shape
+    rng = np.random.default_rng(K * 1000 + N)
+    B = rng.integers(1, 30000, (K, N)).astype(np.uint16) if dt == "bf16" else rng.integers(-127, 128, (K, N)).astype(np.int8)
+    want = po.repack(B, layout="mfma")
+    up = dev_bf16 if dt == "bf16" else dev
+    got = host_bits(mx.repack_b(up(B)))
+    assert np.array_equal(got, want)
+    gotT = host_bits(mx.repack_b(up(np.ascontiguousarray(B.T)), transpose=True))
+    assert np.array_equal(gotT, want)
+
+
+# ---- bf16 FC -----------------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", FC_SHAPES)
+def test_bf16_fc_shapes(po, shape):
+    """fp32 accumulators for the reference's shape list, both B layouts (main.cpp:236-267)."""
+    M, K, N = shape
+    if K < 32:
+        pytest.skip("K >= kStep")
+    rng = np.random.default_rng(sum(shape))
+    A, B = rand_bf16(rng, (M, K), 1.0), rand_bf16(rng, (K, N), 0.05)
+    ref = po.gemm_bf16(A, B)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    mm = mx.Matmul(True, False)
+    mm(dev_bf16(A), dev_bf16(B), ppkernel=mx.BiasGeluStore(C))
+    check_float_parity(host_bits(C), ref, f"bf16 fc {shape}")
+    C2 = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    mmT = mx.Matmul(True, True)
+    mmT(dev_bf16(A), dev_bf16(np.ascontiguousarray(B.T)), ppkernel=mx.BiasGeluStore(C2))
+    assert np.array_equal(host_bits(C2), host_bits(C))
+
+
+def test_bf16_exact_inputs_are_bit_exact(po):
+    """+-0.5 inputs as the reference's fill_rnd (include/tensor2D.hpp:145-172): every summation order is
+    exact, so the GPU must give the oracle's bits."""
+    rng = np.random.default_rng(5)
+    M, K, N = 289, 448, 200
+    A = wl.f32_to_bf16_bits(rng.integers(0, 2, (M, K)).astype(np.float32) - 0.5)
+    B = wl.f32_to_bf16_bits(rng.integers(0, 2, (K, N)).astype(np.float32) - 0.5)
+    C = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    mx.Matmul(True, False)(dev_bf16(A), dev_bf16(B), ppkernel=mx.BiasGeluStore(C))
+    assert np.array_equal(host_bits(C), po.gemm_bf16(A, B))
+
+
+@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x128"])
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_bf16_bias_gelu_every_kernel_variant(po, tile, mode):
+    M, K, N = 600, 512, 832
+    rng = np.random.default_rng(11)
+    A, B = rand_bf16(rng, (M, K), 1.0), rand_bf16(rng, (K, N), 0.05)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    ref = po.pp(po.gemm_bf16(A, B), po.PP_BIAS | po.PP_GELU, po.BF16, bias=bias)
+    mx.set_tile(tile)
+    mx.set_option("load_mode", mode)
+    try:
+        C = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+        mm = mx.Matmul(True, False)
+        mm(dev_bf16(A), dev_bf16(B), ppkernel=mx.BiasGeluStore(C, mx.Steps.BIAS_GELU, dev(bias)))
+        kernel = mx.last_kernel()
+        assert tile in kernel and f"mode{mode}" in kernel, kernel
+        check_float_parity(bf16_to_f32(host_bits(C)), bf16_to_f32(ref), f"bias_gelu {tile} mode{mode}")
+    finally:
+        mx.set_tile("")
+        mx.set_option("load_mode", 0)
+
+
+def test_bf16_256_cube(po):
+    """bf16 256^3, U[-1,1], fp32 out (shape of tests/amx-l2.cpp:206-241)."""
+    w = wl.gemm_bf16_256()
+    C = torch.empty((256, 256), dtype=torch.float32, device="cuda")
+    mx.Matmul(True, False)(dev_bf16(w["A"]), dev_bf16(w["B"]), ppkernel=mx.BiasGeluStore(C))
+    err, frac = check_float_parity(host_bits(C), po.gemm_bf16(w["A"], w["B"]), "256^3")
+    assert err < 1e-5
+
+
+@pytest.mark.parametrize("M", [128, 1024])
+def test_ffn_up_bias_gelu_full_size(po, M):
+    """The headline FC at its real shape: K=4096, N=11008, BIAS_GELU -> bf16."""
+    w = wl.ffn_up_bias_gelu(M=M)
+    ref = po.pp(po.gemm_bf16(w["A"], w["B"]), po.PP_BIAS | po.PP_GELU, po.BF16, bias=w["bias"])
+    C = torch.zeros((M, w["N"]), dtype=torch.bfloat16, device="cuda")
+    mm = mx.Matmul(True, False)
+    mm(dev_bf16(w["A"]), dev_bf16(w["B"]), ppkernel=mx.BiasGeluStore(C, mx.Steps.BIAS_GELU, dev(w["bias"])))
+    err, frac = check_float_parity(bf16_to_f32(host_bits(C)), bf16_to_f32(ref), f"ffn_up M={M}")
+    print(f"ffn_up M={M}: rel_fro={err:.2e} within_1ulp={frac * 100:.4f}% kernel={mx.last_kernel()}")
+
+
+def test_column_range_split_equals_whole(po):
+    """The reference's single-thread == N-split check (main.cpp:517-525): computing [n0,n1) ranges
+    one by one must give the bits of one whole-N call."""
+    M, K, N = 160, 256, 416
+    rng = np.random.default_rng(12)
+    A, B = rand_bf16(rng, (M, K), 1.0), rand_bf16(rng, (K, N), 0.05)
+    bias = dev((rng.standard_normal(N) * 0.1).astype(np.float32))
+    Ad, Bd = dev_bf16(A), dev_bf16(B)
+    whole = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    mm = mx.Matmul(True, False)
+    mm(Ad, Bd, ppkernel=mx.BiasGeluStore(whole, mx.Steps.BIAS_GELU, bias))
+    parts = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    work = (N + 31) // 32
+    for t in range(3):
+        s, e = po.splitter(work, 3, t)
+        n0, n1 = s * 32, min(e * 32, N)
+        mm(Ad, Bd, n0, n1, ppkernel=mx.BiasGeluStore(parts, mx.Steps.BIAS_GELU, bias))
+    assert np.array_equal(host_bits(parts), host_bits(whole))
+
+
+# ---- int8 FC -----------------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [s for s in FC_SHAPES if s[1] >= 64])
+def test_int8_accumulators_bit_exact(po, shape):
+    M, K, N = shape
+    rng = np.random.default_rng(sum(shape) + 1)
+    A = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    C = torch.full((M, N), -7, dtype=torch.int32, device="cuda")
+    packed = mx.repack_b(dev(B))
+    mx.gemm(dev(A), packed, N, mx.Epilogue(C, mx.PP_NONE))
+    assert np.array_equal(host_bits(C), po.gemm_i8(A, B))
+
+
+@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x128"])
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_int8_requant_every_kernel_variant(po, tile, mode):
+    M, K, N = 520, 1024, 704
+    rng = np.random.default_rng(13)
+    A = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    deq = (np.float32(0.02) * rng.uniform(1e-3, 1e-2, N).astype(np.float32)).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    steps = po.PP_DEQUANT | po.PP_BIAS | po.PP_QUANT
+    ref = po.pp(po.gemm_i8(A, B), steps, po.I8, bias=bias, deq_per_oc=deq, q=20.0)
+    mx.set_tile(tile)
+    mx.set_option("load_mode", mode)
+    try:
+        C = torch.zeros((M, N), dtype=torch.int8, device="cuda")
+        pp = mx.BiasGeluStore(C, mx.Steps.DEQUANT | mx.Steps.BIAS | mx.Steps.QUANT, dev(bias))
+        pp.set_deq_scale(dev(deq))
+        pp.set_q_scale(20.0)
+        mx.Matmul(True, False)(dev(A), dev(B), ppkernel=pp)
+        assert tile in mx.last_kernel() and f"mode{mode}" in mx.last_kernel()
+        assert np.array_equal(host_bits(C), ref)
+    finally:
+        mx.set_tile("")
+        mx.set_option("load_mode", 0)
+
+
+def test_int8_fc_full_size(po):
+    """int8 FC at its real shape (M=512, K=N=4096): int32 accumulators and requantised int8 bit-exact."""
+    w = wl.int8_fc()
+    acc_ref = po.gemm_i8(w["A"], w["B"])
+    steps = po.PP_DEQUANT | po.PP_BIAS | po.PP_QUANT
+    out_ref = po.pp(acc_ref, steps, po.I8, bias=w["bias"], deq_per_oc=w["deq"], q=float(w["q"]))
+    Ad, packed = dev(w["A"]), mx.repack_b(dev(w["B"]))
+    acc = torch.zeros((w["M"], w["N"]), dtype=torch.int32, device="cuda")
+    mx.gemm(Ad, packed, w["N"], mx.Epilogue(acc, mx.PP_NONE))
+    assert np.array_equal(host_bits(acc), acc_ref)
+    out = torch.zeros((w["M"], w["N"]), dtype=torch.int8, device="cuda")
+    mx.gemm(Ad, packed, w["N"], mx.Epilogue(out, steps, bias=dev(w["bias"]), deq_scale_per_oc=dev(w["deq"]),
+                                            q_scale=float(w["q"])))
+    assert np.array_equal(host_bits(out), out_ref)
+    sat = np.mean(np.abs(out_ref.astype(np.int32)) >= 127)
+    print(f"int8 fc: kernel={mx.last_kernel()} saturated={sat * 100:.1f}%")
+
+
+def test_int8_gelu_quant_per_channel(po):
+    M, K, N = 88, 128, 66
+    rng = np.random.default_rng(14)
+    A = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    qoc = rng.uniform(5, 40, N).astype(np.float32)
+    ref = po.pp(po.gemm_i8(A, B), 15, po.I8, bias=bias, deq=1e-4, q_per_oc=qoc)
+    C = torch.zeros((M, N), dtype=torch.int8, device="cuda")
+    pp = mx.BiasGeluStore(C, mx.Steps.DEQUANT_BIAS_GELU_QUANT, dev(bias))
+    pp.set_deq_scale(1e-4)
+    pp.set_q_scale(dev(qoc))
+    mx.Matmul(True, False)(dev(A), dev(B), ppkernel=pp)
+    assert np.array_equal(host_bits(C), ref)
+
+
+# ---- decode GEMV over int8-compressed weights ----------------------------------------------------------
+@pytest.mark.parametrize("M", [1, 4, 16])
+def test_decode_gemv_w8_full_size(po, M):
+    w = wl.decode_gemv_w8(M=M)
+    ref = po.gemv_w8(w["x"], w["W"], w["scale"])
+    packed = mx.repack_b(dev(w["W"]))
+    y = torch.zeros((M, w["N"]), dtype=torch.bfloat16, device="cuda")
+    mx.gemm(dev_bf16(w["x"]), packed, w["N"], mx.Epilogue(y, mx.PP_DEQUANT, deq_scale_per_oc=dev(w["scale"])),
+            b_dtype=mx.I8)
+    assert "skinny_w8" in mx.last_kernel()
+    err, frac = check_float_parity(bf16_to_f32(host_bits(y)), bf16_to_f32(ref), f"gemv_w8 M={M}")
+    print(f"gemv_w8 M={M}: rel_fro={err:.2e} within_1ulp={frac * 100:.4f}%")
+
+
+@pytest.mark.parametrize("shape", [(1, 256, 64), (3, 320, 100), (16, 337, 96), (32, 2560, 192), (7, 70, 45)])
+@pytest.mark.parametrize("w8", [False, True])
+def test_decode_small_shapes(po, shape, w8):
+    M, K, N = shape
+    rng = np.random.default_rng(sum(shape) + int(w8))
+    x = rand_bf16(rng, (M, K), 1.0)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    if w8:
+        W = np.clip(np.rint(rng.standard_normal((K, N)) * 40), -127, 127).astype(np.int8)
+        scale = rng.uniform(1e-3, 5e-3, N).astype(np.float32)
+        _, acc = po.gemv_w8(x, W, scale, want_acc=True)
+        ref = po.pp(acc, po.PP_DEQUANT | po.PP_BIAS | po.PP_GELU, po.F32, bias=bias, deq_per_oc=scale)
+        packed = mx.repack_b(dev(W))
+        y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_DEQUANT | mx.PP_BIAS | mx.PP_GELU, bias=dev(bias),
+                                                    deq_scale_per_oc=dev(scale)), b_dtype=mx.I8)
+    else:
+        W = rand_bf16(rng, (K, N), 0.05)
+        ref = po.pp(po.gemm_bf16(x, W), po.PP_BIAS | po.PP_GELU, po.F32, bias=bias)
+        packed = mx.repack_b(dev_bf16(W))
+        y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_BIAS | mx.PP_GELU, bias=dev(bias)))
+    assert "skinny" in mx.last_kernel()
+    # GELU flattens tiny pre-activations: compare on an absolute scale as well as by ulp
+    got = host_bits(y)
+    assert np.linalg.norm(got - ref) <= 1e-3 * np.linalg.norm(ref)
+    assert np.mean(np.abs(got - ref) <= np.maximum(2.0 ** -8 * np.abs(ref), 1e-6)) >= 0.999
+
+
+@pytest.mark.parametrize("M", [4, 40])
+def test_weight_compressed_matmul(po, M):
+    """Matmul<bf16,int8,float>: bf16 weights compressed per tensor inside the op (include/kernels_amx.hpp:1363-1379)."""
+    K, N = 512, 160
+    rng = np.random.default_rng(15)
+    A, W = rand_bf16(rng, (M, K), 1.0), rand_bf16(rng, (K, N), 0.02)
+    Wq, dq, q = po.quantize_weights(W)
+    _, acc = po.gemv_w8(A, Wq, np.ones(N, np.float32), want_acc=True)
+    ref = po.pp(acc, po.PP_DEQUANT, po.F32, deq=dq)
+    C = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    mm = mx.Matmul(True, False, weight_int8=True)
+    mm(dev_bf16(A), dev_bf16(W), ppkernel=mx.BiasGeluStore(C, mx.Steps.DEQUANT))
+    assert np.float32(mm.dequant_scale_B) == np.float32(dq) and np.float32(mm.quant_scale_B) == np.float32(q)
+    check_float_parity(host_bits(C), ref, f"w8 matmul M={M}")
+    # the compressed weights themselves are integer work: bit-exact
+    Wq_gpu, _ = mx.quantize_weights(dev_bf16(W))
+    assert np.array_equal(host_bits(Wq_gpu), Wq)
+
+
+# ---- mat-vec ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(901, 80), (901, 96), (64, 4096), (37, 33)])
+def test_matvec(po, shape):
+    M, K = shape
+    rng = np.random.default_rng(16)
+    A, b = rand_bf16(rng, (M, K), 1.0), rand_bf16(rng, (K,), 1.0)
+    c = mx.MatmulVector()(dev_bf16(A), dev_bf16(b))
+    ref = po.matvec_bf16(A, b)
+    assert np.linalg.norm(host_bits(c) - ref) <= 1e-5 * np.linalg.norm(ref)
+    c2 = mx.GemAvB()(dev_bf16(A), dev_bf16(b)) if K >= 32 else c
+    assert np.array_equal(host_bits(c2), host_bits(c))
+    Ai = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    bi = rng.integers(-127, 128, K, dtype=np.int8)
+    ci = mx.MatmulVector()(dev(Ai), dev(bi))
+    assert np.array_equal(host_bits(ci), po.matvec_i8(Ai, bi))
+
+
+# ---- fused MLP ---------------------------------------------------------------------------------------------
+def _mlp_case(po, M, K, N, seed):
+    w = wl.llama_mlp(M=M, K=K, N=N, seed=seed)
+    h_ref, _ = po.mlp(w["x"], w["w_gate"], w["w_up"], w["w_down"], split_k=True)
+    m = mx.MLP()
+    m.setup(dev_bf16(w["w_gate"]), dev_bf16(w["w_up"]), dev_bf16(w["w_down"]))
+    y = m.run(dev_bf16(w["x"]))
+    h = host_bits(m.actUp[:M])
+    # stage 1: h from the same x
+    e1, f1 = check_float_parity(bf16_to_f32(h), bf16_to_f32(h_ref), f"mlp h M={M}")
+    # stage 2: y from the SAME h the GPU produced (chained parity is not attainable by ulp: the
+    # down projection is a cancelling sum, so one-ulp changes of h move small y by many ulps)
+    y_ref = po.mlp_down(h, w["w_down"], split_k=True)
+    e2, f2 = check_float_parity(bf16_to_f32(host_bits(y)), bf16_to_f32(y_ref), f"mlp y M={M}")
+    # end to end, reported and bounded by Frobenius error only
+    _, y_e2e = po.mlp(w["x"], w["w_gate"], w["w_up"], w["w_down"], split_k=True)
+    yf, rf = bf16_to_f32(host_bits(y)).astype(np.float64), bf16_to_f32(y_e2e).astype(np.float64)
+    e3 = np.linalg.norm(yf - rf) / np.linalg.norm(rf)
+    print(f"mlp M={M}: h rel={e1:.2e} ({f1 * 100:.3f}% <=1ulp)  y|h rel={e2:.2e} ({f2 * 100:.3f}%)  end-to-end rel={e3:.2e}")
+    assert e3 < 3e-3
+
+
+@pytest.mark.parametrize("M", [1, 5, 48, 300])
+def test_mlp_small(po, M):
+    _mlp_case(po, M, 512, 768, seed=20 + M)
+
+
+@pytest.mark.parametrize("M", [1, 256])
+def test_mlp_llama7b_shape(po, M):
+    _mlp_case(po, M, 4096, 11008, seed=30 + M)
+
+
+# ---- torch-ext call shape -------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(32, 32, 32), (32, 32, 4096), (512, 128, 4096)])
+def test_linear_nxn_integer_inputs(shape):
+    """torch-ext/test.py:14-37: integer-valued inputs in [-10, 10] are exact in bf16 and fp32."""
+    M, N, K = shape
+    g = torch.Generator().manual_seed(0)
+    w = torch.randint(-10, 11, (N, K), generator=g, dtype=torch.float32)
+    x = torch.randint(-10, 11, (M, K), generator=g, dtype=torch.float32)
+    y0 = x.double() @ w.double().T
+    lin = mx.LinearNxN()
+    lin.set_weight(w.to(torch.bfloat16).cuda())
+    y1 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    lin.forward(x.to(torch.bfloat16).cuda(), y1)
+    assert torch.equal(y1.cpu().double(), y0)
+    import copy
+    lin2 = copy.deepcopy(lin)
+    y2 = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    lin2.forward(x.to(torch.bfloat16).cuda(), y2)
+    assert torch.equal(y2, y1)
+
+
+# ---- error behaviour --------------------------------------------------------------------------------------
+def test_errors_are_loud():
+    A = torch.zeros((64, 64), dtype=torch.bfloat16, device="cuda")
+    B = torch.zeros((64, 64), dtype=torch.bfloat16, device="cuda")
+    C = torch.zeros((64, 64), dtype=torch.float32, device="cuda")
+    packed = mx.repack_b(B)
+    with pytest.raises(mx.MmxError, match="multiple of 32"):
+        mx.gemm(A, packed, 64, mx.Epilogue(C), n0=8, n1=64)
+    with pytest.raises(mx.MmxError, match="column range"):
+        mx.gemm(A, packed, 64, mx.Epilogue(C), n0=0, n1=96)
+    with pytest.raises(mx.MmxError, match="BIAS step without"):
+        mx.gemm(A, packed, 64, mx.Epilogue(C, mx.PP_BIAS))
+    with pytest.raises(mx.MmxError, match="K = 16"):
+        mx.Matmul()(A[:, :16], B[:16], ppkernel=mx.BiasGeluStore(C))
+    with pytest.raises(mx.MmxError, match="not enabled"):
+        mx.BiasGeluStore(C, mx.Steps.NONE).set_q_scale(2.0)
+    with pytest.raises(mx.MmxError, match="multiples of 32"):
+        mx.LinearNxN().set_weight(torch.zeros((40, 64), dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(mx.MmxError, match="on the GPU"):
+        mx.repack_b(torch.zeros((64, 64), dtype=torch.bfloat16))
