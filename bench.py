@@ -1,0 +1,195 @@
+#!/usr/bin/env python3
+"""Benchmark of the FC-GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+
+One "step" is one pass of the hot path over one batch of synthetic input: the Llama-7B FFN
+up-projection FC, bf16, M=1024, K=4096, N=11008, fused BIAS+GELU epilogue, bf16 output, with the
+activations, the packed weights and the bias already resident in HBM when the timed region starts.
+Prints ONE JSON line.  `value` is TFLOP/s of that FC (flops = 2*M*N*K, the reference's convention,
+main.cpp:279); `roofline` holds the same kernel against the MI355X dense bf16 MFMA peak, timed with
+HIP events on the launch stream; `cpu_baseline` is the CPU restatement of the reference path
+(oracle/) timed on this machine's host cores on the same workload; `extra` reports the other
+configurations of the path (int8 FC, decode GEMV over int8 weights, fused MLP).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_INT8_TOPS = 5000.0     # MI355X dense int8 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (the path shards over N by column panels; see DESIGN.md); "
+                 "--gpus must be 1")
+
+    import numpy as np
+    import torch
+
+    import mm_amx_amd as mx
+    from mm_amx_amd import workloads as wl
+    from gpu_util import dev, dev_bf16
+
+    torch.cuda.set_device(0)
+    mx.init(0)
+
+    # ---- headline: bf16 FC + BIAS_GELU, M=1024 ------------------------------------------------------
+    w = wl.ffn_up_bias_gelu(M=1024)
+    M, K, N = w["M"], w["K"], w["N"]
+    A = dev_bf16(w["A"])
+    Bp = mx.repack_b(dev_bf16(w["B"]))   # one-off, untimed (the reference caches it under constB)
+    bias = dev(w["bias"])
+    C = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    ep = mx.Epilogue(C, mx.PP_BIAS | mx.PP_GELU, bias=bias)
+    flops = 2.0 * M * N * K
+
+    def step():
+        mx.gemm(A, Bp, N, ep)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()                       # same stream the kernels are launched on (torch's current stream)
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    kernel_ms = e0.elapsed_time(e1) / args.steps
+    kernel_name = mx.last_kernel()
+    value = flops / (ms_per_step * 1e-3) / 1e12
+    achieved = flops / (kernel_ms * 1e-3) / 1e12
+
+    out = {
+        "metric": "bf16 FC GEMM TFLOP/s (M=1024, K=4096, N=11008, fused BIAS+GELU, bf16 out)",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "llama7b_ffn_up_bf16_bias_gelu", "M": M, "K": K, "N": N, "kernel": kernel_name,
+                   "inputs": "A~N(0,1) bf16, B~N(0,0.02) bf16 repacked once, bias~N(0,0.1) fp32, all resident in HBM"},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "kernel_avg_us": round(kernel_ms * 1e3, 2)},
+    }
+
+    # ---- CPU baseline: the oracle (a port of the reference path) on this host's cores --------------
+    if not args.no_cpu:
+        from oracle import pyoracle as po
+        cores = os.cpu_count() or 1
+        try:
+            cores = len(os.sched_getaffinity(0))
+        except AttributeError:
+            pass
+        cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+        reps = 0
+        t0 = time.perf_counter()
+        while True:
+            acc = po.gemm_bf16(w["A"], w["B"], nthreads=cores)
+            po.pp(acc, po.PP_BIAS | po.PP_GELU, po.BF16, bias=w["bias"])
+            reps += 1
+            el = time.perf_counter() - t0
+            if el > 10.0 or reps >= 20:
+                break
+        out["cpu_baseline"] = {
+            "value": round(flops * reps / el / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"{reps} x the full workload (M=1024,K=4096,N=11008 + BIAS_GELU) in {el:.1f} s; portable "
+                      f"{po.isa()} restatement of the AMX summation order (the host "
+                      f"{'has' if po.host_has_amx() else 'has no'} AMX; the AMX intrinsics path is not used)",
+        }
+
+    # ---- the other configurations of the path --------------------------------------------------------
+    if not args.no_extra:
+        extra = {}
+
+        def avg_ms(Ain, packs, Nn, epi, iters, **kw):
+            mx.time_gemm(Ain, packs, Nn, epi, max(3, iters // 10), **kw)
+            return mx.time_gemm(Ain, packs, Nn, epi, iters, **kw)
+
+        # bf16 FC sweep over M
+        sweep = {}
+        for Ms in (128, 512, 2048):
+            ws = wl.ffn_up_bias_gelu(M=Ms)
+            As = dev_bf16(ws["A"])
+            Cs = torch.zeros((Ms, N), dtype=torch.bfloat16, device="cuda")
+            ms = avg_ms(As, [Bp], N, mx.Epilogue(Cs, mx.PP_BIAS | mx.PP_GELU, bias=bias), 30)
+            sweep[str(Ms)] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * Ms * N * K / ms / 1e9, 1),
+                              "kernel": mx.last_kernel()}
+            del As, Cs
+        extra["bf16_fc_bias_gelu_sweep_M"] = sweep
+
+        # int8 FC with dequant/bias/requant
+        wi = wl.int8_fc()
+        Ai, Bi = dev(wi["A"]), mx.repack_b(dev(wi["B"]))
+        Ci = torch.zeros((wi["M"], wi["N"]), dtype=torch.int8, device="cuda")
+        epi = mx.Epilogue(Ci, mx.PP_DEQUANT | mx.PP_BIAS | mx.PP_QUANT, bias=dev(wi["bias"]),
+                          deq_scale_per_oc=dev(wi["deq"]), q_scale=float(wi["q"]))
+        ms = avg_ms(Ai, [Bi], wi["N"], epi, 100)
+        ops = 2.0 * wi["M"] * wi["K"] * wi["N"]
+        extra["int8_fc_requant_M512_K4096_N4096"] = {
+            "us": round(ms * 1e3, 2), "tops": round(ops / ms / 1e9, 1), "frac_of_int8_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4),
+            "kernel": mx.last_kernel()}
+        del Ai, Bi, Ci
+
+        # decode GEMV over int8 weights, rotating over 12 weight copies (540 MB > 256 MB of cache)
+        gemv = {}
+        for Mg in (1, 4, 16):
+            wg = wl.decode_gemv_w8(M=Mg)
+            xg, Wg, sg = dev_bf16(wg["x"]), mx.repack_b(dev(wg["W"])), dev(wg["scale"])
+            packs = [Wg] + [Wg.clone() for _ in range(11)]
+            yg = torch.zeros((Mg, wg["N"]), dtype=torch.bfloat16, device="cuda")
+            epg = mx.Epilogue(yg, mx.PP_DEQUANT, deq_scale_per_oc=sg)
+            ms = avg_ms(xg, packs, wg["N"], epg, 240, b_dtype=mx.I8)
+            wbytes = float(wg["K"]) * wg["N"]
+            gemv[str(Mg)] = {"us": round(ms * 1e3, 2), "weight_GBps": round(wbytes / ms / 1e6, 0),
+                             "frac_of_hbm_peak": round(wbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "kernel": mx.last_kernel()}
+            del packs, Wg
+        extra["decode_gemv_int8w_K4096_N11008"] = gemv
+
+        # fused Llama-7B MLP
+        mlp = {}
+        wm = wl.llama_mlp(M=2048)
+        op = mx.MLP()
+        op.setup(dev_bf16(wm["w_gate"]), dev_bf16(wm["w_up"]), dev_bf16(wm["w_down"]))
+        for Mm in (1, 2048):
+            xm = dev_bf16(wm["x"][:Mm])
+            ym = torch.zeros((Mm, wm["K"]), dtype=torch.bfloat16, device="cuda")
+            for _ in range(3):
+                op.run(xm, ym)
+            torch.cuda.synchronize()
+            a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a0.record()
+            for _ in range(20):
+                op.run(xm, ym)
+            a1.record()
+            torch.cuda.synchronize()
+            ms = a0.elapsed_time(a1) / 20
+            fl = 6.0 * Mm * wm["K"] * wm["N"]
+            mlp[str(Mm)] = {"us": round(ms * 1e3, 1), "tflops": round(fl / ms / 1e9, 1),
+                            "weight_GBps": round(3.0 * wm["K"] * wm["N"] * 2 / ms / 1e6, 0)}
+        extra["llama7b_mlp_fused"] = mlp
+        out["extra"] = extra
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from gpu_util import bf16_to_f32, check_float_parity, dev, dev_bf16, host_bits
+from gpu_util import bf16_to_f32, check_float_parity, check_gelu_parity, dev, dev_bf16, host_bits
 
 pytestmark = pytest.mark.gpu
 
@@ -86,16 +86,22 @@ def test_bf16_bias_gelu_every_kernel_variant(po, tile, mode):
     rng = np.random.default_rng(11)
     A, B = rand_bf16(rng, (M, K), 1.0), rand_bf16(rng, (K, N), 0.05)
     bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
-    ref = po.pp(po.gemm_bf16(A, B), po.PP_BIAS | po.PP_GELU, po.BF16, bias=bias)
+    acc_ref = po.gemm_bf16(A, B)
+    ref = po.pp(acc_ref, po.PP_BIAS | po.PP_GELU, po.BF16, bias=bias)
     mx.set_tile(tile)
     mx.set_option("load_mode", mode)
     try:
         C = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+        acc = torch.zeros((M, N), dtype=torch.float32, device="cuda")
         mm = mx.Matmul(True, False)
         mm(dev_bf16(A), dev_bf16(B), ppkernel=mx.BiasGeluStore(C, mx.Steps.BIAS_GELU, dev(bias)))
         kernel = mx.last_kernel()
         assert tile in kernel and f"mode{mode}" in kernel, kernel
-        check_float_parity(bf16_to_f32(host_bits(C)), bf16_to_f32(ref), f"bias_gelu {tile} mode{mode}")
+        mm(dev_bf16(A), dev_bf16(B), ppkernel=mx.BiasGeluStore(acc))
+        check_float_parity(host_bits(acc), acc_ref, f"accumulators {tile} mode{mode}")
+        # the fused epilogue is the oracle's post-op, bit for bit, on the accumulators the GPU produced
+        assert np.array_equal(host_bits(C), po.pp(host_bits(acc), po.PP_BIAS | po.PP_GELU, po.BF16, bias=bias))
+        check_gelu_parity(host_bits(C), ref, acc_ref + bias[None, :], f"bias_gelu {tile} mode{mode}")
     finally:
         mx.set_tile("")
         mx.set_option("load_mode", 0)
@@ -114,12 +120,25 @@ def test_bf16_256_cube(po):
 def test_ffn_up_bias_gelu_full_size(po, M):
     """The headline FC at its real shape: K=4096, N=11008, BIAS_GELU -> bf16."""
     w = wl.ffn_up_bias_gelu(M=M)
-    ref = po.pp(po.gemm_bf16(w["A"], w["B"]), po.PP_BIAS | po.PP_GELU, po.BF16, bias=w["bias"])
+    acc_ref = po.gemm_bf16(w["A"], w["B"])
+    ref = po.pp(acc_ref, po.PP_BIAS | po.PP_GELU, po.BF16, bias=w["bias"])
     C = torch.zeros((M, w["N"]), dtype=torch.bfloat16, device="cuda")
+    acc = torch.zeros((M, w["N"]), dtype=torch.float32, device="cuda")
     mm = mx.Matmul(True, False)
-    mm(dev_bf16(w["A"]), dev_bf16(w["B"]), ppkernel=mx.BiasGeluStore(C, mx.Steps.BIAS_GELU, dev(w["bias"])))
-    err, frac = check_float_parity(bf16_to_f32(host_bits(C)), bf16_to_f32(ref), f"ffn_up M={M}")
-    print(f"ffn_up M={M}: rel_fro={err:.2e} within_1ulp={frac * 100:.4f}% kernel={mx.last_kernel()}")
+    Ad, Bd = dev_bf16(w["A"]), dev_bf16(w["B"])
+    mm(Ad, Bd, ppkernel=mx.BiasGeluStore(C, mx.Steps.BIAS_GELU, dev(w["bias"])))
+    kernel = mx.last_kernel()
+    mm(Ad, Bd, ppkernel=mx.BiasGeluStore(acc))
+    # 1. fp32 accumulators against the reference's (AMX summation order)
+    e_acc, f_acc = check_float_parity(host_bits(acc), acc_ref, f"ffn_up accumulators M={M}")
+    # 2. the fused epilogue equals the reference post-op applied to the GPU's accumulators, bit for bit
+    assert np.array_equal(host_bits(C), po.pp(host_bits(acc), po.PP_BIAS | po.PP_GELU, po.BF16, bias=w["bias"]))
+    # 3. end to end; over ALL elements the one-ulp fraction is limited to about 99.87 % by the noise of
+    #    the reference's own GELU in its deep negative tail (see gpu_util.GELU_WELL_CONDITIONED_ABOVE)
+    err, frac_good, frac = check_gelu_parity(host_bits(C), ref, acc_ref + w["bias"][None, :], f"ffn_up M={M}",
+                                             frac_all=0.998)
+    print(f"ffn_up M={M}: acc rel_fro={e_acc:.2e} ({f_acc * 100:.4f}% <=1ulp)  out rel_fro={err:.2e} "
+          f"within_1ulp={frac_good * 100:.4f}% (well-conditioned) {frac * 100:.4f}% (all)  kernel={kernel}")
 
 
 def test_column_range_split_equals_whole(po):
@@ -239,23 +258,30 @@ def test_decode_small_shapes(po, shape, w8):
     if w8:
         W = np.clip(np.rint(rng.standard_normal((K, N)) * 40), -127, 127).astype(np.int8)
         scale = rng.uniform(1e-3, 5e-3, N).astype(np.float32)
-        _, acc = po.gemv_w8(x, W, scale, want_acc=True)
-        ref = po.pp(acc, po.PP_DEQUANT | po.PP_BIAS | po.PP_GELU, po.F32, bias=bias, deq_per_oc=scale)
+        _, acc_ref = po.gemv_w8(x, W, scale, want_acc=True)
+        ref = po.pp(acc_ref, po.PP_DEQUANT | po.PP_BIAS | po.PP_GELU, po.F32, bias=bias, deq_per_oc=scale)
         packed = mx.repack_b(dev(W))
         y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
         mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_DEQUANT | mx.PP_BIAS | mx.PP_GELU, bias=dev(bias),
                                                     deq_scale_per_oc=dev(scale)), b_dtype=mx.I8)
     else:
         W = rand_bf16(rng, (K, N), 0.05)
-        ref = po.pp(po.gemm_bf16(x, W), po.PP_BIAS | po.PP_GELU, po.F32, bias=bias)
+        scale = None
+        acc_ref = po.gemm_bf16(x, W)
+        ref = po.pp(acc_ref, po.PP_BIAS | po.PP_GELU, po.F32, bias=bias)
         packed = mx.repack_b(dev_bf16(W))
         y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
         mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_BIAS | mx.PP_GELU, bias=dev(bias)))
     assert "skinny" in mx.last_kernel()
-    # GELU flattens tiny pre-activations: compare on an absolute scale as well as by ulp
+    # raw accumulators through the same kernel, then the oracle's post-op on them must give y's bits
+    acc_gpu = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc_gpu, mx.PP_NONE), b_dtype=mx.I8 if w8 else None)
+    check_float_parity(host_bits(acc_gpu), acc_ref, f"decode accumulators {shape} w8={w8}")
+    steps = (po.PP_DEQUANT if w8 else 0) | po.PP_BIAS | po.PP_GELU
+    again = po.pp(host_bits(acc_gpu), steps, po.F32, bias=bias, deq_per_oc=scale if w8 else None)
+    assert np.array_equal(host_bits(y).view(np.uint32), again.view(np.uint32))
     got = host_bits(y)
     assert np.linalg.norm(got - ref) <= 1e-3 * np.linalg.norm(ref)
-    assert np.mean(np.abs(got - ref) <= np.maximum(2.0 ** -8 * np.abs(ref), 1e-6)) >= 0.999
 
 
 @pytest.mark.parametrize("M", [4, 40])

@@ -109,3 +109,17 @@ def test_splitter_partitions(po):
             assert a[1] == b[0]
         sizes = [b - a for a, b in parts]
         assert max(sizes) - min(sizes) <= 1
+
+
+def test_gelu_deep_negative_tail_is_ill_conditioned(po):
+    """Why two implementations of the FC + GELU cannot agree to one bf16 ulp everywhere unless their
+    fp32 accumulators are bit-identical: below about -3.5 the reference polynomial's result moves by
+    more than one bf16 ulp when its input moves by ONE fp32 ulp."""
+    def frac_beyond_one_bf16_ulp(lo, hi):
+        x = np.linspace(lo, hi, 200001).astype(np.float32)
+        x1 = np.nextafter(x, np.float32(0))
+        y, y1 = po.gelu(x).astype(np.float64), po.gelu(x1).astype(np.float64)
+        ulp = np.exp2(np.floor(np.log2(np.maximum(np.abs(y), 2.0 ** -126))) - 7)
+        return np.mean(np.abs(y - y1) > ulp)
+    assert frac_beyond_one_bf16_ulp(-4.9, -4.3) > 0.25
+    assert frac_beyond_one_bf16_ulp(-3.0, 5.0) == 0.0
