@@ -12,7 +12,8 @@ F32, BF16, I8, I32 = 0, 1, 2, 3
 PP_NONE, PP_DEQUANT, PP_BIAS, PP_GELU, PP_QUANT, PP_SILU_GATE = 0, 1, 2, 4, 8, 16
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "libmm_amx_amd.so")
+# MMX_LIB_PATH lets a developer point at an alternative build of the same ABI
+_LIB_PATH = os.environ.get("MMX_LIB_PATH") or os.path.join(_HERE, "libmm_amx_amd.so")
 
 EXPORTS = ["mmx_last_error", "mmx_init", "mmx_packed_b_bytes", "mmx_repack_b", "mmx_repack_gate_up",
            "mmx_quantize_weights", "mmx_dequant_packed", "mmx_gemm", "mmx_matvec", "mmx_mlp", "mmx_set_tile",

@@ -48,7 +48,7 @@ struct TileCfg {
     int bm, bn;
 };
 static TileCfg g_forced = {0, 0};
-static int g_load_mode = 0;
+static int g_load_mode = 2;
 TileCfg forced_tile() { return g_forced; }
 int load_mode() { return g_load_mode; }
 

@@ -23,6 +23,8 @@
 //           (K*sizeof(T) not a multiple of 128) and for A rows that are not 16-byte aligned.
 //           Rows past M and elements past K are read as zero, never touched in memory.
 #pragma once
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace mmx {
@@ -105,6 +107,15 @@ __device__ __forceinline__ void lds_dma_wait() {
     if constexpr (MODE == 1) __builtin_amdgcn_s_waitcnt(0);
     if constexpr (MODE == 2) asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
 }
+
+// LDS ring of the hand-scheduled pipeline: R half-stages of (BM + BN) rows x 64 bytes.
+template <int BM, int BN>
+struct Ring {
+    static constexpr int HS = (BM + BN) * 64;  // bytes per half-stage
+    static constexpr int AH = BM * 64;         // A part of a half-stage
+    static constexpr int R = (5 * HS <= 160 * 1024 - 4096) ? 5 : 4;
+    static constexpr int BYTES = R * HS;
+};
 
 template <typename TIn, int BM, int BN, int MODE, typename TOut>
 __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs g) {
@@ -210,17 +221,149 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs g) {
             for (int j = 0; j < NJ; j++) acc[i][j] = MF::run(a[i], b[j], acc[i][j]);
     };
 
+    if constexpr (MODE == 2) {
+        // ---- hand-scheduled ring pipeline -------------------------------------------------------------
+        // One wave per SIMD means nothing hides a stall, and a wave issues in order: a burst of LDS
+        // reads or of global loads in front of the MFMAs leaves the matrix pipe idle while the burst
+        // drains into the LDS / address FIFOs.  So every MFMA is followed by at most one LDS read (for
+        // the next k-step) and one HBM->LDS load, and the order is pinned.
+        //
+        // LDS is a ring of R half-stages (64 bytes of K per row = two k-steps each).  While half-stage
+        // h is multiplied, the loads of half-stages h+1 .. h+R-1 are in flight: (R-1) x 768 MFMA
+        // cycles of prefetch distance, enough to cover an HBM miss.  One workgroup barrier per
+        // half-stage; it waits only for the loads of the NEXT half-stage (s_waitcnt vmcnt(N) with the
+        // younger loads still outstanding).
+        using RG = Ring<BM, BN>;
+        constexpr int R = RG::R, HS = RG::HS, AH = RG::AH;
+        constexpr int A_IT2 = BM / 64, B_IT2 = BN / 64;   // 16-byte chunks per thread per half-stage
+        constexpr int MN = MI * NJ;                       // MFMAs per k-step
+        constexpr int NL = A_IT2 + B_IT2;                 // HBM->LDS loads per thread per half-stage
+        constexpr int H = (NL + 1) / 2;                   // issued in two groups, one load per MFMA slot
+        static_assert(H <= MN && MI + NJ <= MN, "not enough MFMA slots to spread the loads over");
+        static_assert((R - 2) * NL <= 63, "vmcnt is a 6-bit counter");
+
+        // 64-byte rows: the 16-byte chunk c of row r sits at slot c ^ f(r), f chosen so that the 32 rows
+        // an MFMA operand touches spread over all banks whether 8 or 16 lanes are served per cycle
+        const auto swz = [](int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); };
+
+        uint32_t aoff[A_IT2], boff[B_IT2];
+#pragma unroll
+        for (int it = 0; it < A_IT2; it++) {
+            const int c = it * 256 + tid;
+            const int row = c >> 2, slot = c & 3;
+            int grow = m0 + row;
+            grow = grow < g.M ? grow : g.M - 1;
+            aoff[it] = (uint32_t)grow * (uint32_t)g.lda + (uint32_t)((slot ^ swz(row)) * 16);
+        }
+#pragma unroll
+        for (int it = 0; it < B_IT2; it++) {
+            const int c = it * 256 + tid;
+            int panel = panel0 + (c >> 7);  // 128 chunks = one panel's two fragments of this half-stage
+            panel = panel < g.npanels ? panel : g.npanels - 1;
+            boff[it] = (uint32_t)(panel - panel0) * (uint32_t)g.panel_stride + (uint32_t)((c & 127) * 16);
+        }
+        const char* const b_base = g.Bp + (int64_t)panel0 * g.panel_stride;
+        const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)(smem + wave * 1024));
+        const int last_hs = 2 * g.nk - 1;
+
+        // load number q of half-stage hs into ring slot `buf` (B chunks first, then A chunks)
+        auto dma = [&](int q, int hs, int buf) {
+            hs = hs < last_hs ? hs : last_hs;  // past the end: re-fetch the last one into a free slot
+            uint32_t m0v, off;
+            const char* base;
+            if (q < B_IT2) {
+                m0v = lds_wave + buf * HS + AH + q * 4096;
+                off = boff[q];
+                base = b_base + (int64_t)hs * 2048;
+            } else {
+                m0v = lds_wave + buf * HS + (q - B_IT2) * 4096;
+                off = aoff[q - B_IT2];
+                base = g.A + (int64_t)hs * 64;
+            }
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                         :
+                         : "s"(m0v), "v"(off), "s"(base)
+                         : "memory");
+        };
+        const int a_row_off = (wm * WM + l32) * 64;
+        const int a_swz = swz(l32);
+        const int b_frag_off = AH + wn * NJ * 2 * 1024 + lane * 16;
+
+        // one k-step: MFMAs on (ca, cb); meanwhile fill (na, nb) with k-step RS of ring slot rbuf and
+        // issue loads [Q0, Q1) of half-stage fhs into ring slot fbuf
+        auto kstep = [&](const frag (&ca)[MI], const frag (&cb)[NJ], frag (&na)[MI], frag (&nb)[NJ], int rbuf,
+                         auto rs_c, auto q0_c, auto q1_c, int fhs, int fbuf) {
+            constexpr int RS = decltype(rs_c)::value, Q0 = decltype(q0_c)::value, Q1 = decltype(q1_c)::value;
+            const char* sA = smem + rbuf * HS + a_row_off + (((2 * RS + g32) ^ a_swz) * 16);
+            const char* sB = smem + rbuf * HS + b_frag_off + RS * 1024;
+#pragma unroll
+            for (int t = 0; t < MN; t++) {
+                acc[t / NJ][t % NJ] = MF::run(ca[t / NJ], cb[t % NJ], acc[t / NJ][t % NJ]);
+                if (t < NJ) nb[t] = *reinterpret_cast<const frag*>(sB + t * 2 * 1024);
+                else if (t < NJ + MI) na[t - NJ] = *reinterpret_cast<const frag*>(sA + (t - NJ) * 32 * 64);
+                if (Q0 + t < Q1) dma(Q0 + t, fhs, fbuf);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        using std::integral_constant;
+        typedef integral_constant<int, 0> c0;
+        typedef integral_constant<int, 1> c1;
+        typedef integral_constant<int, H> cH;
+        typedef integral_constant<int, NL> cNL;
+
+        // prologue: half-stages 0 .. R-2 completely, and the first group of half-stage R-1
+#pragma unroll
+        for (int hs = 0; hs < R - 1; hs++)
+#pragma unroll
+            for (int q = 0; q < NL; q++) dma(q, hs, hs);
+#pragma unroll
+        for (int q = 0; q < H; q++) dma(q, R - 1, R - 1);
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"((R - 2) * NL + H) : "memory");  // half-stage 0 has landed
+        __syncthreads();
+        {
+            const char* sA = smem + a_row_off + ((g32 ^ a_swz) * 16);
+            const char* sB = smem + b_frag_off;
+#pragma unroll
+            for (int i = 0; i < MI; i++) fa[0][i] = *reinterpret_cast<const frag*>(sA + i * 32 * 64);
+#pragma unroll
+            for (int j = 0; j < NJ; j++) fb[0][j] = *reinterpret_cast<const frag*>(sB + j * 2 * 1024);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        int buf = 0;  // ring slot of the half-stage being multiplied
+        for (int hs = 0; hs <= last_hs; hs++) {
+            const int nbuf = buf + 1 < R ? buf + 1 : 0;           // slot of half-stage hs+1
+            const int pbuf = buf == 0 ? R - 1 : buf - 1;          // slot of hs-1 == slot of hs+R-1
+            // k-step 0: read k-step 1 of this half-stage; second group of the loads of half-stage hs+R-1
+            kstep(fa[0], fb[0], fa[1], fb[1], buf, c1{}, cH{}, cNL{}, hs + R - 1, pbuf);
+            // every wave now holds all of half-stage hs in registers; half-stage hs+1 must have landed,
+            // the (R-2) younger ones may still be in flight
+            asm volatile("s_waitcnt vmcnt(%0)" : : "n"((R - 2) * NL) : "memory");
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+            // k-step 1: read k-step 0 of the next half-stage; first group of the loads of half-stage
+            // hs+R goes into the slot this half-stage has just vacated
+            kstep(fa[1], fb[1], fa[0], fb[0], nbuf, c0{}, c0{}, cH{}, hs + R, buf);
+            buf = nbuf;
+        }
+        asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+        __syncthreads();
+    } else {
     fetch(0, 0);
     commit(0);
     lds_dma_wait<MODE>();
     __syncthreads();
     read_frags(0, 0, fa[0], fb[0]);
 
-    // Scheduling groups: within each region issue the LDS reads of the next k-step first, then
-    // the MFMAs of the current one (mask 0x100 = DS read, 0x008 = MFMA).
-#define MMX_READS_THEN_MFMA()                                          \
-    __builtin_amdgcn_sched_group_barrier(0x100, MI + NJ, 0);           \
-    __builtin_amdgcn_sched_group_barrier(0x008, MI * NJ, 0);           \
+    // Scheduling groups: alternate one MFMA of the current k-step with one LDS read of the next
+    // (mask 0x008 = MFMA, 0x100 = DS read), then the remaining MFMAs.
+#define MMX_INTERLEAVE()                                                   \
+    for (int r_ = 0; r_ < MI + NJ; r_++) {                                 \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 \
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                 \
+    }                                                                      \
+    __builtin_amdgcn_sched_group_barrier(0x008, MI * NJ - (MI + NJ), 0);   \
     __builtin_amdgcn_sched_barrier(0)
 
     for (int kt = 0; kt < g.nk; kt++) {
@@ -232,13 +375,13 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs g) {
         __builtin_amdgcn_sched_barrier(0);
         read_frags(stage, 1, fa[1], fb[1]);
         mma(fa[0], fb[0]);
-        MMX_READS_THEN_MFMA();
+        MMX_INTERLEAVE();
         read_frags(stage, 2, fa[0], fb[0]);
         mma(fa[1], fb[1]);
-        MMX_READS_THEN_MFMA();
+        MMX_INTERLEAVE();
         read_frags(stage, 3, fa[1], fb[1]);
         mma(fa[0], fb[0]);
-        MMX_READS_THEN_MFMA();
+        MMX_INTERLEAVE();
         // Everything this wave reads from the current stage is now in registers, and the next
         // stage has had three k-steps to land: synchronise here, then start reading the next
         // stage while the last k-step of this one is multiplied.
@@ -248,10 +391,11 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs g) {
         __builtin_amdgcn_sched_barrier(0);
         read_frags(stage ^ 1, 0, fa[0], fb[0]);
         mma(fa[1], fb[1]);
-        MMX_READS_THEN_MFMA();
+        MMX_INTERLEAVE();
     }
-#undef MMX_READS_THEN_MFMA
+#undef MMX_INTERLEAVE
     __syncthreads();
+    }
 
     // ---- epilogue: registers -> post-op -> LDS (per-wave staging band) -> row-contiguous stores
     const Epilogue& ep = g.ep;
@@ -372,7 +516,7 @@ static inline TileCfg choose_tile(int M, int Ncols, bool need_pairs) {
 
 template <typename TIn, int BM, int BN, int MODE, typename TOut>
 static int launch_cfg(const GemmArgs& g, int grid, hipStream_t st, const char* name) {
-    constexpr int lds = 2 * (BM + BN) * 128;
+    constexpr int lds = MODE == 2 ? Ring<BM, BN>::BYTES : 2 * (BM + BN) * 128;
     auto kern = gemm_kernel<TIn, BM, BN, MODE, TOut>;
     static bool attr_done = false;  // one flag per instantiation
     if (!attr_done) {
@@ -422,6 +566,8 @@ static inline int prepare_gemm(GemmArgs& g, TileCfg& t, int& mode, int elesz, co
     // the unmasked loads need aligned rows and a K that fills whole k-iterations
     const bool fast_ok = g.a_vec_ok && (g.kbytes % 128 == 0);
     mode = fast_ok ? load_mode() : 3;
+    // mode 2 addresses A through 32-bit per-thread offsets
+    if (mode == 2 && ((int64_t)M * lda >= ((int64_t)1 << 32) - 4096 || g.panel_stride >= ((int64_t)1 << 28))) mode = 0;
     t = choose_tile(M, n1 - n0, pairs);
     if (mode == 3) t = {128, 128};
     if (pairs && (t.bn % 128) != 0)
