@@ -494,21 +494,23 @@ struct TileCfg {
 TileCfg forced_tile();
 int load_mode();
 
-// Pick the tile that minimises (rounds over the CUs) x (work per tile) / (per-tile efficiency).
+// Pick the tile that minimises (tiles per CU, rounded up) x (work per tile) / (per-tile efficiency).
+// Workgroups that share a CU share its matrix pipe, so what counts is how many tiles the busiest CU
+// has to finish.  The efficiency factors are measured on the 1024 x 4096 x 11008 FC: larger tiles
+// re-use each LDS fragment for more MFMAs and load fewer bytes per flop.
 static inline TileCfg choose_tile(int M, int Ncols, bool need_pairs) {
     const TileCfg f = forced_tile();
     if (f.bm) return f;
-    static const struct { int bm, bn; float eff; int per_cu; } cand[] = {
-        {256, 256, 1.00f, 1}, {256, 192, 0.97f, 1}, {128, 256, 0.90f, 1}, {128, 128, 0.80f, 2}};
+    static const struct { int bm, bn; float eff; } cand[] = {
+        {256, 256, 1.00f}, {256, 192, 0.97f}, {128, 256, 0.90f}, {128, 128, 0.80f}};
     const int cus = num_cus();
     float best = 1e30f;
     TileCfg pick = {128, 128};
     for (const auto& c : cand) {
         if (need_pairs && (c.bn % 128) != 0) continue;
         const int tiles = ((M + c.bm - 1) / c.bm) * ((Ncols + c.bn - 1) / c.bn);
-        const int slots = cus * c.per_cu;
-        const int rounds = (tiles + slots - 1) / slots;
-        const float t = (float)rounds * c.per_cu * (float)(c.bm * c.bn) / c.eff;
+        const int per_cu = (tiles + cus - 1) / cus;
+        const float t = (float)per_cu * (float)(c.bm * c.bn) / c.eff;
         if (t < best) { best = t; pick = {c.bm, c.bn}; }
     }
     return pick;

@@ -58,6 +58,44 @@ __device__ __forceinline__ void store_out(const Epilogue& ep, int m, int n, floa
     }
 }
 
+// cross-wave reduction of the partial 32x32 blocks + post-op + store (shared by both decode kernels)
+template <int NP>
+__device__ __forceinline__ void skinny_finish(const SkinnyArgs& s, const float (&red)[8][NP][16][64], int panel_first, int tid) {
+    const Epilogue& ep = s.ep;
+    for (int idx = tid; idx < 16 * 64; idx += 512) {
+        const int v = idx >> 6, ln = idx & 63;
+        const int m = ln & 31;
+        if (m >= s.M) continue;
+        const int nloc = 8 * (v >> 2) + 4 * (ln >> 5) + (v & 3);
+        float sum[NP];
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            float t = 0.0f;
+#pragma unroll
+            for (int w8 = 0; w8 < 8; w8++) t += red[w8][p][v][ln];
+            sum[p] = t;
+        }
+        if (ep.steps & MMX_PP_SILU_GATE) {
+            if constexpr (NP == 2) {
+                const int n = ((panel_first >> 1) << 5) + nloc;  // output column (half width)
+                if (n < (s.n1 >> 1)) store_out(ep, m, n, silu(sum[0]) * sum[1]);
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                const int n = ((panel_first + p) << 5) + nloc;
+                if (n >= s.n1) continue;
+                float r = sum[p];
+                if (ep.steps & MMX_PP_DEQUANT) r = r * (ep.deq_oc ? ep.deq_oc[n] : ep.deq);
+                if (ep.steps & MMX_PP_BIAS) r = r + ep.bias[n];
+                if (ep.steps & MMX_PP_GELU) r = gelu_erf_minimax(r);
+                if (ep.steps & MMX_PP_QUANT) r = r * (ep.q_oc ? ep.q_oc[n] : ep.q);
+                store_out(ep, m, n, r);
+            }
+        }
+    }
+}
+
 template <bool W8, int NP>
 __global__ __launch_bounds__(512) void skinny_kernel(const SkinnyArgs s) {
     constexpr int U = 4;  // fragments in flight per wave
@@ -122,39 +160,115 @@ __global__ __launch_bounds__(512) void skinny_kernel(const SkinnyArgs s) {
         for (int v = 0; v < 16; v++) red[wave][p][v][lane] = acc[p][v];
     __syncthreads();
 
-    const Epilogue& ep = s.ep;
-    for (int idx = tid; idx < 16 * 64; idx += 512) {
-        const int v = idx >> 6, ln = idx & 63;
-        const int m = ln & 31;
-        if (m >= s.M) continue;
-        const int nloc = 8 * (v >> 2) + 4 * (ln >> 5) + (v & 3);
-        float sum[NP];
+    skinny_finish<NP>(s, red, panel_first, tid);
+}
+
+// ---- streaming variant for the smallest M -----------------------------------------------------------
+// When the activations fit in LDS (M * K_pad * 2 <= 32 KiB) the kernel is organised around one goal:
+// have every byte of the weights requested from HBM as early as possible.  Each wave first issues the
+// load of its slice of x, then 16 KiB of weight loads, and only then waits for x, publishes it to LDS
+// and starts consuming the weights in arrival order.  x fragments are re-read from LDS (a separate counter from the HBM loads, so they never
+// queue behind the weight stream).
+// 128 VGPRs at most: two workgroups per CU, so that every panel of a 11008-column matrix is resident at once
+template <bool W8, int NP>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void skinny_stream_kernel(const SkinnyArgs s, int kpad) {
+    constexpr int U = 16 / NP;  // fragments per wave in flight at once (16 KiB of weights)
+    __shared__ float red[8][NP][16][64];
+    extern __shared__ __attribute__((aligned(16))) char xs[];  // [M + 1][kpad] bf16, last row all zero
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: keeps the control flow below uniform
+    const int l32 = lane & 31, g32 = lane >> 5;
+    const int panel_first = (s.n0 >> 5) + blockIdx.x * NP;
+    const int panel_end = (s.n1 + 31) >> 5;
+
+    // x: 16 bytes per thread per pass, zero padded to kpad (plus the zero row); issued before any weight load
+    const int chunks_per_row = kpad >> 3;
+    const int real_chunks = s.M * chunks_per_row;
+    const int total_chunks = real_chunks + chunks_per_row;
+    constexpr int XP = 5;  // passes of 512 threads: up to 40 KiB
+    bf16x8 xreg[XP];
 #pragma unroll
-        for (int p = 0; p < NP; p++) {
-            float t = 0.0f;
+    for (int p = 0; p < XP; p++) {
+        const int c = p * 512 + tid;
+        const int m = c / chunks_per_row, k0 = (c - m * chunks_per_row) * 8;
+        // the launcher guarantees 16-byte aligned rows and K % 8 == 0: a chunk is all data or all padding
+        const bool has = c < real_chunks && k0 < s.K;
+        const bf16x8 v = *reinterpret_cast<const bf16x8*>(s.x + (int64_t)(has ? m : 0) * s.ldx + (int64_t)(has ? k0 : 0) * 2);
 #pragma unroll
-            for (int w8 = 0; w8 < 8; w8++) t += red[w8][p][v][ln];
-            sum[p] = t;
+        for (int e = 0; e < 8; e++) xreg[p][e] = has ? v[e] : (__bf16)0.0f;
+    }
+
+    f32x16 acc[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[p][v] = 0.0f;
+
+    // wave w multiplies fragments [w*per_wave, (w+1)*per_wave); indices past the end are clamped for the
+    // load and paired with the zero row of x, so the code below has no per-fragment branches
+    const int per_wave = (s.nfrag + 7) / 8;
+    const int f_begin = wave * per_wave;
+    const int f_last = s.nfrag - 1;
+    const char* wbase[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++) {
+        int panel = panel_first + p;
+        panel = (panel < panel_end && panel < s.npanels) ? panel : s.npanels - 1;  // columns past n1 are never stored
+        wbase[p] = s.Wp + (int64_t)panel * s.panel_stride + lane * 16;
+    }
+    const char* xrow = xs + (l32 < s.M ? l32 : s.M) * kpad * 2;
+    const char* zrow = xs + s.M * kpad * 2;
+    const int nbatch = (per_wave + U - 1) / U;  // same for every wave
+    for (int b = 0; b < nbatch; b++) {
+        const int f0 = f_begin + b * U;
+        // the whole batch is requested before anything else happens
+        u32x4 w[NP][U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            int f = f0 + u;
+            f = f < f_last ? f : f_last;
+#pragma unroll
+            for (int p = 0; p < NP; p++) w[p][u] = *reinterpret_cast<const u32x4*>(wbase[p] + (int64_t)f * 1024);
         }
-        if (ep.steps & MMX_PP_SILU_GATE) {
-            if constexpr (NP == 2) {
-                const int n = ((panel_first >> 1) << 5) + nloc;  // output column (half width)
-                if (n < (s.n1 >> 1)) store_out(ep, m, n, silu(sum[0]) * sum[1]);
-            }
-        } else {
+        if (b == 0) {
+            // x was requested first and loads return in order: publish it while the weights are in flight
 #pragma unroll
-            for (int p = 0; p < NP; p++) {
-                const int n = ((panel_first + p) << 5) + nloc;
-                if (n >= s.n1) continue;
-                float r = sum[p];
-                if (ep.steps & MMX_PP_DEQUANT) r = r * (ep.deq_oc ? ep.deq_oc[n] : ep.deq);
-                if (ep.steps & MMX_PP_BIAS) r = r + ep.bias[n];
-                if (ep.steps & MMX_PP_GELU) r = gelu_erf_minimax(r);
-                if (ep.steps & MMX_PP_QUANT) r = r * (ep.q_oc ? ep.q_oc[n] : ep.q);
-                store_out(ep, m, n, r);
+            for (int p = 0; p < XP; p++) {
+                const int c = p * 512 + tid;
+                if (c < total_chunks) *reinterpret_cast<bf16x8*>(xs + c * 16) = xreg[p];
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory");
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int f = f0 + u;
+            const bool valid = (f - f_begin) < per_wave && f <= f_last;  // scalar
+            const int fc = f < f_last ? f : f_last;
+            const char* xr = valid ? xrow : zrow;
+            if constexpr (W8) {
+                const bf16x8 xa = *reinterpret_cast<const bf16x8*>(xr + (32 * fc + 16 * g32) * 2);
+                const bf16x8 xb = *reinterpret_cast<const bf16x8*>(xr + (32 * fc + 16 * g32 + 8) * 2);
+#pragma unroll
+                for (int p = 0; p < NP; p++) {
+                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(w[p][u].x, w[p][u].y), xa, acc[p], 0, 0, 0);
+                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(w[p][u].z, w[p][u].w), xb, acc[p], 0, 0, 0);
+                }
+            } else {
+                const bf16x8 xa = *reinterpret_cast<const bf16x8*>(xr + (16 * fc + 8 * g32) * 2);
+#pragma unroll
+                for (int p = 0; p < NP; p++)
+                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w[p][u]), xa, acc[p], 0, 0, 0);
             }
         }
     }
+
+#pragma unroll
+    for (int p = 0; p < NP; p++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) red[wave][p][v][lane] = acc[p][v];
+    __syncthreads();
+    skinny_finish<NP>(s, red, panel_first, tid);
 }
 
 int launch_skinny(bool w8, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
@@ -175,6 +289,21 @@ int launch_skinny(bool w8, const void* x, int64_t ldx, const void* Wp, int M, in
     s.ep = ep;
     const int panels = ((n1 + 31) >> 5) - (n0 >> 5);
     const bool pairs = (ep.steps & MMX_PP_SILU_GATE) != 0;
+    const int kpad = kbytes_pad / (w8 ? 1 : 2);  // elements of K the packed weights cover
+    const int xbytes = (M + 1) * kpad * 2;  // x plus one zero row
+    if (xbytes <= 40960 && s.x_vec_ok && (K % 8) == 0) {
+        // the activations fit in LDS: streaming variant
+        if (pairs && (panels & 1)) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
+        note_kernel(pairs ? (w8 ? "skinny_stream_w8_gateup" : "skinny_stream_bf16_gateup") : (w8 ? "skinny_stream_w8" : "skinny_stream_bf16"));
+        if (pairs) {
+            if (w8) hipLaunchKernelGGL((skinny_stream_kernel<true, 2>), dim3(panels / 2), dim3(512), xbytes, st, s, kpad);
+            else hipLaunchKernelGGL((skinny_stream_kernel<false, 2>), dim3(panels / 2), dim3(512), xbytes, st, s, kpad);
+        } else {
+            if (w8) hipLaunchKernelGGL((skinny_stream_kernel<true, 1>), dim3(panels), dim3(512), xbytes, st, s, kpad);
+            else hipLaunchKernelGGL((skinny_stream_kernel<false, 1>), dim3(panels), dim3(512), xbytes, st, s, kpad);
+        }
+        return check_hip(hipGetLastError(), "skinny_stream_kernel launch");
+    }
     if (pairs) {
         if (panels & 1) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
         note_kernel(w8 ? "skinny_w8_gateup" : "skinny_bf16_gateup");
