@@ -26,6 +26,13 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_INT8_TOPS = 5000.0     # MI355X dense int8 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
+# HBM-side bytes per launch of the headline kernel, from two counter runs of this script under
+# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (KiB per dispatch: 81930 and 22020), each scaled by
+# what the same counter reads for the 256 MiB device copy of --calibrate-copy (factors 2.000 and 1.000);
+# the summary is profiles/gemm_bf16_256x192_ffn_up_M1024_hbm_traffic.txt.  Counters cannot be read from
+# inside the process, so the figure is only reported when the kernel that ran is the one profiled.
+MEASURED_TRAFFIC_BYTES = {"gemm_bf16_256x192_ring_out_bf16": (81930 * 2.000 + 22020 * 1.000) * 1024}
+
 
 def main():
     ap = argparse.ArgumentParser()
@@ -34,6 +41,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a 256 MiB device-to-device copy: a kernel of known traffic to scale profiler byte counters by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the path shards over N by column panels; see DESIGN.md); "
@@ -93,9 +102,21 @@ def main():
         "config": {"workload": "llama7b_ffn_up_bf16_bias_gelu", "M": M, "K": K, "N": N, "kernel": kernel_name,
                    "inputs": "A~N(0,1) bf16, B~N(0,0.02) bf16 repacked once, bias~N(0,0.1) fp32, all resident in HBM"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(kernel_name),
+                     "algorithmic_flop_per_launch": flops,
+                     "algorithmic_bytes_per_launch": 2 * M * K + 2 * K * N + 4 * N + 2 * M * N,
                      "kernel_avg_us": round(kernel_ms * 1e3, 2)},
     }
+
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        out["calibration_copy_bytes"] = {"read": 256 << 20, "written": 256 << 20}
+        del src, dst
 
     # ---- CPU baseline: the oracle (a port of the reference path) on this host's cores --------------
     if not args.no_cpu:
@@ -113,7 +134,7 @@ def main():
             po.pp(acc, po.PP_BIAS | po.PP_GELU, po.BF16, bias=w["bias"])
             reps += 1
             el = time.perf_counter() - t0
-            if el > 10.0 or reps >= 20:
+            if el > 10.0:
                 break
         out["cpu_baseline"] = {
             "value": round(flops * reps / el / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",

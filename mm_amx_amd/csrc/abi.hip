@@ -250,7 +250,7 @@ int mmx_time_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, co
     int rc = check_hip(hipEventCreate(&e0), "hipEventCreate");
     if (rc) return rc;
     rc = check_hip(hipEventCreate(&e1), "hipEventCreate");
-    if (rc) { hipEventDestroy(e0); return rc; }
+    if (rc) { (void)hipEventDestroy(e0); return rc; }
     rc = check_hip(hipEventRecord(e0, st), "hipEventRecord");
     for (int i = 0; i < iters && !rc; i++)
         rc = gemm_dispatch(a_dtype, b_dtype, A, lda_bytes, Bpacked_rot[i % n_rot], M, K, N, n0, n1, ep, st);
@@ -258,8 +258,8 @@ int mmx_time_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, co
     if (!rc) rc = check_hip(hipEventSynchronize(e1), "hipEventSynchronize");
     float ms = 0.0f;
     if (!rc) rc = check_hip(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime");
-    hipEventDestroy(e0);
-    hipEventDestroy(e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
     if (!rc) *ms_out = ms / iters;
     return rc;
 }

@@ -516,11 +516,23 @@ static inline TileCfg choose_tile(int M, int Ncols, bool need_pairs) {
     return pick;
 }
 
+template <typename T> constexpr const char* type_tag();
+template <> constexpr const char* type_tag<__bf16>() { return "bf16"; }
+template <> constexpr const char* type_tag<uint16_t>() { return "bf16"; }
+template <> constexpr const char* type_tag<int8_t>() { return "i8"; }
+template <> constexpr const char* type_tag<int32_t>() { return "i32"; }
+template <> constexpr const char* type_tag<float>() { return "f32"; }
+
 template <typename TIn, int BM, int BN, int MODE, typename TOut>
-static int launch_cfg(const GemmArgs& g, int grid, hipStream_t st, const char* name) {
+static int launch_cfg(const GemmArgs& g, int grid, hipStream_t st) {
     constexpr int lds = MODE == 2 ? Ring<BM, BN>::BYTES : 2 * (BM + BN) * 128;
     auto kern = gemm_kernel<TIn, BM, BN, MODE, TOut>;
-    static bool attr_done = false;  // one flag per instantiation
+    static bool attr_done = false;  // one flag and one name per instantiation
+    static char name[64];
+    if (!name[0]) {
+        static const char* const loads[] = {"regs", "dma", "ring", "masked"};
+        snprintf(name, sizeof name, "gemm_%s_%dx%d_%s_out_%s", type_tag<TIn>(), BM, BN, loads[MODE], type_tag<TOut>());
+    }
     if (!attr_done) {
         int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds),
@@ -534,7 +546,7 @@ static int launch_cfg(const GemmArgs& g, int grid, hipStream_t st, const char* n
 }
 
 #define MMX_LAUNCH(TIn, BM, BN, MODE, TOut) \
-    launch_cfg<TIn, BM, BN, MODE, TOut>(g, grid, st, "gemm_" #TIn "_" #BM "x" #BN "_mode" #MODE "_" #TOut)
+    launch_cfg<TIn, BM, BN, MODE, TOut>(g, grid, st)
 #define MMX_LAUNCH_MODES(TIn, BM, BN, TOut)                                  \
     (mode == 2 ? MMX_LAUNCH(TIn, BM, BN, 2, TOut)                            \
                : mode == 1 ? MMX_LAUNCH(TIn, BM, BN, 1, TOut) : MMX_LAUNCH(TIn, BM, BN, 0, TOut))
