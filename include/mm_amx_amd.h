@@ -136,8 +136,9 @@ int mmx_set_tile(const char* shape);
 /* Name of the kernel variant the last mmx_gemm call of this thread launched. */
 const char* mmx_last_kernel(void);
 /* Sets a kernel option.  "load_mode": how the MFMA tile kernel brings A and B tiles into LDS —
- * 0 through registers (default; always used when M/K tails or alignment need masking),
- * 1 global_load_lds through the compiler builtin, 2 global_load_lds issued from inline asm. */
+ * 0 through registers, 1 direct HBM->LDS loads through the compiler builtin, 2 (default) direct
+ * HBM->LDS loads in a hand-scheduled ring pipeline.  Shapes whose M/K tails or alignment need
+ * masked loads use a masked kernel whatever this is set to. */
 int mmx_set_option(const char* name, int value);
 /* HIP-event timing of `iters` back-to-back launches of the given gemm on `stream`, launch i
  * using the packed weights Bpacked_rot[i % n_rot] (rotate over several copies so that a
