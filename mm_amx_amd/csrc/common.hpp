@@ -73,6 +73,53 @@ __device__ __forceinline__ float gelu_erf_minimax(float x) {
     return p;
 }
 
+// The same function on the 16 accumulators a lane holds of one 32x32 block.  A wavefront that is
+// alone on its SIMD cannot issue a dependent vector instruction back to back, so the 16 Horner
+// chains advance in lockstep, one coefficient at a time.  The three selects only matter outside
+// 2^-24 < |x| <= 5; they are skipped when no element of any lane of the wavefront is out there
+// (v_max/v_min drop a NaN operand: a NaN then comes out of the polynomial as NaN, as it would
+// out of the select).  Same result bit for bit.
+__device__ __forceinline__ void gelu_erf_minimax_x16(float (&r)[16]) {
+    constexpr uint32_t coef[14] = {0xa3198977u, 0x268a7927u, 0xa998c963u, 0x2c67ddb2u, 0xaf013b2cu, 0x315d4a4fu, 0xb3969b11u,
+                                   0x35a776e9u, 0xb79b0914u, 0x3970b255u, 0xbb1b7399u, 0x3ca3621fu, 0xbe082bc7u, 0x3f4c4228u};
+    float x2[16], p[16];
+#pragma unroll
+    for (int v = 0; v < 16; v++) x2[v] = r[v] * r[v];
+#pragma unroll
+    for (int v = 0; v < 16; v++) p[v] = __builtin_fmaf(u2f(0x1f1c83fdu), x2[v], u2f(coef[0]));
+#pragma unroll
+    for (int c = 1; c < 14; c++) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) p[v] = __builtin_fmaf(p[v], x2[v], u2f(coef[c]));
+    }
+#pragma unroll
+    for (int v = 0; v < 16; v++) p[v] = __builtin_fmaf(p[v], r[v], 1.0f);
+#pragma unroll
+    for (int v = 0; v < 16; v++) p[v] = p[v] * (r[v] * 0.5f);
+    float amax = __builtin_fabsf(r[0]), amin = amax;
+#pragma unroll
+    for (int v = 1; v < 16; v++) {
+        amax = __builtin_fmaxf(amax, __builtin_fabsf(r[v]));
+        amin = __builtin_fminf(amin, __builtin_fabsf(r[v]));
+    }
+    const bool needs_select = !(amax <= 5.0f) || !(amin > u2f(0x33800000u));
+    if (__builtin_amdgcn_ballot_w64(needs_select) != 0) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            float x = r[v];
+            // opaque to the optimiser, so that the selects stay inside this rarely taken branch: as
+            // straight-line code they would cost every block 9 more instructions per element
+            asm volatile("" : "+v"(x));
+            const float x_pos = __builtin_fabsf(x);
+            if (x < -5.0f) x = 0.0f;
+            if (!(x_pos <= 5.0f)) p[v] = x;
+            if (x_pos <= u2f(0x33800000u)) p[v] = r[v] * 0.5f;
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < 16; v++) r[v] = p[v];
+}
+
 // tests/amx-mlp.cpp:383-448 — exp_ps_avx512, operation for operation.
 __device__ __forceinline__ float exp_poly(float x) {
     const float ln_flt_min = u2f(0xc2aeac50u), ln_flt_max = u2f(0x42b17218u);

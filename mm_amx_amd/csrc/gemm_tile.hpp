@@ -29,6 +29,27 @@
 
 namespace mmx {
 
+// compile-time loop: f(integral_constant<int, B>) ... f(integral_constant<int, E-1>); unlike
+// "#pragma unroll" it cannot be refused by the unroller's size limit (the accumulator array must
+// only ever be indexed by constants, or it would be placed in scratch memory)
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
+
+// Reads one accumulator register at the point of use.  Left to the compiler, the AGPR -> VGPR copies
+// of all accumulators are placed right behind the main loop, which overflows the vector registers
+// and makes the epilogue shuffle values in and out of AGPRs.
+template <typename T>
+__device__ __forceinline__ T acc_read(T a) {
+    T r;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(r) : "a"(a));
+    return r;
+}
+
 template <typename TIn>
 struct Mfma;
 template <>
@@ -118,7 +139,7 @@ struct Ring {
 };
 
 template <typename TIn, int BM, int BN, int MODE, typename TOut>
-__global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs g) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_kernel(const GemmArgs g) {
     using MF = Mfma<TIn>;
     using frag = typename MF::frag;
     using accv = typename MF::accv;
@@ -218,7 +239,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs g) {
 #pragma unroll
         for (int i = 0; i < MI; i++)
 #pragma unroll
-            for (int j = 0; j < NJ; j++) acc[i][j] = MF::run(a[i], b[j], acc[i][j]);
+            for (int j = 0; j < NJ; j++) acc[i][j] = MF::run(b[j], a[i], acc[i][j]);
     };
 
     if constexpr (MODE == 2) {
@@ -299,7 +320,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs g) {
             const char* sB = smem + rbuf * HS + b_frag_off + RS * 1024;
 #pragma unroll
             for (int t = 0; t < MN; t++) {
-                acc[t / NJ][t % NJ] = MF::run(ca[t / NJ], cb[t % NJ], acc[t / NJ][t % NJ]);
+                acc[t / NJ][t % NJ] = MF::run(cb[t % NJ], ca[t / NJ], acc[t / NJ][t % NJ]);
                 if (t < NJ) nb[t] = *reinterpret_cast<const frag*>(sB + t * 2 * 1024);
                 else if (t < NJ + MI) na[t - NJ] = *reinterpret_cast<const frag*>(sA + (t - NJ) * 32 * 64);
                 if (Q0 + t < Q1) dma(Q0 + t, fhs, fbuf);
@@ -347,8 +368,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs g) {
             kstep(fa[1], fb[1], fa[0], fb[0], nbuf, c0{}, c0{}, cH{}, hs + R, buf);
             buf = nbuf;
         }
-        asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
-        __syncthreads();
+        asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // the re-fetched slots past the end must land before the wave ends
     } else {
     fetch(0, 0);
     commit(0);
@@ -394,95 +414,146 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs g) {
         MMX_INTERLEAVE();
     }
 #undef MMX_INTERLEAVE
-    __syncthreads();
     }
 
-    // ---- epilogue: registers -> post-op -> LDS (per-wave staging band) -> row-contiguous stores
+    // the explicit accumulator reads below are invisible to the compiler's hazard checks: let the last
+    // MFMAs retire (a 32x32 MFMA needs up to 18 wait states before its result may be read)
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    // ---- epilogue: accumulators -> post-op -> global memory, block by block ---------------------------
+    // The weights are the first MFMA operand, so a lane holds ONE output row of a 32x32 block
+    // (m = lane % 32) and four runs of four consecutive columns (n = 8q + 4(lane / 32) + 0..3, q = 0..3).
+    // The two half-waves swap two of their runs (v_permlane32_swap), after which each lane owns 16
+    // consecutive columns of its row and writes them with 16-byte stores: no LDS, no barrier.
     const Epilogue& ep = g.ep;
     const bool silu_gate = (ep.steps & MMX_PP_SILU_GATE) != 0;
-    constexpr int SZ = sizeof(TOut);
-    constexpr int SROW = WN * SZ + 16;  // staging row stride, padded
-    char* stg = smem + wave * (32 * SROW);
     const int out_n1 = silu_gate ? (g.n1 >> 1) : g.n1;
-    const int out_col_base = silu_gate ? ((ntile0 + wn * WN) >> 1) : (ntile0 + wn * WN);
-    const int wn_out = silu_gate ? WN / 2 : WN;
+    const int wave_col0 = ntile0 + wn * WN;  // first column of this wave, in accumulator columns
 
+    // 16 per-column values of block column bcol for this lane: index v <-> column bcol + 8(v/4) + 4 g32 + v%4
+    auto load_per_oc = [&](const float* p, int bcol, float (&dst)[16]) {
 #pragma unroll
-    for (int i = 0; i < MI; i++) {
-        __syncthreads();
-        if (silu_gate) {
-            if constexpr (NJ % 2 == 0) {
+        for (int q = 0; q < 4; q++) {
+            const int n = bcol + 8 * q + 4 * g32;
+            if (n + 4 <= g.n1 && (reinterpret_cast<uintptr_t>(p) & 15) == 0) {
+                const f32x4 t = *reinterpret_cast<const f32x4*>(p + n);
 #pragma unroll
-                for (int j = 0; j < NJ; j += 2) {
+                for (int e = 0; e < 4; e++) dst[4 * q + e] = t[e];
+            } else {
 #pragma unroll
-                    for (int v = 0; v < 16; v++) {
-                        const float gt = MF::to_f32(acc[i][j][v]);
-                        const float up = MF::to_f32(acc[i][j + 1][v]);
-                        const float r = silu(gt) * up;
-                        const int row = 8 * (v >> 2) + 4 * g32 + (v & 3);
-                        *reinterpret_cast<TOut*>(stg + row * SROW + ((j >> 1) * 32 + l32) * SZ) = cvt_out<TOut>(r);
-                    }
-                }
+                for (int e = 0; e < 4; e++) dst[4 * q + e] = (n + e < g.n1) ? p[n + e] : 0.0f;
             }
+        }
+    };
+    // stores the 16 values r[] (or raw int32 accumulators) of one block: row grow, output columns
+    // ocol + 8(v/4) + 4 g32 + v%4
+    auto store_block = [&](const float (&r)[16], const accv& raw, int grow, int ocol) {
+        constexpr int SZ = sizeof(TOut);
+        constexpr int DW = SZ;  // dwords per run of four elements
+        uint32_t w[4][DW];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            if constexpr (std::is_same<TOut, float>::value) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) w[q][e] = f2u(r[4 * q + e]);
+            } else if constexpr (std::is_same<TOut, int32_t>::value) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) w[q][e] = (uint32_t)raw[4 * q + e];
+            } else if constexpr (std::is_same<TOut, uint16_t>::value) {
+                w[q][0] = (uint32_t)to_bf16(r[4 * q]) | ((uint32_t)to_bf16(r[4 * q + 1]) << 16);
+                w[q][1] = (uint32_t)to_bf16(r[4 * q + 2]) | ((uint32_t)to_bf16(r[4 * q + 3]) << 16);
+            } else {
+                w[q][0] = (uint32_t)(uint8_t)to_s8_sat(r[4 * q]) | ((uint32_t)(uint8_t)to_s8_sat(r[4 * q + 1]) << 8) |
+                          ((uint32_t)(uint8_t)to_s8_sat(r[4 * q + 2]) << 16) |
+                          ((uint32_t)(uint8_t)to_s8_sat(r[4 * q + 3]) << 24);
+            }
+        }
+        // lower half-wave: runs 0,1 of both halves = columns 0..15; upper half-wave: runs 2,3 = 16..31
+        uint32_t o[4 * DW];
+#pragma unroll
+        for (int d = 0; d < DW; d++) {
+            const auto s02 = __builtin_amdgcn_permlane32_swap(w[0][d], w[2][d], false, false);
+            const auto s13 = __builtin_amdgcn_permlane32_swap(w[1][d], w[3][d], false, false);
+            o[d] = s02[0];
+            o[DW + d] = s02[1];
+            o[2 * DW + d] = s13[0];
+            o[3 * DW + d] = s13[1];
+        }
+        const int c0 = ocol + 16 * g32;
+        if (grow >= g.M || c0 >= out_n1) return;
+        char* dst = ep.C + (int64_t)grow * ep.ldc + (int64_t)c0 * SZ;
+        if (ep.c_vec_ok && c0 + 16 <= out_n1) {
+#pragma unroll
+            for (int t = 0; t < DW; t++)
+                *reinterpret_cast<u32x4*>(dst + 16 * t) = u32x4{o[4 * t], o[4 * t + 1], o[4 * t + 2], o[4 * t + 3]};
         } else {
 #pragma unroll
-            for (int j = 0; j < NJ; j++) {
-                const int ncol = ntile0 + wn * WN + 32 * j + l32;
-                const bool col_ok = ncol < g.n1;
+            for (int e = 0; e < 16; e++) {
+                if (c0 + e < out_n1) {
+                    const uint32_t word = o[e * SZ / 4];
+                    if constexpr (SZ == 4) reinterpret_cast<uint32_t*>(dst)[e] = word;
+                    else if constexpr (SZ == 2) reinterpret_cast<uint16_t*>(dst)[e] = (uint16_t)(word >> (16 * (e & 1)));
+                    else reinterpret_cast<uint8_t*>(dst)[e] = (uint8_t)(word >> (8 * (e & 3)));
+                }
+            }
+        }
+    };
+
+    if (silu_gate) {
+        if constexpr (NJ % 2 == 0) {
+            static_for<0, NJ / 2>([&](auto jc) __attribute__((always_inline)) {
+                constexpr int j = 2 * decltype(jc)::value;
+                static_for<0, MI>([&](auto ic) __attribute__((always_inline)) {
+                    constexpr int i = decltype(ic)::value;
+                    float r[16];
+#pragma unroll
+                    for (int v = 0; v < 16; v++)
+                        r[v] = silu(MF::to_f32(acc_read(acc[i][j][v]))) * MF::to_f32(acc_read(acc[i][j + 1][v]));
+                    store_block(r, acc[i][j], m0 + wm * WM + 32 * i + l32, ((wave_col0 + 32 * j) >> 1));
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+            });
+        }
+    } else {
+        static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) {
+            constexpr int j = decltype(jc)::value;
+            const int bcol = wave_col0 + 32 * j;
+            float deq_v[16], bias_v[16], q_v[16];
+            if ((ep.steps & MMX_PP_DEQUANT) && ep.deq_oc) load_per_oc(ep.deq_oc, bcol, deq_v);
+            if (ep.steps & MMX_PP_BIAS) load_per_oc(ep.bias, bcol, bias_v);
+            if ((ep.steps & MMX_PP_QUANT) && ep.q_oc) load_per_oc(ep.q_oc, bcol, q_v);
+            static_for<0, MI>([&](auto ic) __attribute__((always_inline)) {
+                constexpr int i = decltype(ic)::value;
                 float r[16];
 #pragma unroll
-                for (int v = 0; v < 16; v++) r[v] = MF::to_f32(acc[i][j][v]);
+                for (int v = 0; v < 16; v++) r[v] = MF::to_f32(acc_read(acc[i][j][v]));
                 if (ep.steps & MMX_PP_DEQUANT) {
-                    const float d = ep.deq_oc ? (col_ok ? ep.deq_oc[ncol] : 0.0f) : ep.deq;
+                    if (ep.deq_oc) {
 #pragma unroll
-                    for (int v = 0; v < 16; v++) r[v] = r[v] * d;
+                        for (int v = 0; v < 16; v++) r[v] = r[v] * deq_v[v];
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 16; v++) r[v] = r[v] * ep.deq;
+                    }
                 }
                 if (ep.steps & MMX_PP_BIAS) {
-                    const float bv = col_ok ? ep.bias[ncol] : 0.0f;
 #pragma unroll
-                    for (int v = 0; v < 16; v++) r[v] = r[v] + bv;
+                    for (int v = 0; v < 16; v++) r[v] = r[v] + bias_v[v];
                 }
-                if (ep.steps & MMX_PP_GELU) {
-#pragma unroll
-                    for (int v = 0; v < 16; v++) r[v] = gelu_erf_minimax(r[v]);
-                }
+                if (ep.steps & MMX_PP_GELU) gelu_erf_minimax_x16(r);
                 if (ep.steps & MMX_PP_QUANT) {
-                    const float qv = ep.q_oc ? (col_ok ? ep.q_oc[ncol] : 0.0f) : ep.q;
+                    if (ep.q_oc) {
 #pragma unroll
-                    for (int v = 0; v < 16; v++) r[v] = r[v] * qv;
-                }
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const int row = 8 * (v >> 2) + 4 * g32 + (v & 3);
-                    TOut o;
-                    if constexpr (sizeof(TOut) == 4 && !__is_same(TOut, float)) {
-                        o = (TOut)acc[i][j][v];  // raw int32 accumulator
+                        for (int v = 0; v < 16; v++) r[v] = r[v] * q_v[v];
                     } else {
-                        o = cvt_out<TOut>(r[v]);
+#pragma unroll
+                        for (int v = 0; v < 16; v++) r[v] = r[v] * ep.q;
                     }
-                    *reinterpret_cast<TOut*>(stg + row * SROW + (j * 32 + l32) * SZ) = o;
                 }
-            }
-        }
-        __syncthreads();
-        const int ppr = wn_out * SZ / 16;  // 16-byte pieces per staged row
-        const int per_piece = 16 / SZ;
-        for (int idx = lane; idx < 32 * ppr; idx += 64) {
-            const int row = idx / ppr, piece = idx - row * ppr;
-            const int grow = m0 + wm * WM + 32 * i + row;
-            const int col0 = out_col_base + piece * per_piece;
-            if (grow < g.M && col0 < out_n1) {
-                const char* src = stg + row * SROW + piece * 16;
-                char* dst = ep.C + (int64_t)grow * ep.ldc + (int64_t)col0 * SZ;
-                if (ep.c_vec_ok && col0 + per_piece <= out_n1) {
-                    *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(src);
-                } else {
-                    for (int e = 0; e < per_piece; e++)
-                        if (col0 + e < out_n1)
-                            reinterpret_cast<TOut*>(dst)[e] = reinterpret_cast<const TOut*>(src)[e];
-                }
-            }
-        }
+                store_block(r, acc[i][j], m0 + wm * WM + 32 * i + l32, bcol);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        });
     }
 }
 
