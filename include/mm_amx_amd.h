@@ -131,14 +131,14 @@ int mmx_mlp(const void* x, int64_t ldx_bytes, const void* w_gate_up, const void*
             void* y, int64_t ldy_bytes, int M, int K, int N, void* stream);
 
 /* ---- introspection / tuning (no reference counterpart) --------------------------------------- */
-/* Force the MFMA tile shape ("256x256", "256x192", "128x256", "128x128", "" = automatic). */
+/* Force the MFMA tile shape ("256x256", "256x192", "128x256", "128x192", "128x128", "" = automatic). */
 int mmx_set_tile(const char* shape);
 /* Name of the kernel variant the last mmx_gemm call of this thread launched. */
 const char* mmx_last_kernel(void);
 /* Sets a kernel option.  "load_mode": how the MFMA tile kernel brings A and B tiles into LDS —
- * 0 through registers, 1 direct HBM->LDS loads through the compiler builtin, 2 (default) direct
- * HBM->LDS loads in a hand-scheduled ring pipeline.  Shapes whose M/K tails or alignment need
- * masked loads use a masked kernel whatever this is set to. */
+ * 2 (default) direct HBM->LDS loads in a hand-scheduled ring pipeline, 0 through registers (the
+ * fallback for operands beyond 32-bit offsets).  Shapes whose K tail or alignment need masked
+ * loads use a masked kernel whatever this is set to. */
 int mmx_set_option(const char* name, int value);
 /* HIP-event timing of `iters` back-to-back launches of the given gemm on `stream`, launch i
  * using the packed weights Bpacked_rot[i % n_rot] (rotate over several copies so that a

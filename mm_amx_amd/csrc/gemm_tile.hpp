@@ -11,17 +11,16 @@
 //      (row & 7) so that the 32 rows an MFMA operand needs hit all LDS banks;
 //   B  [BN/32 panels x 4 fragments x 1 KiB] already in MFMA operand order in HBM -> copied
 //      verbatim, every ds_read_b128 of a fragment is lane-contiguous.
-// Two LDS stages; loads of stage k+1 are in flight while stage k is multiplied.  Three load modes:
-//   MODE 0  global -> VGPR -> LDS (16-byte loads, rows past M clamped to the last row);
-//   MODE 1  global_load_lds_dwordx4 (HBM -> LDS without passing through VGPRs) through the
-//           compiler builtin; the compiler then waits for ALL outstanding LDS reads before each
-//           group of MFMAs (it counts the LDS-DMA as an out-of-order event);
-//   MODE 2  the same instruction issued from inline asm, so that the compiler's in-order
-//           accounting of ds_read results stays exact; its completion is awaited explicitly
-//           (s_waitcnt vmcnt(0) before the workgroup barrier);
-//   MODE 3  global -> VGPR -> LDS with per-element masking: the general path for K tails
-//           (K*sizeof(T) not a multiple of 128) and for A rows that are not 16-byte aligned.
-//           Rows past M and elements past K are read as zero, never touched in memory.
+// Three ways of bringing the tiles into LDS (template parameter MODE):
+//   MODE 2  the product path: global_load_lds_dwordx4 (HBM -> LDS without passing through VGPRs)
+//           issued from inline asm into a ring of half-stages, hand-scheduled against the MFMAs
+//           (see the comment at the pipeline);
+//   MODE 0  global -> VGPR -> LDS with 16-byte loads, two LDS stages, rows past M clamped to the
+//           last row: the fallback when A or the packed weights are too large for the 32-bit
+//           offsets MODE 2 addresses with, and a tested alternative;
+//   MODE 3  MODE 0 with per-element masking: the general path for K tails (K*sizeof(T) not a
+//           multiple of 128) and for A rows that are not 16-byte aligned.  Rows past M and
+//           elements past K are read as zero, never touched in memory.
 #pragma once
 #include <type_traits>
 
@@ -110,25 +109,6 @@ __device__ __forceinline__ u32x4 load_a_chunk_masked(const char* rowptr, int kby
     return u32x4{w[0], w[1], w[2], w[3]};
 }
 
-// 16 bytes per lane from global memory straight into LDS at lds_wave_base + lane*16
-// (lds_wave_base must be uniform across the wavefront: it travels in M0).
-template <int MODE>
-__device__ __forceinline__ void lds_dma16(const char* src, char* lds_wave_base) {
-    if constexpr (MODE == 1) {
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                         (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
-    } else {
-        const uint32_t m0 = __builtin_amdgcn_readfirstlane(
-            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_wave_base);
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0), "v"(src) : "memory");
-    }
-}
-template <int MODE>
-__device__ __forceinline__ void lds_dma_wait() {
-    if constexpr (MODE == 1) __builtin_amdgcn_s_waitcnt(0);
-    if constexpr (MODE == 2) asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
-}
-
 // LDS ring of the hand-scheduled pipeline: R half-stages of (BM + BN) rows x 64 bytes.
 template <int BM, int BN>
 struct Ring {
@@ -173,12 +153,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0;
 
-    constexpr bool DIRECT = (MODE == 1 || MODE == 2);
-    u32x4 ra[DIRECT ? 1 : A_IT], rb[DIRECT ? 1 : B_IT];
+    u32x4 ra[MODE == 2 ? 1 : A_IT], rb[MODE == 2 ? 1 : B_IT];  // staging registers of modes 0 and 3
 
-    auto fetch = [&](int kt, int stage) {
-        char* sA = smem + stage * STAGE;
-        char* sB = sA + A_BYTES;
+    auto fetch = [&](int kt) {
 #pragma unroll
         for (int it = 0; it < A_IT; it++) {
             const int c = it * 256 + tid;
@@ -188,8 +165,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             if constexpr (MODE != 3) {
                 grow = grow < g.M ? grow : g.M - 1;
                 const char* src = g.A + (int64_t)grow * g.lda + kt * 128 + chunk * 16;
-                if constexpr (DIRECT) lds_dma16<MODE>(src, sA + (it * 256 + wave * 64) * 16);
-                else ra[it] = *reinterpret_cast<const u32x4*>(src);
+                ra[it] = *reinterpret_cast<const u32x4*>(src);
             } else {
                 ra[it] = u32x4{0u, 0u, 0u, 0u};
                 if (grow < g.M)
@@ -205,22 +181,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             int panel = panel0 + it;
             panel = panel < g.npanels ? panel : g.npanels - 1;
             const char* src = g.Bp + (int64_t)panel * g.panel_stride + (int64_t)kt * 4096 + tid * 16;
-            if constexpr (DIRECT) {
-                lds_dma16<MODE>(src, sB + (it * 256 + wave * 64) * 16);
-            } else {
-                rb[it] = *reinterpret_cast<const u32x4*>(src);
-            }
+            rb[it] = *reinterpret_cast<const u32x4*>(src);
         }
     };
     auto commit = [&](int stage) {
-        if constexpr (!DIRECT) {
-            char* sA = smem + stage * STAGE;
-            char* sB = sA + A_BYTES;
+        char* sA = smem + stage * STAGE;
+        char* sB = sA + A_BYTES;
 #pragma unroll
-            for (int it = 0; it < A_IT; it++) *reinterpret_cast<u32x4*>(sA + (it * 256 + tid) * 16) = ra[it];
+        for (int it = 0; it < A_IT; it++) *reinterpret_cast<u32x4*>(sA + (it * 256 + tid) * 16) = ra[it];
 #pragma unroll
-            for (int it = 0; it < B_IT; it++) *reinterpret_cast<u32x4*>(sB + (it * 256 + tid) * 16) = rb[it];
-        }
+        for (int it = 0; it < B_IT; it++) *reinterpret_cast<u32x4*>(sB + (it * 256 + tid) * 16) = rb[it];
     };
 
     // Fragment registers are double buffered: the ds_reads of k-step s+1 are issued before the
@@ -370,9 +340,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         }
         asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // the re-fetched slots past the end must land before the wave ends
     } else {
-    fetch(0, 0);
+    fetch(0);
     commit(0);
-    lds_dma_wait<MODE>();
     __syncthreads();
     read_frags(0, 0, fa[0], fb[0]);
 
@@ -391,7 +360,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         // the last iteration re-fetches its own stage into the idle buffer: harmless, and it keeps
         // the loop body free of branches so that the schedule below is one straight block
         const int kt_next = (kt + 1 < g.nk) ? kt + 1 : kt;
-        fetch(kt_next, stage ^ 1);
+        fetch(kt_next);
         __builtin_amdgcn_sched_barrier(0);
         read_frags(stage, 1, fa[1], fb[1]);
         mma(fa[0], fb[0]);
@@ -406,8 +375,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         // stage has had three k-steps to land: synchronise here, then start reading the next
         // stage while the last k-step of this one is multiplied.
         commit(stage ^ 1);
-        lds_dma_wait<MODE>();
-        __syncthreads();
+            __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
         read_frags(stage ^ 1, 0, fa[0], fb[0]);
         mma(fa[1], fb[1]);
@@ -573,7 +541,7 @@ static inline TileCfg choose_tile(int M, int Ncols, bool need_pairs) {
     const TileCfg f = forced_tile();
     if (f.bm) return f;
     static const struct { int bm, bn; float eff; } cand[] = {
-        {256, 256, 1.00f}, {256, 192, 0.97f}, {128, 256, 0.90f}, {128, 128, 0.80f}};
+        {256, 256, 1.00f}, {256, 192, 0.97f}, {128, 256, 0.90f}, {128, 192, 0.86f}, {128, 128, 0.80f}};
     const int cus = num_cus();
     float best = 1e30f;
     TileCfg pick = {128, 128};
@@ -601,7 +569,7 @@ static int launch_cfg(const GemmArgs& g, int grid, hipStream_t st) {
     static bool attr_done = false;  // one flag and one name per instantiation
     static char name[64];
     if (!name[0]) {
-        static const char* const loads[] = {"regs", "dma", "ring", "masked"};
+        static const char* const loads[] = {"regs", "", "ring", "masked"};
         snprintf(name, sizeof name, "gemm_%s_%dx%d_%s_out_%s", type_tag<TIn>(), BM, BN, loads[MODE], type_tag<TOut>());
     }
     if (!attr_done) {
@@ -618,9 +586,8 @@ static int launch_cfg(const GemmArgs& g, int grid, hipStream_t st) {
 
 #define MMX_LAUNCH(TIn, BM, BN, MODE, TOut) \
     launch_cfg<TIn, BM, BN, MODE, TOut>(g, grid, st)
-#define MMX_LAUNCH_MODES(TIn, BM, BN, TOut)                                  \
-    (mode == 2 ? MMX_LAUNCH(TIn, BM, BN, 2, TOut)                            \
-               : mode == 1 ? MMX_LAUNCH(TIn, BM, BN, 1, TOut) : MMX_LAUNCH(TIn, BM, BN, 0, TOut))
+#define MMX_LAUNCH_MODES(TIn, BM, BN, TOut) \
+    (mode == 2 ? MMX_LAUNCH(TIn, BM, BN, 2, TOut) : MMX_LAUNCH(TIn, BM, BN, 0, TOut))
 
 template <typename TIn, typename TOut>
 static int launch_tiles(const GemmArgs& g, TileCfg t, int mode, int grid, hipStream_t st) {
@@ -628,6 +595,7 @@ static int launch_tiles(const GemmArgs& g, TileCfg t, int mode, int grid, hipStr
     if (t.bm == 256 && t.bn == 256) return MMX_LAUNCH_MODES(TIn, 256, 256, TOut);
     if (t.bm == 256 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 256, 192, TOut);
     if (t.bm == 128 && t.bn == 256) return MMX_LAUNCH_MODES(TIn, 128, 256, TOut);
+    if (t.bm == 128 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 128, 192, TOut);
     if (t.bm == 128 && t.bn == 128) return MMX_LAUNCH_MODES(TIn, 128, 128, TOut);
     return set_error(MMX_E_UNSUPPORTED, "no MFMA tile kernel for %dx%d", t.bm, t.bn);
 }

@@ -19,7 +19,7 @@ FC_SHAPES = [(16, 65, 32), (16, 66, 32), (16, 67, 32), (16, 68, 32), (16, 69, 32
 
 
 DEFAULT_LOAD_MODE = 2   # what the library starts with: the hand-scheduled HBM->LDS ring pipeline
-LOAD_NAMES = {0: "regs", 1: "dma", 2: "ring"}
+LOAD_NAMES = {0: "regs", 2: "ring"}
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -83,8 +83,8 @@ def test_bf16_exact_inputs_are_bit_exact(po):
     assert np.array_equal(host_bits(C), po.gemm_bf16(A, B))
 
 
-@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x128"])
-@pytest.mark.parametrize("mode", [0, 1, 2])
+@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x192", "128x128"])
+@pytest.mark.parametrize("mode", [0, 2])
 def test_bf16_bias_gelu_every_kernel_variant(po, tile, mode):
     M, K, N = 600, 512, 832
     rng = np.random.default_rng(11)
@@ -178,8 +178,8 @@ def test_int8_accumulators_bit_exact(po, shape):
     assert np.array_equal(host_bits(C), po.gemm_i8(A, B))
 
 
-@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x128"])
-@pytest.mark.parametrize("mode", [0, 1, 2])
+@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x192", "128x128"])
+@pytest.mark.parametrize("mode", [0, 2])
 def test_int8_requant_every_kernel_variant(po, tile, mode):
     M, K, N = 520, 1024, 704
     rng = np.random.default_rng(13)
