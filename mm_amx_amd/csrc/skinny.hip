@@ -58,11 +58,43 @@ __device__ __forceinline__ void store_out(const Epilogue& ep, int m, int n, floa
     }
 }
 
+// Per-column post-op operands of the (at most two) outputs per panel a thread finishes, requested
+// before the weight stream starts so that their latency is not paid after it.
+template <int NP>
+struct FinishOperands {
+    float deq[2][NP], bias[2][NP], q[2][NP];
+};
+template <int NP>
+__device__ __forceinline__ void skinny_prefetch(const SkinnyArgs& s, int panel_first, int tid, FinishOperands<NP>& o) {
+    const Epilogue& ep = s.ep;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int idx = tid + 512 * t;
+        const int v = idx >> 6, ln = idx & 63;
+        const int nloc = 8 * (v >> 2) + 4 * (ln >> 5) + (v & 3);
+        const bool row_live = (ln & 31) < s.M;
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            const int n = ((panel_first + p) << 5) + nloc;
+            const bool ok = row_live && n < s.n1 && !(ep.steps & MMX_PP_SILU_GATE);
+            o.deq[t][p] = ep.deq;
+            o.bias[t][p] = 0.0f;
+            o.q[t][p] = ep.q;
+            if (ok && (ep.steps & MMX_PP_DEQUANT) && ep.deq_oc) o.deq[t][p] = ep.deq_oc[n];
+            if (ok && (ep.steps & MMX_PP_BIAS)) o.bias[t][p] = ep.bias[n];
+            if (ok && (ep.steps & MMX_PP_QUANT) && ep.q_oc) o.q[t][p] = ep.q_oc[n];
+        }
+    }
+}
+
 // cross-wave reduction of the partial 32x32 blocks + post-op + store (shared by both decode kernels)
 template <int NP>
-__device__ __forceinline__ void skinny_finish(const SkinnyArgs& s, const float (&red)[8][NP][16][64], int panel_first, int tid) {
+__device__ __forceinline__ void skinny_finish(const SkinnyArgs& s, const float (&red)[8][NP][16][64], int panel_first, int tid,
+                                              const FinishOperands<NP>& o) {
     const Epilogue& ep = s.ep;
-    for (int idx = tid; idx < 16 * 64; idx += 512) {
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int idx = tid + 512 * t;
         const int v = idx >> 6, ln = idx & 63;
         const int m = ln & 31;
         if (m >= s.M) continue;
@@ -70,10 +102,10 @@ __device__ __forceinline__ void skinny_finish(const SkinnyArgs& s, const float (
         float sum[NP];
 #pragma unroll
         for (int p = 0; p < NP; p++) {
-            float t = 0.0f;
+            float acc = 0.0f;
 #pragma unroll
-            for (int w8 = 0; w8 < 8; w8++) t += red[w8][p][v][ln];
-            sum[p] = t;
+            for (int w8 = 0; w8 < 8; w8++) acc += red[w8][p][v][ln];
+            sum[p] = acc;
         }
         if (ep.steps & MMX_PP_SILU_GATE) {
             if constexpr (NP == 2) {
@@ -86,10 +118,10 @@ __device__ __forceinline__ void skinny_finish(const SkinnyArgs& s, const float (
                 const int n = ((panel_first + p) << 5) + nloc;
                 if (n >= s.n1) continue;
                 float r = sum[p];
-                if (ep.steps & MMX_PP_DEQUANT) r = r * (ep.deq_oc ? ep.deq_oc[n] : ep.deq);
-                if (ep.steps & MMX_PP_BIAS) r = r + ep.bias[n];
+                if (ep.steps & MMX_PP_DEQUANT) r = r * o.deq[t][p];
+                if (ep.steps & MMX_PP_BIAS) r = r + o.bias[t][p];
                 if (ep.steps & MMX_PP_GELU) r = gelu_erf_minimax(r);
-                if (ep.steps & MMX_PP_QUANT) r = r * (ep.q_oc ? ep.q_oc[n] : ep.q);
+                if (ep.steps & MMX_PP_QUANT) r = r * o.q[t][p];
                 store_out(ep, m, n, r);
             }
         }
@@ -111,6 +143,9 @@ __global__ __launch_bounds__(512) void skinny_kernel(const SkinnyArgs s) {
     for (int p = 0; p < NP; p++)
 #pragma unroll
         for (int v = 0; v < 16; v++) acc[p][v] = 0.0f;
+
+    FinishOperands<NP> fin;
+    skinny_prefetch<NP>(s, panel_first, tid, fin);
 
     const int per_wave = (s.nfrag + 7) / 8;
     const int f_begin = wave * per_wave;
@@ -160,44 +195,51 @@ __global__ __launch_bounds__(512) void skinny_kernel(const SkinnyArgs s) {
         for (int v = 0; v < 16; v++) red[wave][p][v][lane] = acc[p][v];
     __syncthreads();
 
-    skinny_finish<NP>(s, red, panel_first, tid);
+    skinny_finish<NP>(s, red, panel_first, tid, fin);
 }
 
 // ---- streaming variant for the smallest M -----------------------------------------------------------
-// When the activations fit in LDS (M * K_pad * 2 <= 32 KiB) the kernel is organised around one goal:
-// have every byte of the weights requested from HBM as early as possible.  Each wave first issues the
-// load of its slice of x, then 16 KiB of weight loads, and only then waits for x, publishes it to LDS
-// and starts consuming the weights in arrival order.  x fragments are re-read from LDS (a separate counter from the HBM loads, so they never
-// queue behind the weight stream).
-// 128 VGPRs at most: two workgroups per CU, so that every panel of a 11008-column matrix is resident at once
+// When the activations fit in LDS the kernel is organised around one goal: have every byte of the
+// weights requested from HBM as early as possible.  x goes from global memory straight into LDS
+// (global_load_lds, no registers), the few per-column post-op operands are requested, then each wave
+// issues 16 KiB of weight loads.  Loads return in order, so "at most the weight loads outstanding"
+// means x has landed: one barrier, and the weights are consumed in arrival order.  x fragments are
+// read from LDS (their own counter: they never queue behind the weight stream).  Lanes of rows >= M
+// and fragments past the end of K read a row of zeros instead, so the loop has no branches.
+// Requires K to fill whole 128-byte groups of the packed weights (no zero padding of x needed).
+// 128 VGPRs at most: two workgroups per CU, so that every panel of an 11008-column matrix is resident at once.
 template <bool W8, int NP>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void skinny_stream_kernel(const SkinnyArgs s, int kpad) {
-    constexpr int U = 16 / NP;  // fragments per wave in flight at once (16 KiB of weights)
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void skinny_stream_kernel(const SkinnyArgs s, int zero_off) {
+    constexpr int U = 16 / NP;  // fragments per panel per wave in flight at once (16 KiB of weights)
     __shared__ float red[8][NP][16][64];
-    extern __shared__ __attribute__((aligned(16))) char xs[];  // [M + 1][kpad] bf16, last row all zero
+    extern __shared__ __attribute__((aligned(1024))) char xs[];  // [M][K] bf16, then at zero_off a row of zeros
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: keeps the control flow below uniform
     const int l32 = lane & 31, g32 = lane >> 5;
     const int panel_first = (s.n0 >> 5) + blockIdx.x * NP;
     const int panel_end = (s.n1 + 31) >> 5;
+    const int row_bytes = s.K * 2;
+    const int real_bytes = s.M * row_bytes;
 
-    // x: 16 bytes per thread per pass, zero padded to kpad (plus the zero row); issued before any weight load
-    const int chunks_per_row = kpad >> 3;
-    const int real_chunks = s.M * chunks_per_row;
-    const int total_chunks = real_chunks + chunks_per_row;
-    constexpr int XP = 5;  // passes of 512 threads: up to 40 KiB
-    bf16x8 xreg[XP];
-#pragma unroll
-    for (int p = 0; p < XP; p++) {
-        const int c = p * 512 + tid;
-        const int m = c / chunks_per_row, k0 = (c - m * chunks_per_row) * 8;
-        // the launcher guarantees 16-byte aligned rows and K % 8 == 0: a chunk is all data or all padding
-        const bool has = c < real_chunks && k0 < s.K;
-        const bf16x8 v = *reinterpret_cast<const bf16x8*>(s.x + (int64_t)(has ? m : 0) * s.ldx + (int64_t)(has ? k0 : 0) * 2);
-#pragma unroll
-        for (int e = 0; e < 8; e++) xreg[p][e] = has ? v[e] : (__bf16)0.0f;
+    // x -> LDS, 1 KiB per wave per instruction; the lanes past the end of x re-read its last 16 bytes
+    // into the gap in front of the zero row (zero_off is the next multiple of 1 KiB)
+    {
+        const uint32_t lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)xs);
+        for (int off = wave * 1024; off < real_bytes; off += 8 * 1024) {
+            int bo = off + lane * 16;
+            bo = bo < real_bytes ? bo : real_bytes - 16;
+            const int m = bo / row_bytes;
+            const char* src = s.x + (int64_t)m * s.ldx + (bo - m * row_bytes);
+            const uint32_t m0v = lds_base + off;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0v), "v"(src) : "memory");
+        }
+        for (int c = tid * 16; c < row_bytes; c += 512 * 16) *reinterpret_cast<u32x4*>(xs + zero_off + c) = u32x4{0u, 0u, 0u, 0u};
     }
+    // the few per-column operands of the post-op travel ahead of the weights as well
+    FinishOperands<NP> fin;
+    skinny_prefetch<NP>(s, panel_first, tid, fin);
+    __builtin_amdgcn_sched_barrier(0);
 
     f32x16 acc[NP];
 #pragma unroll
@@ -206,7 +248,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         for (int v = 0; v < 16; v++) acc[p][v] = 0.0f;
 
     // wave w multiplies fragments [w*per_wave, (w+1)*per_wave); indices past the end are clamped for the
-    // load and paired with the zero row of x, so the code below has no per-fragment branches
+    // load and paired with the zero row of x
     const int per_wave = (s.nfrag + 7) / 8;
     const int f_begin = wave * per_wave;
     const int f_last = s.nfrag - 1;
@@ -217,28 +259,35 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         panel = (panel < panel_end && panel < s.npanels) ? panel : s.npanels - 1;  // columns past n1 are never stored
         wbase[p] = s.Wp + (int64_t)panel * s.panel_stride + lane * 16;
     }
-    const char* xrow = xs + (l32 < s.M ? l32 : s.M) * kpad * 2;
-    const char* zrow = xs + s.M * kpad * 2;
+    const char* zrow = xs + zero_off;
+    const char* xrow = l32 < s.M ? xs + l32 * row_bytes : zrow;
     const int nbatch = (per_wave + U - 1) / U;  // same for every wave
     for (int b = 0; b < nbatch; b++) {
         const int f0 = f_begin + b * U;
-        // the whole batch is requested before anything else happens
+        // the whole batch is requested before any of it is consumed
         u32x4 w[NP][U];
-#pragma unroll
-        for (int u = 0; u < U; u++) {
+        auto request = [&](int u) __attribute__((always_inline)) {
             int f = f0 + u;
             f = f < f_last ? f : f_last;
 #pragma unroll
             for (int p = 0; p < NP; p++) w[p][u] = *reinterpret_cast<const u32x4*>(wbase[p] + (int64_t)f * 1024);
-        }
+        };
         if (b == 0) {
-            // x was requested first and loads return in order: publish it while the weights are in flight
+            // A CU accepts only so many outstanding requests: a wave that had to get all of its weight
+            // requests accepted before it may look at x would sit there for most of the transfer.  So:
+            // a quarter of the batch (enough, over all waves, to keep HBM busy), then wait for x (loads
+            // return in order: "at most these outstanding" means x has landed), publish it, then the rest.
+            constexpr int U0 = U / 4;
 #pragma unroll
-            for (int p = 0; p < XP; p++) {
-                const int c = p * 512 + tid;
-                if (c < total_chunks) *reinterpret_cast<bf16x8*>(xs + c * 16) = xreg[p];
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory");
+            for (int u = 0; u < U0; u++) request(u);
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" : : "n"(U0 * NP) : "memory");
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = U0; u < U; u++) request(u);
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; u++) request(u);
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
@@ -268,7 +317,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #pragma unroll
         for (int v = 0; v < 16; v++) red[wave][p][v][lane] = acc[p][v];
     __syncthreads();
-    skinny_finish<NP>(s, red, panel_first, tid);
+    skinny_finish<NP>(s, red, panel_first, tid, fin);
 }
 
 int launch_skinny(bool w8, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
@@ -290,18 +339,15 @@ int launch_skinny(bool w8, const void* x, int64_t ldx, const void* Wp, int M, in
     const int panels = ((n1 + 31) >> 5) - (n0 >> 5);
     const bool pairs = (ep.steps & MMX_PP_SILU_GATE) != 0;
     const int kpad = kbytes_pad / (w8 ? 1 : 2);  // elements of K the packed weights cover
-    const int xbytes = (M + 1) * kpad * 2;  // x plus one zero row
-    if (xbytes <= 40960 && s.x_vec_ok && (K % 8) == 0) {
+    const int zero_off = (M * K * 2 + 1023) & ~1023;
+    const int xbytes = zero_off + K * 2;  // x, a gap up to the next KiB, one row of zeros
+    if (kpad == K && xbytes <= 40960 && s.x_vec_ok && !(pairs && w8)) {
         // the activations fit in LDS: streaming variant
         if (pairs && (panels & 1)) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
-        note_kernel(pairs ? (w8 ? "skinny_stream_w8_gateup" : "skinny_stream_bf16_gateup") : (w8 ? "skinny_stream_w8" : "skinny_stream_bf16"));
-        if (pairs) {
-            if (w8) hipLaunchKernelGGL((skinny_stream_kernel<true, 2>), dim3(panels / 2), dim3(512), xbytes, st, s, kpad);
-            else hipLaunchKernelGGL((skinny_stream_kernel<false, 2>), dim3(panels / 2), dim3(512), xbytes, st, s, kpad);
-        } else {
-            if (w8) hipLaunchKernelGGL((skinny_stream_kernel<true, 1>), dim3(panels), dim3(512), xbytes, st, s, kpad);
-            else hipLaunchKernelGGL((skinny_stream_kernel<false, 1>), dim3(panels), dim3(512), xbytes, st, s, kpad);
-        }
+        note_kernel(pairs ? "skinny_stream_bf16_gateup" : (w8 ? "skinny_stream_w8" : "skinny_stream_bf16"));
+        if (pairs) hipLaunchKernelGGL((skinny_stream_kernel<false, 2>), dim3(panels / 2), dim3(512), xbytes, st, s, zero_off);
+        else if (w8) hipLaunchKernelGGL((skinny_stream_kernel<true, 1>), dim3(panels), dim3(512), xbytes, st, s, zero_off);
+        else hipLaunchKernelGGL((skinny_stream_kernel<false, 1>), dim3(panels), dim3(512), xbytes, st, s, zero_off);
         return check_hip(hipGetLastError(), "skinny_stream_kernel launch");
     }
     if (pairs) {
