@@ -208,7 +208,9 @@ __global__ __launch_bounds__(512) void skinny_kernel(const SkinnyArgs s) {
 // and fragments past the end of K read a row of zeros instead, so the loop has no branches.
 // Requires K to fill whole 128-byte groups of the packed weights (no zero padding of x needed).
 // 128 VGPRs at most: two workgroups per CU, so that every panel of an 11008-column matrix is resident at once.
-template <bool W8, int NP>
+// ONE: every wave's share of K is a single batch (the common decode shapes); a variant of its own so that
+// each kernel holds one code path and stays within its registers.
+template <bool W8, int NP, bool ONE>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void skinny_stream_kernel(const SkinnyArgs s, int zero_off) {
     constexpr int U = 16 / NP;  // fragments per panel per wave in flight at once (16 KiB of weights)
     __shared__ float red[8][NP][16][64];
@@ -262,55 +264,65 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const char* zrow = xs + zero_off;
     const char* xrow = l32 < s.M ? xs + l32 * row_bytes : zrow;
     const int nbatch = (per_wave + U - 1) / U;  // same for every wave
-    for (int b = 0; b < nbatch; b++) {
-        const int f0 = f_begin + b * U;
-        // the whole batch is requested before any of it is consumed
-        u32x4 w[NP][U];
-        auto request = [&](int u) __attribute__((always_inline)) {
-            int f = f0 + u;
-            f = f < f_last ? f : f_last;
+    // U fragments per panel are in flight per wave at all times: register set u holds fragment u of a
+    // batch and is re-requested for the next batch as soon as it has been multiplied
+    u32x4 w[NP][U];
+#define MMX_REQUEST(BT, UU)                                                                                     \
+    do {                                                                                                        \
+        int f_ = f_begin + (BT) * U + (UU);                                                                     \
+        f_ = f_ < f_last ? f_ : f_last;                                                                         \
+        _Pragma("unroll") for (int p = 0; p < NP; p++)                                                          \
+            w[p][UU] = *reinterpret_cast<const u32x4*>(wbase[p] + (int64_t)f_ * 1024);                          \
+    } while (0)
+#define MMX_MULTIPLY(BT, UU)                                                                                    \
+    do {                                                                                                        \
+        const int f_ = f_begin + (BT) * U + (UU);                                                               \
+        const bool valid_ = (f_ - f_begin) < per_wave && f_ <= f_last; /* scalar */                             \
+        const int fc_ = f_ < f_last ? f_ : f_last;                                                              \
+        const char* xr_ = valid_ ? xrow : zrow;                                                                 \
+        if constexpr (W8) {                                                                                     \
+            const bf16x8 xa_ = *reinterpret_cast<const bf16x8*>(xr_ + (32 * fc_ + 16 * g32) * 2);               \
+            const bf16x8 xb_ = *reinterpret_cast<const bf16x8*>(xr_ + (32 * fc_ + 16 * g32 + 8) * 2);           \
+            _Pragma("unroll") for (int p = 0; p < NP; p++) {                                                    \
+                acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(w[p][UU].x, w[p][UU].y), xa_, acc[p], 0, 0, 0); \
+                acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(w[p][UU].z, w[p][UU].w), xb_, acc[p], 0, 0, 0); \
+            }                                                                                                   \
+        } else {                                                                                                \
+            const bf16x8 xa_ = *reinterpret_cast<const bf16x8*>(xr_ + (16 * fc_ + 8 * g32) * 2);                \
+            _Pragma("unroll") for (int p = 0; p < NP; p++)                                                      \
+                acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w[p][UU]), xa_, acc[p], 0, 0, 0); \
+        }                                                                                                       \
+    } while (0)
+    {
+        // A CU accepts only so many outstanding requests: a wave that had to get all of its weight
+        // requests accepted before it may look at x would sit there for most of the transfer.  So:
+        // a quarter of the first batch (enough, over all waves, to keep HBM busy), then wait for x (loads
+        // return in order: "at most these outstanding" means x has landed), publish it, then the rest.
+        constexpr int U0 = U / 4;
 #pragma unroll
-            for (int p = 0; p < NP; p++) w[p][u] = *reinterpret_cast<const u32x4*>(wbase[p] + (int64_t)f * 1024);
-        };
-        if (b == 0) {
-            // A CU accepts only so many outstanding requests: a wave that had to get all of its weight
-            // requests accepted before it may look at x would sit there for most of the transfer.  So:
-            // a quarter of the batch (enough, over all waves, to keep HBM busy), then wait for x (loads
-            // return in order: "at most these outstanding" means x has landed), publish it, then the rest.
-            constexpr int U0 = U / 4;
+        for (int u = 0; u < U0; u++) MMX_REQUEST(0, u);
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" : : "n"(U0 * NP) : "memory");
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int u = 0; u < U0; u++) request(u);
-            __builtin_amdgcn_sched_barrier(0);
-            asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" : : "n"(U0 * NP) : "memory");
-            __builtin_amdgcn_sched_barrier(0);
+        for (int u = U0; u < U; u++) MMX_REQUEST(0, u);
+    }
+    if constexpr (ONE) {  // every offset of this path is a compile-time constant
 #pragma unroll
-            for (int u = U0; u < U; u++) request(u);
-        } else {
+        for (int u = 0; u < U; u++) MMX_MULTIPLY(0, u);
+    } else {
+        for (int bt = 0; bt + 1 < nbatch; bt++) {
 #pragma unroll
-            for (int u = 0; u < U; u++) request(u);
-        }
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int f = f0 + u;
-            const bool valid = (f - f_begin) < per_wave && f <= f_last;  // scalar
-            const int fc = f < f_last ? f : f_last;
-            const char* xr = valid ? xrow : zrow;
-            if constexpr (W8) {
-                const bf16x8 xa = *reinterpret_cast<const bf16x8*>(xr + (32 * fc + 16 * g32) * 2);
-                const bf16x8 xb = *reinterpret_cast<const bf16x8*>(xr + (32 * fc + 16 * g32 + 8) * 2);
-#pragma unroll
-                for (int p = 0; p < NP; p++) {
-                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(w[p][u].x, w[p][u].y), xa, acc[p], 0, 0, 0);
-                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(w[p][u].z, w[p][u].w), xb, acc[p], 0, 0, 0);
-                }
-            } else {
-                const bf16x8 xa = *reinterpret_cast<const bf16x8*>(xr + (16 * fc + 8 * g32) * 2);
-#pragma unroll
-                for (int p = 0; p < NP; p++)
-                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w[p][u]), xa, acc[p], 0, 0, 0);
+            for (int u = 0; u < U; u++) {
+                MMX_MULTIPLY(bt, u);
+                MMX_REQUEST(bt + 1, u);
             }
         }
+#pragma unroll
+        for (int u = 0; u < U; u++) MMX_MULTIPLY(nbatch - 1, u);
     }
+#undef MMX_REQUEST
+#undef MMX_MULTIPLY
 
 #pragma unroll
     for (int p = 0; p < NP; p++)
@@ -341,13 +353,22 @@ int launch_skinny(bool w8, const void* x, int64_t ldx, const void* Wp, int M, in
     const int kpad = kbytes_pad / (w8 ? 1 : 2);  // elements of K the packed weights cover
     const int zero_off = (M * K * 2 + 1023) & ~1023;
     const int xbytes = zero_off + K * 2;  // x, a gap up to the next KiB, one row of zeros
-    if (kpad == K && xbytes <= 40960 && s.x_vec_ok && !(pairs && w8)) {
+    if (kpad == K && xbytes <= 46 * 1024 && s.x_vec_ok && !(pairs && w8)) {  // LDS: 2 x (this + 32 KiB) per CU
         // the activations fit in LDS: streaming variant
         if (pairs && (panels & 1)) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
         note_kernel(pairs ? "skinny_stream_bf16_gateup" : (w8 ? "skinny_stream_w8" : "skinny_stream_bf16"));
-        if (pairs) hipLaunchKernelGGL((skinny_stream_kernel<false, 2>), dim3(panels / 2), dim3(512), xbytes, st, s, zero_off);
-        else if (w8) hipLaunchKernelGGL((skinny_stream_kernel<true, 1>), dim3(panels), dim3(512), xbytes, st, s, zero_off);
-        else hipLaunchKernelGGL((skinny_stream_kernel<false, 1>), dim3(panels), dim3(512), xbytes, st, s, zero_off);
+        const int per_wave = (s.nfrag + 7) / 8;
+#define MMX_STREAM(W8, NP, GRID)                                                                                     \
+    do {                                                                                                             \
+        if (per_wave <= 16 / NP)                                                                                     \
+            hipLaunchKernelGGL((skinny_stream_kernel<W8, NP, true>), dim3(GRID), dim3(512), xbytes, st, s, zero_off); \
+        else                                                                                                         \
+            hipLaunchKernelGGL((skinny_stream_kernel<W8, NP, false>), dim3(GRID), dim3(512), xbytes, st, s, zero_off); \
+    } while (0)
+        if (pairs) MMX_STREAM(false, 2, panels / 2);
+        else if (w8) MMX_STREAM(true, 1, panels);
+        else MMX_STREAM(false, 1, panels);
+#undef MMX_STREAM
         return check_hip(hipGetLastError(), "skinny_stream_kernel launch");
     }
     if (pairs) {
