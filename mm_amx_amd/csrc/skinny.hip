@@ -198,6 +198,95 @@ __global__ __launch_bounds__(512) void skinny_kernel(const SkinnyArgs s) {
     skinny_finish<NP>(s, red, panel_first, tid, fin);
 }
 
+// ---- direct variant for aligned operands whose x does not fit in LDS ---------------------------------
+// Every lane reads its own 16 (bf16 weights) or 32 (int8 weights) bytes of x per fragment straight from
+// global memory (served by L2: all workgroups read the same x) together with the fragment, U of
+// them in flight per wave as a rolling window.  Lanes of rows >= M read row 0: in the MFMA an output
+// column depends on its own activation row only, and the columns of those lanes are never stored.
+// Requires 16-byte aligned x rows and a K that fills whole 128-byte groups of the packed weights.
+template <bool W8, int NP>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void skinny_direct_kernel(const SkinnyArgs s) {
+    constexpr int U = (W8 ? 6 : 8) / NP;
+    constexpr int XB = W8 ? 64 : 32;  // bytes of a row of x one fragment covers
+    __shared__ float red[8][NP][16][64];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, g32 = lane >> 5;
+    const int panel_first = (s.n0 >> 5) + blockIdx.x * NP;
+    const int panel_end = (s.n1 + 31) >> 5;
+
+    FinishOperands<NP> fin;
+    skinny_prefetch<NP>(s, panel_first, tid, fin);
+    __builtin_amdgcn_sched_barrier(0);
+
+    f32x16 acc[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[p][v] = 0.0f;
+
+    const int per_wave = (s.nfrag + 7) / 8;
+    const int f_begin = wave * per_wave;
+    const int f_last = s.nfrag - 1;
+    const char* wbase[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++) {
+        int panel = panel_first + p;
+        panel = (panel < panel_end && panel < s.npanels) ? panel : s.npanels - 1;
+        wbase[p] = s.Wp + (int64_t)panel * s.panel_stride + lane * 16;
+    }
+    const char* xlane = s.x + (int64_t)(l32 < s.M ? l32 : 0) * s.ldx + g32 * (XB / 2);
+    const int nbatch = (per_wave + U - 1) / U;
+
+    u32x4 w[NP][U];
+    bf16x8 xa[U], xb[W8 ? U : 1];
+#define MMX_REQUEST(BT, UU)                                                                 \
+    do {                                                                                    \
+        int f_ = f_begin + (BT) * U + (UU);                                                 \
+        f_ = f_ < f_last ? f_ : f_last;                                                     \
+        _Pragma("unroll") for (int p = 0; p < NP; p++)                                      \
+            w[p][UU] = *reinterpret_cast<const u32x4*>(wbase[p] + (int64_t)f_ * 1024);      \
+        xa[UU] = *reinterpret_cast<const bf16x8*>(xlane + (int64_t)f_ * XB);                \
+        if constexpr (W8) xb[UU] = *reinterpret_cast<const bf16x8*>(xlane + (int64_t)f_ * XB + 16); \
+    } while (0)
+    // a fragment index past this wave's share (or past the end of K) contributes nothing: its weights are zeroed
+#define MMX_MULTIPLY(BT, UU)                                                                \
+    do {                                                                                    \
+        const int f_ = f_begin + (BT) * U + (UU);                                           \
+        const bool valid_ = (f_ - f_begin) < per_wave && f_ <= f_last; /* scalar */         \
+        _Pragma("unroll") for (int p = 0; p < NP; p++) {                                    \
+            const u32x4 wv_ = valid_ ? w[p][UU] : u32x4{0u, 0u, 0u, 0u};                    \
+            if constexpr (W8) {                                                             \
+                acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(wv_.x, wv_.y), xa[UU], acc[p], 0, 0, 0); \
+                acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(wv_.z, wv_.w), xb[UU], acc[p], 0, 0, 0); \
+            } else {                                                                        \
+                acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wv_), xa[UU], acc[p], 0, 0, 0); \
+            }                                                                               \
+        }                                                                                   \
+    } while (0)
+#pragma unroll
+    for (int u = 0; u < U; u++) MMX_REQUEST(0, u);
+    for (int bt = 0; bt + 1 < nbatch; bt++) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            MMX_MULTIPLY(bt, u);
+            MMX_REQUEST(bt + 1, u);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) MMX_MULTIPLY(nbatch - 1, u);
+#undef MMX_REQUEST
+#undef MMX_MULTIPLY
+
+#pragma unroll
+    for (int p = 0; p < NP; p++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) red[wave][p][v][lane] = acc[p][v];
+    __syncthreads();
+    skinny_finish<NP>(s, red, panel_first, tid, fin);
+}
+
 // ---- streaming variant for the smallest M -----------------------------------------------------------
 // When the activations fit in LDS the kernel is organised around one goal: have every byte of the
 // weights requested from HBM as early as possible.  x goes from global memory straight into LDS
@@ -370,6 +459,15 @@ int launch_skinny(bool w8, const void* x, int64_t ldx, const void* Wp, int M, in
         else MMX_STREAM(false, 1, panels);
 #undef MMX_STREAM
         return check_hip(hipGetLastError(), "skinny_stream_kernel launch");
+    }
+    if (kpad == K && s.x_vec_ok && !(pairs && w8)) {
+        // aligned, but x is too large for LDS: every lane reads its own part of x
+        if (pairs && (panels & 1)) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
+        note_kernel(pairs ? "skinny_direct_bf16_gateup" : (w8 ? "skinny_direct_w8" : "skinny_direct_bf16"));
+        if (pairs) hipLaunchKernelGGL((skinny_direct_kernel<false, 2>), dim3(panels / 2), dim3(512), 0, st, s);
+        else if (w8) hipLaunchKernelGGL((skinny_direct_kernel<true, 1>), dim3(panels), dim3(512), 0, st, s);
+        else hipLaunchKernelGGL((skinny_direct_kernel<false, 1>), dim3(panels), dim3(512), 0, st, s);
+        return check_hip(hipGetLastError(), "skinny_direct_kernel launch");
     }
     if (pairs) {
         if (panels & 1) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
