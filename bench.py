@@ -27,11 +27,11 @@ PEAK_INT8_TOPS = 5000.0     # MI355X dense int8 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # HBM-side bytes per launch of the headline kernel, from two counter runs of this script under
-# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (KiB per dispatch: 81930 and 22020), each scaled by
+# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (KiB per dispatch: 81960 and 27920), each scaled by
 # what the same counter reads for the 256 MiB device copy of --calibrate-copy (factors 2.000 and 1.000);
 # the summary is profiles/gemm_bf16_256x192_ffn_up_M1024_hbm_traffic.txt.  Counters cannot be read from
 # inside the process, so the figure is only reported when the kernel that ran is the one profiled.
-MEASURED_TRAFFIC_BYTES = {"gemm_bf16_256x192_ring_out_bf16": (81930 * 2.000 + 22020 * 1.000) * 1024}
+MEASURED_TRAFFIC_BYTES = {"gemm_bf16_256x192_ring_out_bf16": (81960 * 2.000 + 27920 * 1.000) * 1024}
 
 
 def main():
@@ -150,6 +150,14 @@ def main():
         def avg_ms(Ain, packs, Nn, epi, iters, **kw):
             mx.time_gemm(Ain, packs, Nn, epi, max(3, iters // 10), **kw)
             return mx.time_gemm(Ain, packs, Nn, epi, iters, **kw)
+
+        # bf16 256^3, fp32 out, no post-op (launch-latency bound; reported, not a roofline case)
+        w1 = wl.gemm_bf16_256()
+        A1, B1 = dev_bf16(w1["A"]), mx.repack_b(dev_bf16(w1["B"]))
+        C1 = torch.zeros((256, 256), dtype=torch.float32, device="cuda")
+        ms = avg_ms(A1, [B1], 256, mx.Epilogue(C1, mx.PP_NONE), 200)
+        extra["bf16_gemm_256x256x256"] = {"us": round(ms * 1e3, 2), "tflops": round(2.0 * 256 ** 3 / ms / 1e9, 2),
+                                          "kernel": mx.last_kernel()}
 
         # bf16 FC sweep over M
         sweep = {}
