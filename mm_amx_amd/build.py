@@ -35,6 +35,8 @@ def build(verbose=False):
     if failed:
         raise RuntimeError("hipcc failed")
     subprocess.check_call(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
+    for obj in objs:
+        os.remove(obj)
     return LIB
 
 

@@ -397,3 +397,72 @@ def test_errors_are_loud():
         mx.LinearNxN().set_weight(torch.zeros((40, 64), dtype=torch.bfloat16, device="cuda"))
     with pytest.raises(mx.MmxError, match="on the GPU"):
         mx.repack_b(torch.zeros((64, 64), dtype=torch.bfloat16))
+
+
+# ---- seeded sweep over ragged shapes, strides and column ranges ----------------------------------------
+def _strided(rows, cols, dtype, pad, fill):
+    """A [rows, cols] view into a wider buffer (row stride cols + pad elements), buffer pre-filled."""
+    buf = torch.full((rows, cols + pad), fill, dtype=dtype, device="cuda")
+    return buf, buf[:, :cols]
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_int8_random_shapes_strides_and_ranges(po, seed):
+    """int8 FC with requant on ragged shapes: every M, K, N tail, input rows and output rows with
+    arbitrary strides (aligned and unaligned), a column sub-range; bit-exact, and nothing outside
+    C[:, n0:n1] is written."""
+    rng = np.random.default_rng(1000 + seed)
+    M = int(rng.integers(1, 300))
+    K = int(rng.integers(64, 700))
+    N = int(rng.integers(1, 400))
+    A = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    deq = rng.uniform(1e-5, 4e-5, N).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.2).astype(np.float32)
+    q = rng.uniform(10.0, 30.0, N).astype(np.float32)
+    steps = po.PP_DEQUANT | po.PP_BIAS | po.PP_QUANT
+    ref = po.pp(po.gemm_i8(A, B), steps, po.I8, bias=bias, deq_per_oc=deq, q_per_oc=q)
+    Abuf, Ad = _strided(M, K, torch.int8, int(rng.integers(0, 40)), 0)
+    Ad.copy_(dev(A))
+    Cbuf, Cd = _strided(M, N, torch.int8, int(rng.integers(0, 40)), 77)
+    work = (N + 31) // 32
+    lo = int(rng.integers(0, work))
+    n0, n1 = lo * 32, min(N, int(rng.integers(lo * 32 + 1, N + 1)))
+    ep = mx.Epilogue(Cd, steps, bias=dev(bias), deq_scale_per_oc=dev(deq), q_scale_per_oc=dev(q))
+    mx.gemm(Ad, mx.repack_b(dev(B)), N, ep, n0=n0, n1=n1)
+    got = host_bits(Cbuf)
+    want = np.full(got.shape, 77, dtype=np.int8)
+    want[:, n0:n1] = ref[:, n0:n1]
+    assert np.array_equal(got, want), f"M={M} K={K} N={N} range=[{n0},{n1}) kernel={mx.last_kernel()}"
+
+
+@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_bf16_random_shapes_strides_and_ranges(po, seed, out_dtype):
+    """bf16 FC with BIAS on ragged shapes and strides: the fused post-op equals the oracle's on the GPU's own
+    accumulators bit for bit, accumulators within tolerance, nothing outside C[:, n0:n1] is written."""
+    rng = np.random.default_rng(2000 + seed)
+    M = int(rng.integers(1, 300))
+    K = int(rng.integers(32, 700))
+    N = int(rng.integers(1, 400))
+    A, B = rand_bf16(rng, (M, K), 1.0), rand_bf16(rng, (K, N), 0.05)
+    bias = (rng.standard_normal(N) * 0.2).astype(np.float32)
+    acc_ref = po.gemm_bf16(A, B)
+    Abuf, Ad = _strided(M, K, torch.bfloat16, int(rng.integers(0, 24)), 0.0)
+    Ad.copy_(dev_bf16(A))
+    packed = mx.repack_b(dev_bf16(B))
+    acc = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    mx.gemm(Ad, packed, N, mx.Epilogue(acc, mx.PP_NONE))
+    check_float_parity(host_bits(acc), acc_ref, f"accumulators M={M} K={K} N={N}", frac_within=0.998)
+    Cbuf, Cd = _strided(M, N, out_dtype, int(rng.integers(0, 24)), 3.0)
+    work = (N + 31) // 32
+    lo = int(rng.integers(0, work))
+    n0, n1 = lo * 32, min(N, int(rng.integers(lo * 32 + 1, N + 1)))
+    mx.gemm(Ad, packed, N, mx.Epilogue(Cd, mx.PP_BIAS, bias=dev(bias)), n0=n0, n1=n1)
+    odt = po.BF16 if out_dtype == torch.bfloat16 else po.F32
+    ref = po.pp(host_bits(acc), po.PP_BIAS, odt, bias=bias)
+    got = host_bits(Cbuf)
+    fill = host_bits(torch.full((1,), 3.0, dtype=out_dtype, device="cuda"))[0]
+    want = np.full(got.shape, fill, dtype=got.dtype)
+    want[:, n0:n1] = ref[:, n0:n1]
+    assert np.array_equal(got, want), f"M={M} K={K} N={N} range=[{n0},{n1}) kernel={mx.last_kernel()}"
