@@ -466,3 +466,14 @@ def test_bf16_random_shapes_strides_and_ranges(po, seed, out_dtype):
     want = np.full(got.shape, fill, dtype=got.dtype)
     want[:, n0:n1] = ref[:, n0:n1]
     assert np.array_equal(got, want), f"M={M} K={K} N={N} range=[{n0},{n1}) kernel={mx.last_kernel()}"
+
+
+def test_mmbench_driver_runs_and_checks():
+    """The comparison driver in the shape of benchmark/mmbench: result keys and correctness flag."""
+    from mm_amx_amd import mmbench
+    for backend in ("mmamx", "torch"):
+        r = mmbench.benchmark(False, True, 64, 256, 512, 0.05, 4, True, backend=backend)
+        assert set(r) >= {"latency_ms", "times", "duration", "correct"} and r["times"] >= 1
+        assert r["correct"], (backend, r)
+    r = mmbench.benchmark(True, False, 33, 96, 128, 0.02, 0, True)  # transposed B, repacked on every call
+    assert r["correct"], r
