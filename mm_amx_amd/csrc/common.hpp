@@ -146,11 +146,66 @@ __device__ __forceinline__ float exp_poly(float x) {
     return s;
 }
 
-// tests/amx-mlp.cpp:450-456 — x * 1/(1+exp(-x)); the reciprocal is the correctly rounded one
-// (the reference's vrcp14ps approximation is an x86 instruction with no GPU counterpart).
+// vrcp14ps, bit for bit (the reference's sigmoid uses it, tests/amx-mlp.cpp:453).  A power of two gives
+// the exact reciprocal; otherwise the top 6 mantissa bits select a segment (table word = 18-bit
+// intercept a << 10 | 10-bit slope b), the next 10 bits are the offset d, the 17-bit significand is
+// (a*256 - b*d) >> 9 and the 7 low mantissa bits of the result are zero.  The table was derived from the
+// instruction and the model agrees with it on all 2^32 inputs.
+__constant__ static const uint32_t kRcp14Seg[64] = {
+    0x0fffe7f1u, 0x0fc0dbd1u, 0x0f83cbb5u, 0x0f488399u, 0x0f0eef7du, 0x0ed71f65u, 0x0ea0cf4bu, 0x0e6c1b35u,
+    0x0e38cb1du, 0x0e06f309u, 0x0dd662f3u, 0x0da72adfu, 0x0d7932cdu, 0x0d4c6ebbu, 0x0d20c6a9u, 0x0cf63297u,
+    0x0cccbe87u, 0x0ca44677u, 0x0c7cda69u, 0x0c564e59u, 0x0c30b64bu, 0x0c0bfe3du, 0x0be82a31u, 0x0bc51623u,
+    0x0ba2da17u, 0x0b81620bu, 0x0b60b601u, 0x0b40a9f5u, 0x0b215debu, 0x0b02b5dfu, 0x0ae4b9d5u, 0x0ac75dcbu,
+    0x0aaaa9c3u, 0x0a8e7db9u, 0x0a72f1b1u, 0x0a57e1a7u, 0x0a3d699fu, 0x0a237597u, 0x0a0a018fu, 0x09f10d87u,
+    0x09d8a181u, 0x09c09579u, 0x09a90571u, 0x0991ed6bu, 0x097b4565u, 0x0964f55du, 0x094f1957u, 0x0939a151u,
+    0x09248d4bu, 0x090fd545u, 0x08fb793fu, 0x08e7893bu, 0x08d3d935u, 0x08c0852fu, 0x08ad912bu, 0x089add25u,
+    0x08888921u, 0x08767d1du, 0x0864b517u, 0x08534d13u, 0x0842250fu, 0x08313d0bu, 0x08209507u, 0x08102d03u};
+
+// inputs and results outside the normal range: denormal inputs are normalised (not flushed), a result
+// beyond the largest float is inf, one below the normal range is the significand shifted right,
+// zero -> inf, inf -> 0, NaN -> quiet NaN
+static __device__ __attribute__((noinline)) float rcp14_special(float x) {
+    const uint32_t u = f2u(x);
+    const uint32_t sign = u & 0x80000000u;
+    int ex = (int)((u >> 23) & 0xffu);
+    uint32_t m = u & 0x7fffffu;
+    if (ex == 0xff) return m ? u2f(u | 0x00400000u) : u2f(sign);
+    if (ex == 0) {
+        if (m == 0) return u2f(sign | 0x7f800000u);
+        const int k = 31 - __builtin_clz(m);
+        m = (m << (23 - k)) & 0x7fffffu;
+        ex = k - 22;
+    }
+    uint32_t sig;
+    int rex;
+    if (m == 0) {
+        sig = 0x10000u;
+        rex = 254 - ex;
+    } else {
+        const uint32_t w = kRcp14Seg[m >> 17], d = (m >> 7) & 1023u;
+        sig = (((w >> 10) << 8) - (w & 1023u) * d) >> 9;
+        rex = 253 - ex;
+    }
+    if (rex >= 255) return u2f(sign | 0x7f800000u);
+    uint32_t mant24 = sig << 7;
+    if (rex <= 0) return u2f(sign | (mant24 >> (1 - rex)));
+    return u2f(sign | ((uint32_t)rex << 23) | (mant24 & 0x7fffffu));
+}
+
+__device__ __forceinline__ float rcp14(float x) {
+    const uint32_t u = f2u(x);
+    const uint32_t ex = (u >> 23) & 0xffu, m = u & 0x7fffffu;
+    if (!(ex - 1u < 252u)) return rcp14_special(x);  // exponent field 0, 253, 254, 255: rare
+    const uint32_t w = kRcp14Seg[m >> 17], d = (m >> 7) & 1023u;
+    const uint32_t sig = (((w >> 10) << 8) - (w & 1023u) * d) >> 9;
+    const uint32_t body = m ? (((253u - ex) << 23) | ((sig << 7) & 0x7fffffu)) : ((254u - ex) << 23);
+    return u2f((u & 0x80000000u) | body);
+}
+
+// tests/amx-mlp.cpp:450-456 — x * vrcp14ps(1 + exp(-x)), operation for operation
 __device__ __forceinline__ float silu(float x) {
     const float e = exp_poly(0.0f - x);
-    const float sig = 1.0f / (1.0f + e);
+    const float sig = rcp14(1.0f + e);
     return x * sig;
 }
 

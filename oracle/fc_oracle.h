@@ -27,13 +27,15 @@
  *   orc_gemv_w8            pinned  — through orc_gemm_bf16 on exactly converted weights
  *   orc_matvec_*           pinned  — against the compiled reference MatmulVector/GemAvB
  *                                    for ceil(K/kStep) <= 4 (the reference is wrong beyond)
- *   orc_silu               PARITY UNPINNED at the bit level: the reference's sigmoid uses
- *                          the Intel-only vrcp14ps approximation whose table is not
- *                          published and whose source file (tests/amx-mlp.cpp) needs
- *                          xbyak and cannot be built here.  The exp polynomial is
- *                          restated exactly; the reciprocal is correctly rounded.  Pinned
- *                          by mathematics only: |silu - x/(1+e^-x)| bounds, silu(0)=0,
- *                          limits.
+ *   orc_rcp14              pinned  — against the vrcp14ps instruction itself on all 2^32 inputs
+ *                                    (any AVX-512 host) and against committed vectors elsewhere
+ *   orc_exp_poly, orc_silu PARITY UNPINNED at the bit level: their source (tests/amx-mlp.cpp)
+ *                          needs xbyak and cannot be compiled here, so no run of the reference
+ *                          stands behind them.  Both are short straight-line sequences
+ *                          restated operation for operation (every instruction they use is
+ *                          pinned: fused multiply-add, floor, round-to-nearest convert,
+ *                          vrcp14ps); what is checked is the mathematics: |exp_poly - exp| and
+ *                          |silu - x/(1+e^-x)| bounds, silu(0) = 0, limits, overflow to inf.
  *   orc_mlp_*              pinned per GEMM stage (same as orc_gemm_bf16); the SiLU stage
  *                          inherits the note above.
  */
@@ -125,7 +127,11 @@ void orc_matvec_i8(const int8_t* A, int64_t lda, const int8_t* b, int32_t* c, in
 
 /* ---- fused MLP --------------------------------------------------------------------- */
 float orc_exp_poly(float x);  /* exp_ps_avx512 */
-float orc_silu(float x);      /* silu_ps_avx512 with a correctly rounded reciprocal */
+float orc_rcp14(float x);     /* vrcp14ps, bit for bit */
+void orc_rcp14_n(const float* src, float* dst, size_t n);
+void orc_silu_n(const float* src, float* dst, size_t n);
+void orc_exp_poly_n(const float* src, float* dst, size_t n);
+float orc_silu(float x);      /* silu_ps_avx512 */
 /* h[M,N] bf16 = bf16( silu(gate) * up ) from fp32 accumulators */
 void orc_silu_mul_bf16(const float* gate, const float* up, uint16_t* h, size_t n);
 /* x[M,K] bf16; w_gate,w_up [N,K] bf16; w_down [K,N] bf16 (torch nn.Linear.weight layouts).

@@ -107,10 +107,24 @@ def gelu(x):
     return out
 
 
-def silu(x):
+def _map(name, x):
     x = _c(x, np.float32)
-    f = lib().orc_silu
-    return np.array([f(float(v)) for v in x.ravel()], np.float32).reshape(x.shape)
+    out = np.empty_like(x)
+    getattr(lib(), name)(_p(x), _p(out), C.c_size_t(x.size))
+    return out
+
+
+def silu(x):
+    return _map("orc_silu_n", x)
+
+
+def exp_poly(x):
+    return _map("orc_exp_poly_n", x)
+
+
+def rcp14(x):
+    """vrcp14ps on every element (software model, see oracle/fc_oracle.c)."""
+    return _map("orc_rcp14_n", x)
 
 
 def pp(acc, steps, out_dtype, bias=None, deq=1.0, deq_per_oc=None, q=0.0, q_per_oc=None):

@@ -212,4 +212,33 @@ void ref_rcp14(const float* x, float* y, int n) {
     }
 }
 
+/* compares fn with the vrcp14ps instruction on every one of the 2^32 bit patterns (NaN results compare
+ * as NaN); returns the number of mismatches and the first mismatching input */
+long long ref_rcp14_check_all(float (*fn)(float), unsigned* first_bad) {
+    long long bad = 0;
+    unsigned first = 0;
+    int have_first = 0;
+#pragma omp parallel for schedule(static) reduction(+ : bad)
+    for (long long base = 0; base < (1ll << 32); base += 16) {
+        unsigned in[16], out[16];
+        for (int i = 0; i < 16; i++) in[i] = (unsigned)(base + i);
+        _mm512_storeu_si512((void*)out, _mm512_castps_si512(_mm512_rcp14_ps(_mm512_castsi512_ps(_mm512_loadu_si512((const void*)in)))));
+        for (int i = 0; i < 16; i++) {
+            float xf;
+            memcpy(&xf, &in[i], 4);
+            const float g = fn(xf);
+            unsigned gb;
+            memcpy(&gb, &g, 4);
+            const bool hw_nan = (out[i] & 0x7fffffffu) > 0x7f800000u, g_nan = (gb & 0x7fffffffu) > 0x7f800000u;
+            if (hw_nan ? !g_nan : gb != out[i]) {
+                bad++;
+#pragma omp critical
+                if (!have_first || in[i] < first) { first = in[i]; have_first = 1; }
+            }
+        }
+    }
+    if (first_bad) *first_bad = first;
+    return bad;
+}
+
 } // extern "C"

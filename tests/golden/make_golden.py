@@ -75,6 +75,20 @@ def main():
     r.ref_gelu(p(x), p(y), x.size)
     out["gelu_x"], out["gelu_y"] = x, y
 
+    # vrcp14ps: the instruction itself on sampled and special inputs (bit patterns in, bit patterns out)
+    xb = np.concatenate([
+        rng.integers(0, 1 << 32, 20000, dtype=np.uint64).astype(np.uint32),                 # anything
+        (np.uint32(0x3F800000) | rng.integers(0, 1 << 23, 10000).astype(np.uint32)),         # [1, 2)
+        (np.float32(1.0) + np.exp(rng.standard_normal(10000) * 3).astype(np.float32)).view(np.uint32),  # 1 + e^t
+        np.arange(0, 1 << 23, 16411, dtype=np.uint32),                                        # denormals
+        np.array([0x00000000, 0x80000000, 0x00000001, 0x001FFFFF, 0x00200000, 0x00200001, 0x00400000, 0x007FFFFF,
+                  0x00800000, 0x3F800000, 0x3F800001, 0x3FFFFFFF, 0x40000000, 0x7E800000, 0x7E800001, 0x7F000000,
+                  0x7F000001, 0x7F7FFFFF, 0x7F800000, 0xFF800000, 0x7FC00000, 0x7F800001, 0xFFFFFFFF, 0xBFC00000],
+                 np.uint32)])
+    yb = np.empty_like(xb)
+    r.ref_rcp14(p(xb), p(yb), xb.size)
+    out["rcp14_x"], out["rcp14_y"] = xb, yb
+
     # repackB_1x2 (AMX tile order), K and N tails, both element sizes and both transposes
     for es, dt in ((2, np.uint16), (1, np.int8)):
         K, N = 69, 40

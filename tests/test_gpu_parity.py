@@ -334,6 +334,13 @@ def _mlp_case(po, M, K, N, seed):
     h = host_bits(m.actUp[:M])
     # stage 1: h from the same x
     e1, f1 = check_float_parity(bf16_to_f32(h), bf16_to_f32(h_ref), f"mlp h M={M}")
+    # the fused SiLU(gate)*up store equals the oracle's, bit for bit, on the accumulators the GPU produced
+    # (gate and up alternate in 32-column panels of the packed matrix)
+    acc = torch.zeros((M, 2 * N), dtype=torch.float32, device="cuda")
+    mx.gemm(dev_bf16(w["x"]), m.gate_up, 2 * N, mx.Epilogue(acc, mx.PP_NONE))
+    a = host_bits(acc).reshape(M, N // 32, 2, 32)
+    gate, up = np.ascontiguousarray(a[:, :, 0, :]).reshape(M, N), np.ascontiguousarray(a[:, :, 1, :]).reshape(M, N)
+    assert np.array_equal(h, po.silu_mul_bf16(gate, up))
     # stage 2: y from the SAME h the GPU produced (chained parity is not attainable by ulp: the
     # down projection is a cancelling sum, so one-ulp changes of h move small y by many ulps)
     y_ref = po.mlp_down(h, w["w_down"], split_k=True)
@@ -344,6 +351,35 @@ def _mlp_case(po, M, K, N, seed):
     e3 = np.linalg.norm(yf - rf) / np.linalg.norm(rf)
     print(f"mlp M={M}: h rel={e1:.2e} ({f1 * 100:.3f}% <=1ulp)  y|h rel={e2:.2e} ({f2 * 100:.3f}%)  end-to-end rel={e3:.2e}")
     assert e3 < 3e-3
+
+
+@pytest.mark.parametrize("M", [32, 64])
+def test_silu_gate_special_values(po, M):
+    """SiLU(gate)*up on chosen gate values: one non-zero x per row and unit weights make the accumulators
+    equal the chosen values exactly, including those where exp overflows, where 1 + e^-x leaves the
+    normal range of the reciprocal (gate < -87), zero, and huge magnitudes.  bf16(silu(g) * 1) must be
+    the oracle's bits."""
+    K, N = 64, 64
+    vals = np.array([0.0, 1.0, -1.0, 0.5, -0.5, 3.0, -3.0, 17.0, -17.0, 80.0, -80.0, 87.0, -87.0, -87.5, -88.0, -88.5,
+                     -88.75, -89.0, -90.0, -100.0, -104.0, 120.0, -120.0, 2.0 ** 60, -(2.0 ** 60), 2.0 ** 100, -(2.0 ** 100),
+                     1e-3, -1e-3, 2.0 ** -40, -(2.0 ** -40), 0.25], np.float32)
+    g = np.resize(wl.bf16_bits_to_f32(wl.f32_to_bf16_bits(vals)), M).astype(np.float32)
+    x = np.zeros((M, K), np.uint16)
+    x[:, 0] = wl.f32_to_bf16_bits(g)
+    w_gate = np.zeros((N, K), np.uint16)
+    w_gate[:, 0] = wl.f32_to_bf16_bits(np.ones(N, np.float32))
+    w_up = w_gate.copy()
+    x[:, 1] = wl.f32_to_bf16_bits(np.ones(M, np.float32))      # up accumulator = 1 exactly: x[:,1] * w_up[:,1]
+    w_up[:, 0] = 0
+    w_up[:, 1] = wl.f32_to_bf16_bits(np.ones(N, np.float32))
+    packed = mx.repack_gate_up(dev_bf16(w_gate), dev_bf16(w_up))
+    h = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    mx.gemm(dev_bf16(x), packed, 2 * N, mx.Epilogue(h, mx.PP_SILU_GATE))
+    want = po.silu_mul_bf16(np.repeat(g[:, None], N, 1), np.ones((M, N), np.float32))
+    got = host_bits(h)
+    nan = np.isnan(bf16_to_f32(want))
+    assert np.array_equal(np.isnan(bf16_to_f32(got)), nan)
+    assert np.array_equal(got[~nan], want[~nan]), (mx.last_kernel(), g[np.flatnonzero((got != want).any(1))][:8])
 
 
 @pytest.mark.parametrize("M", [1, 5, 48, 300])

@@ -109,3 +109,13 @@ def test_bf16_rounding(po):
     back = po.bf16_to_f32(got)
     ok = f != np.float32(1e-40)
     assert np.all(np.abs(back[ok] - f[ok]) <= np.abs(f[ok]) * 2.0 ** -8)
+
+
+def test_rcp14_model(po):
+    """vrcp14ps: the software model against recorded outputs of the instruction (random bit patterns,
+    [1, 2), the 1 + e^t values SiLU feeds it, denormals, specials).  NaN results compare as NaN."""
+    x, want = G["rcp14_x"], G["rcp14_y"]
+    got = po.rcp14(x.view(np.float32)).view(np.uint32)
+    nan = (want & 0x7FFFFFFF) > 0x7F800000
+    assert ((got & 0x7FFFFFFF) > 0x7F800000)[nan].all()
+    assert np.array_equal(got[~nan], want[~nan])

@@ -13,10 +13,28 @@ def test_exp_polynomial_and_silu(po):
     assert po.lib().orc_exp_poly(200.0) > 1e38
     s = po.silu(xs).astype(np.float64)
     exact = xs.astype(np.float64) / (1 + np.exp(-xs.astype(np.float64)))
-    assert np.max(np.abs(s - exact)) < 2e-6
+    # the sigmoid comes from a 14-bit reciprocal: relative error below 2^-14 (plus the polynomial's)
+    assert np.all(np.abs(s - exact) <= np.abs(exact) * (2.0 ** -14 + 2e-6) + 1e-30)
     assert po.lib().orc_silu(0.0) == 0.0
-    assert abs(po.lib().orc_silu(30.0) - 30.0) < 1e-5
+    assert abs(po.lib().orc_silu(30.0) - 30.0) < 30 * 2.0 ** -14
     assert abs(po.lib().orc_silu(-30.0)) < 1e-10
+
+
+def test_rcp14_properties(po):
+    """What the definition of vrcp14ps fixes without the instruction at hand: relative error below 2^-14,
+    powers of two exact, monotone, sign symmetric, specials."""
+    rng = np.random.default_rng(5)
+    x = np.concatenate([np.exp(rng.uniform(-80, 80, 200000)), np.linspace(1, 2, 100001)]).astype(np.float32)
+    r = po.rcp14(x).astype(np.float64)
+    assert np.max(np.abs(r * x.astype(np.float64) - 1)) < 2.0 ** -14
+    p2 = (2.0 ** np.arange(-126, 127)).astype(np.float32)
+    assert np.array_equal(po.rcp14(p2), (1.0 / p2.astype(np.float64)).astype(np.float32))
+    xs = np.sort(x)
+    assert np.all(np.diff(po.rcp14(xs)) <= 0)
+    assert np.array_equal(po.rcp14(-x).view(np.uint32), po.rcp14(x).view(np.uint32) | 0x80000000)
+    sp = np.array([0.0, -0.0, np.inf, -np.inf], np.float32)
+    assert np.array_equal(po.rcp14(sp).view(np.uint32), np.array([0x7F800000, 0xFF800000, 0, 0x80000000], np.uint32))
+    assert np.isnan(po.rcp14(np.array([np.nan], np.float32))[0])
 
 
 def test_mlp_against_fp64(po):
