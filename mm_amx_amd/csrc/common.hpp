@@ -209,6 +209,43 @@ __device__ __forceinline__ float silu(float x) {
     return x * sig;
 }
 
+// silu(gate) * up on the 16 accumulator pairs a lane holds of one 32x32 block: the 16 chains advance in
+// lockstep (a lone wavefront cannot issue dependent instructions back to back), the table look-ups of
+// the reciprocal are issued together, and the rare operands outside the reciprocal's plain range are
+// patched afterwards behind a wave-uniform branch.  Same operations per element as silu() above.
+// `seg_of_lane` is kRcp14Seg[lane]: the 64-entry table lives in one register across the wavefront and is
+// indexed with ds_bpermute (no memory access, no latency of a load to wait for per block).
+__device__ __forceinline__ void silu_mul_x16(const float (&g)[16], const float (&up)[16], float (&r)[16], uint32_t seg_of_lane) {
+    float one_plus[16];
+#pragma unroll
+    for (int v = 0; v < 16; v++) one_plus[v] = 1.0f + exp_poly(0.0f - g[v]);
+    uint32_t w[16];
+    bool special = false;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        const uint32_t u = f2u(one_plus[v]);
+        w[v] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(((u & 0x7fffffu) >> 17) << 2), (int)seg_of_lane);
+        special |= !(((u >> 23) & 0xffu) - 1u < 252u);
+    }
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        const uint32_t u = f2u(one_plus[v]);
+        const uint32_t ex = (u >> 23) & 0xffu, m = u & 0x7fffffu, d = (m >> 7) & 1023u;
+        const uint32_t sig = (((w[v] >> 10) << 8) - (w[v] & 1023u) * d) >> 9;
+        const uint32_t body = m ? (((253u - ex) << 23) | ((sig << 7) & 0x7fffffu)) : ((254u - ex) << 23);
+        r[v] = (g[v] * u2f((u & 0x80000000u) | body)) * up[v];
+    }
+    if (__builtin_amdgcn_ballot_w64(special) != 0) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            float x = one_plus[v];
+            asm volatile("" : "+v"(x));  // keeps the patch inside this rarely taken branch
+            const uint32_t ex = (f2u(x) >> 23) & 0xffu;
+            if (!(ex - 1u < 252u)) r[v] = (g[v] * rcp14_special(x)) * up[v];
+        }
+    }
+}
+
 // fp32 -> bf16, round to nearest even (vcvtne2ps2bf16, include/kernels_amx.hpp:654)
 __device__ __forceinline__ uint16_t to_bf16(float x) {
     __bf16 b = (__bf16)x;

@@ -469,14 +469,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
     if (silu_gate) {
         if constexpr (NJ % 2 == 0) {
+            const uint32_t seg_of_lane = kRcp14Seg[lane];
             static_for<0, NJ / 2>([&](auto jc) __attribute__((always_inline)) {
                 constexpr int j = 2 * decltype(jc)::value;
                 static_for<0, MI>([&](auto ic) __attribute__((always_inline)) {
                     constexpr int i = decltype(ic)::value;
-                    float r[16];
+                    float gt[16], up[16], r[16];
 #pragma unroll
-                    for (int v = 0; v < 16; v++)
-                        r[v] = silu(MF::to_f32(acc_read(acc[i][j][v]))) * MF::to_f32(acc_read(acc[i][j + 1][v]));
+                    for (int v = 0; v < 16; v++) {
+                        gt[v] = MF::to_f32(acc_read(acc[i][j][v]));
+                        up[v] = MF::to_f32(acc_read(acc[i][j + 1][v]));
+                    }
+                    silu_mul_x16(gt, up, r, seg_of_lane);
                     store_block(r, acc[i][j], m0 + wm * WM + 32 * i + l32, ((wave_col0 + 32 * j) >> 1));
                     __builtin_amdgcn_sched_barrier(0);
                 });
