@@ -131,7 +131,7 @@ int mmx_mlp(const void* x, int64_t ldx_bytes, const void* w_gate_up, const void*
             void* y, int64_t ldy_bytes, int M, int K, int N, void* stream);
 
 /* ---- introspection / tuning (no reference counterpart) --------------------------------------- */
-/* Force the MFMA tile shape ("256x256", "256x192", "128x256", "128x192", "128x128", "" = automatic). */
+/* Force the MFMA tile shape ("256x256", "256x192", "128x256", "128x192", "128x128", "128x64", "" = automatic). */
 int mmx_set_tile(const char* shape);
 /* Name of the kernel variant the last mmx_gemm call of this thread launched. */
 const char* mmx_last_kernel(void);

@@ -123,7 +123,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     using MF = Mfma<TIn>;
     using frag = typename MF::frag;
     using accv = typename MF::accv;
-    constexpr int WM = BM / 2, WN = BN / 2;
+    // the four waves form a 2x2 grid over the tile, or 4x1 when the tile is only 64 columns wide
+    constexpr int WGN = BN >= 128 ? 2 : 1, WGM = 4 / WGN;
+    constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int MI = WM / 32, NJ = WN / 32;
     constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
     constexpr int A_IT = BM / 32, B_IT = BN / 32;  // 16-byte chunks per thread per stage
@@ -133,7 +135,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WGN, wn = wave % WGN;
     const int l32 = lane & 31, g32 = lane >> 5;
 
     // XCD-aware tile order: workgroup ids go round-robin over the 8 XCDs, so give each XCD a
@@ -230,7 +232,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         constexpr int MN = MI * NJ;                       // MFMAs per k-step
         constexpr int NL = A_IT2 + B_IT2;                 // HBM->LDS loads per thread per half-stage
         constexpr int H = (NL + 1) / 2;                   // issued in two groups, one load per MFMA slot
-        static_assert(H <= MN && MI + NJ <= MN, "not enough MFMA slots to spread the loads over");
+        constexpr int RPS = (MI + NJ + MN - 1) / MN;      // LDS reads per MFMA slot (1 unless the wave tile is tiny)
+        static_assert(H <= MN, "not enough MFMA slots to spread the loads over");
         static_assert((R - 2) * NL <= 63, "vmcnt is a 6-bit counter");
 
         // 64-byte rows: the 16-byte chunk c of row r sits at slot c ^ f(r), f chosen so that the 32 rows
@@ -291,8 +294,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
             for (int t = 0; t < MN; t++) {
                 acc[t / NJ][t % NJ] = MF::run(cb[t % NJ], ca[t / NJ], acc[t / NJ][t % NJ]);
-                if (t < NJ) nb[t] = *reinterpret_cast<const frag*>(sB + t * 2 * 1024);
-                else if (t < NJ + MI) na[t - NJ] = *reinterpret_cast<const frag*>(sA + (t - NJ) * 32 * 64);
+#pragma unroll
+                for (int rd = t * RPS; rd < (t + 1) * RPS; rd++) {
+                    if (rd < NJ) nb[rd] = *reinterpret_cast<const frag*>(sB + rd * 2 * 1024);
+                    else if (rd < NJ + MI) na[rd - NJ] = *reinterpret_cast<const frag*>(sA + (rd - NJ) * 32 * 64);
+                }
                 if (Q0 + t < Q1) dma(Q0 + t, fhs, fbuf);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -545,7 +551,7 @@ static inline TileCfg choose_tile(int M, int Ncols, bool need_pairs) {
     const TileCfg f = forced_tile();
     if (f.bm) return f;
     static const struct { int bm, bn; float eff; } cand[] = {
-        {256, 256, 1.00f}, {256, 192, 0.97f}, {128, 256, 0.90f}, {128, 192, 0.86f}, {128, 128, 0.80f}};
+        {256, 256, 1.00f}, {256, 192, 0.97f}, {128, 256, 0.90f}, {128, 192, 0.86f}, {128, 128, 0.80f}, {128, 64, 0.48f}};
     const int cus = num_cus();
     float best = 1e30f;
     TileCfg pick = {128, 128};
@@ -601,6 +607,7 @@ static int launch_tiles(const GemmArgs& g, TileCfg t, int mode, int grid, hipStr
     if (t.bm == 128 && t.bn == 256) return MMX_LAUNCH_MODES(TIn, 128, 256, TOut);
     if (t.bm == 128 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 128, 192, TOut);
     if (t.bm == 128 && t.bn == 128) return MMX_LAUNCH_MODES(TIn, 128, 128, TOut);
+    if (t.bm == 128 && t.bn == 64 && mode == 2) return MMX_LAUNCH(TIn, 128, 64, 2, TOut);  // ring pipeline only
     return set_error(MMX_E_UNSUPPORTED, "no MFMA tile kernel for %dx%d", t.bm, t.bn);
 }
 
@@ -627,6 +634,7 @@ static inline int prepare_gemm(GemmArgs& g, TileCfg& t, int& mode, int elesz, co
     if (mode == 2 && ((int64_t)M * lda >= ((int64_t)1 << 32) - 4096 || g.panel_stride >= ((int64_t)1 << 28))) mode = 0;
     t = choose_tile(M, n1 - n0, pairs);
     if (mode == 3) t = {128, 128};
+    if (mode != 2 && t.bn == 64) t = {128, 128};  // the 64-wide tile exists for the ring pipeline only
     if (pairs && (t.bn % 128) != 0)
         return set_error(MMX_E_INVALID, "SILU_GATE needs a tile width that is a multiple of 128");
     g.tiles_m = (M + t.bm - 1) / t.bm;
