@@ -198,7 +198,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(const SkinnyArgs s) {
     skinny_finish<NP>(s, red, panel_first, tid, fin);
 }
 
-// ---- direct variant for aligned operands whose x does not fit in LDS ---------------------------------
+// ---- direct variant for aligned operands whose x does not fit in LDS, few rows (4 < M <= 8) ----------
 // Every lane reads its own 16 (bf16 weights) or 32 (int8 weights) bytes of x per fragment straight from
 // global memory (served by L2: all workgroups read the same x) together with the fragment, U of
 // them in flight per wave as a rolling window.  Lanes of rows >= M read row 0: in the MFMA an output
@@ -279,6 +279,150 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #undef MMX_REQUEST
 #undef MMX_MULTIPLY
 
+#pragma unroll
+    for (int p = 0; p < NP; p++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) red[wave][p][v][lane] = acc[p][v];
+    __syncthreads();
+    skinny_finish<NP>(s, red, panel_first, tid, fin);
+}
+
+// ---- chunked variant for aligned operands whose x does not fit in LDS, many rows (8 < M <= 32) ------
+// K is walked in chunks of 8*FPW fragments; in a chunk every wave multiplies FPW fragments of each
+// panel.  The x a chunk needs ([M][RB bytes], RB = 8*FPW fragments' worth of a row) is fetched by the
+// whole workgroup with fully coalesced 16-byte loads (a lane per 16 bytes, rows back to back), written
+// to LDS and read from there as MFMA operands: fetched per lane straight from global memory, the 32
+// rows of an operand make every load touch 32 cache lines, and the CU's vector cache becomes the
+// bottleneck (19 us instead of 12 for the 4096 x 11008 int8 GEMV at M = 16).
+// Weights and x of chunk c+W are requested while chunk c is multiplied (W = 3 chunks in flight; all
+// loads are ordinary loads, so the compiler's own counting of outstanding loads places the waits).
+// Two LDS buffers: chunk c+1 is written while slower waves still read chunk c; the barrier of chunk
+// c+1 is what allows chunk c+2 to overwrite chunk c.  16-byte pieces of a row are XOR-swizzled with
+// the row so that the 32 rows an operand reads spread over the banks.
+// Lanes of rows >= M read row 0 (their output columns are never stored); fragments past the end of K
+// get zero weights and a clamped (finite) x.
+template <bool W8, int NP, int FPW, int XD>  // XD: 16-byte x loads per thread per chunk (8 KiB of x each)
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void skinny_chunk_kernel(const SkinnyArgs s) {
+    constexpr int W = (FPW == 2 && (W8 || NP == 2)) ? 2 : 3;  // chunks in flight (what 128 registers hold)
+    constexpr int XB = W8 ? 64 : 32;     // bytes of a row of x one fragment covers
+    constexpr int FC = 8 * FPW;          // fragments per chunk
+    constexpr int RB = FC * XB;          // bytes of a row of x per chunk
+    constexpr int BUF = 8 * XD * 1024;   // one LDS buffer: BUF / RB rows of x (the launcher checks M against it)
+    static_assert(RB >= 256 && BUF / RB >= 16, "chunk geometry");
+    extern __shared__ __attribute__((aligned(1024))) char smem[];  // 2 x BUF, later the cross-wave reduction
+    typedef float Red[8][NP][16][64];
+    Red& red = *reinterpret_cast<Red*>(smem);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, g32 = lane >> 5;
+    const int panel_first = (s.n0 >> 5) + blockIdx.x * NP;
+    const int panel_end = (s.n1 + 31) >> 5;
+
+    FinishOperands<NP> fin;
+    skinny_prefetch<NP>(s, panel_first, tid, fin);
+
+    f32x16 acc[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[p][v] = 0.0f;
+
+    const int f_last = s.nfrag - 1;
+    const int nchunk = (s.nfrag + FC - 1) / FC;
+    const int row_bytes = s.K * 2;
+    const char* wbase[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++) {
+        int panel = panel_first + p;
+        panel = (panel < panel_end && panel < s.npanels) ? panel : s.npanels - 1;
+        wbase[p] = s.Wp + (int64_t)panel * s.panel_stride + lane * 16;
+    }
+    // this thread's share of a chunk of x: XD pieces of 16 bytes; piece t sits at (row xrow[t], 16-byte
+    // column xcol[t]) of the chunk and goes to LDS offset xdst[t]
+    const char* xsrc[XD];
+    int xcol[XD], xdst[XD];
+#pragma unroll
+    for (int t = 0; t < XD; t++) {
+        const int pos = (wave + 8 * t) * 1024 + lane * 16;
+        const int r = pos / RB, cl = (pos % RB) / 16;
+        xsrc[t] = s.x + (int64_t)(r < s.M ? r : s.M - 1) * s.ldx;
+        xcol[t] = cl * 16;
+        xdst[t] = r * RB + ((cl ^ (r & 15)) * 16);
+    }
+    const int mrow = l32 < s.M ? l32 : 0;
+    const char* xread = smem + mrow * RB;
+    const int xswz = mrow & 15;
+
+    u32x4 w[W][FPW][NP];
+    bf16x8 xr[W][XD];
+#define MMX_LOAD(C, J)                                                                                         \
+    do {                                                                                                       \
+        _Pragma("unroll") for (int t = 0; t < XD; t++) {                                                       \
+            int kb_ = (C) * RB + xcol[t];                                                                      \
+            kb_ = kb_ < row_bytes - 16 ? kb_ : row_bytes - 16;                                                 \
+            xr[J][t] = *reinterpret_cast<const bf16x8*>(xsrc[t] + kb_);                                        \
+        }                                                                                                      \
+        _Pragma("unroll") for (int u = 0; u < FPW; u++) {                                                      \
+            int f_ = (C) * FC + wave * FPW + u;                                                                \
+            f_ = f_ < f_last ? f_ : f_last;                                                                    \
+            _Pragma("unroll") for (int p = 0; p < NP; p++)                                                     \
+                w[J][u][p] = *reinterpret_cast<const u32x4*>(wbase[p] + (int64_t)f_ * 1024);                   \
+        }                                                                                                      \
+    } while (0)
+#define MMX_CHUNK(C, J)                                                                                        \
+    do {                                                                                                       \
+        char* buf_ = smem + ((C) & 1) * BUF;                                                                   \
+        _Pragma("unroll") for (int t = 0; t < XD; t++) *reinterpret_cast<bf16x8*>(buf_ + xdst[t]) = xr[J][t];  \
+        __syncthreads();                                                                                       \
+        _Pragma("unroll") for (int u = 0; u < FPW; u++) {                                                      \
+            const int fl_ = wave * FPW + u;                                                                    \
+            const bool valid_ = (C) * FC + fl_ <= f_last; /* scalar */                                         \
+            const char* xb_ = xread + ((C) & 1) * BUF;                                                         \
+            if constexpr (W8) {                                                                                \
+                const int c0_ = fl_ * 4 + g32 * 2;                                                             \
+                const bf16x8 xa_ = *reinterpret_cast<const bf16x8*>(xb_ + ((c0_ ^ xswz) * 16));                \
+                const bf16x8 xc_ = *reinterpret_cast<const bf16x8*>(xb_ + (((c0_ + 1) ^ xswz) * 16));          \
+                _Pragma("unroll") for (int p = 0; p < NP; p++) {                                               \
+                    const u32x4 wv_ = valid_ ? w[J][u][p] : u32x4{0u, 0u, 0u, 0u};                             \
+                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(wv_.x, wv_.y), xa_, acc[p], 0, 0, 0); \
+                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(wv_.z, wv_.w), xc_, acc[p], 0, 0, 0); \
+                }                                                                                              \
+            } else {                                                                                           \
+                const int c0_ = fl_ * 2 + g32;                                                                 \
+                const bf16x8 xa_ = *reinterpret_cast<const bf16x8*>(xb_ + ((c0_ ^ xswz) * 16));                \
+                _Pragma("unroll") for (int p = 0; p < NP; p++) {                                               \
+                    const u32x4 wv_ = valid_ ? w[J][u][p] : u32x4{0u, 0u, 0u, 0u};                             \
+                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, wv_), xa_, acc[p], 0, 0, 0); \
+                }                                                                                              \
+            }                                                                                                  \
+        }                                                                                                      \
+    } while (0)
+
+    if (0 < nchunk) MMX_LOAD(0, 0);
+    if (1 < nchunk) MMX_LOAD(1, 1);
+    if constexpr (W == 3) {
+        if (2 < nchunk) MMX_LOAD(2, 2);
+    }
+    for (int c0 = 0; c0 < nchunk; c0 += W) {
+        MMX_CHUNK(c0, 0);
+        if (c0 + W < nchunk) MMX_LOAD(c0 + W, 0);
+        if (c0 + 1 < nchunk) {
+            MMX_CHUNK(c0 + 1, 1);
+            if (c0 + 1 + W < nchunk) MMX_LOAD(c0 + 1 + W, 1);
+        }
+        if constexpr (W == 3) {
+            if (c0 + 2 < nchunk) {
+                MMX_CHUNK(c0 + 2, 2);
+                if (c0 + 2 + W < nchunk) MMX_LOAD(c0 + 2 + W, 2);
+            }
+        }
+    }
+#undef MMX_LOAD
+#undef MMX_CHUNK
+    static_assert(W == 2 || W == 3, "the loop above is unrolled by hand");
+
+    __syncthreads();  // all reads of x are done: the buffers become the reduction scratch
 #pragma unroll
     for (int p = 0; p < NP; p++)
 #pragma unroll
@@ -460,14 +604,38 @@ int launch_skinny(bool w8, const void* x, int64_t ldx, const void* Wp, int M, in
 #undef MMX_STREAM
         return check_hip(hipGetLastError(), "skinny_stream_kernel launch");
     }
-    if (kpad == K && s.x_vec_ok && !(pairs && w8)) {
-        // aligned, but x is too large for LDS: every lane reads its own part of x
+    if (kpad == K && s.x_vec_ok && !(pairs && w8) && M <= 8) {
+        // aligned, x too large for LDS, few rows: every lane reads its own part of x
         if (pairs && (panels & 1)) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
         note_kernel(pairs ? "skinny_direct_bf16_gateup" : (w8 ? "skinny_direct_w8" : "skinny_direct_bf16"));
         if (pairs) hipLaunchKernelGGL((skinny_direct_kernel<false, 2>), dim3(panels / 2), dim3(512), 0, st, s);
         else if (w8) hipLaunchKernelGGL((skinny_direct_kernel<true, 1>), dim3(panels), dim3(512), 0, st, s);
         else hipLaunchKernelGGL((skinny_direct_kernel<false, 1>), dim3(panels), dim3(512), 0, st, s);
         return check_hip(hipGetLastError(), "skinny_direct_kernel launch");
+    }
+    if (kpad == K && s.x_vec_ok && !(pairs && w8)) {
+        // aligned, x too large for LDS, many rows: x goes through LDS chunk by chunk
+        if (pairs && (panels & 1)) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
+        note_kernel(pairs ? "skinny_chunk_bf16_gateup" : (w8 ? "skinny_chunk_w8" : "skinny_chunk_bf16"));
+        // LDS: two x buffers of 8 or 16 KiB, later the reduction scratch (32 KiB per panel)
+#define MMX_CHUNKED(W8, NP, FPW, XD, GRID)                                                                          \
+    do {                                                                                                            \
+        constexpr int lds_ = (2 * 8 * XD * 1024) > (8 * NP * 16 * 64 * 4) ? (2 * 8 * XD * 1024) : (8 * NP * 16 * 64 * 4); \
+        hipLaunchKernelGGL((skinny_chunk_kernel<W8, NP, FPW, XD>), dim3(GRID), dim3(512), lds_, st, s);            \
+    } while (0)
+        // rows of x per buffer = 8 KiB * XD / (8 * FPW fragments * 64 or 32 bytes)
+        if (pairs) {
+            if (M <= 16) MMX_CHUNKED(false, 2, 2, 1, panels / 2);
+            else MMX_CHUNKED(false, 2, 1, 1, panels / 2);
+        } else if (w8) {
+            if (M <= 16) MMX_CHUNKED(true, 1, 1, 1, panels);
+            else MMX_CHUNKED(true, 1, 1, 2, panels);
+        } else {
+            if (M <= 16) MMX_CHUNKED(false, 1, 2, 1, panels);
+            else MMX_CHUNKED(false, 1, 1, 1, panels);
+        }
+#undef MMX_CHUNKED
+        return check_hip(hipGetLastError(), "skinny_chunk_kernel launch");
     }
     if (pairs) {
         if (panels & 1) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
