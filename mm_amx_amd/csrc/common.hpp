@@ -262,4 +262,20 @@ __device__ __forceinline__ int8_t to_s8_sat(float r) {
     return (int8_t)(int)t;
 }
 
+// Four values through to_s8_sat packed into one dword (byte e = element e): round to nearest even, the
+// x86 "indefinite" cases (NaN, |r| >= 2^31; -2^31 itself saturates to the same -128) forced to -128,
+// then +128 and v_cvt_pk_u8_f32, whose saturation to [0, 255] is the clamp to [-128, 127], and one XOR
+// turns the biased bytes back into two's complement.
+__device__ __forceinline__ uint32_t to_s8_sat_x4(float r0, float r1, float r2, float r3) {
+    const float r[4] = {r0, r1, r2, r3};
+    uint32_t packed = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        float t = __builtin_rintf(r[e]);
+        if (!(__builtin_fabsf(r[e]) < 2147483648.0f)) t = -128.0f;
+        packed = __builtin_amdgcn_cvt_pk_u8_f32(t + 128.0f, (uint32_t)e, packed);
+    }
+    return packed ^ 0x80808080u;
+}
+
 }  // namespace mmx

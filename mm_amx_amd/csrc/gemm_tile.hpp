@@ -437,9 +437,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 w[q][0] = (uint32_t)to_bf16(r[4 * q]) | ((uint32_t)to_bf16(r[4 * q + 1]) << 16);
                 w[q][1] = (uint32_t)to_bf16(r[4 * q + 2]) | ((uint32_t)to_bf16(r[4 * q + 3]) << 16);
             } else {
-                w[q][0] = (uint32_t)(uint8_t)to_s8_sat(r[4 * q]) | ((uint32_t)(uint8_t)to_s8_sat(r[4 * q + 1]) << 8) |
-                          ((uint32_t)(uint8_t)to_s8_sat(r[4 * q + 2]) << 16) |
-                          ((uint32_t)(uint8_t)to_s8_sat(r[4 * q + 3]) << 24);
+                w[q][0] = to_s8_sat_x4(r[4 * q], r[4 * q + 1], r[4 * q + 2], r[4 * q + 3]);
             }
         }
         // lower half-wave: runs 0,1 of both halves = columns 0..15; upper half-wave: runs 2,3 = 16..31

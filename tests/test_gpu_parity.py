@@ -517,3 +517,26 @@ def test_mmbench_driver_runs_and_checks():
         assert r["correct"], (backend, r)
     r = mmbench.benchmark(True, False, 33, 96, 128, 0.02, 0, True)  # transposed B, repacked on every call
     assert r["correct"], r
+
+
+def test_int8_store_rounding_and_saturation_edges(po):
+    """The int8 store on chosen accumulator values: ties (x.5 to even), the saturation edges, values beyond
+    the int32 range and infinities (x86's cvtps2dq gives INT_MIN there, which saturates to -128, also for
+    large POSITIVE values: include/kernels_amx.hpp:658-661).  One non-zero x per row and unit weights make
+    the accumulators equal the chosen values exactly."""
+    vals = np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 126.5, 127.0, 127.5, 128.0, 300.0, -127.5, -128.0, -128.5, -129.0,
+                     -300.0, 2.0 ** 31, -(2.0 ** 31), 2.0 ** 32, -(2.0 ** 32), 2.0 ** 30, -(2.0 ** 30), 1e38, -1e38,
+                     np.inf, -np.inf, 0.0, 63.5, 64.5, -63.5, -64.5, 1e-3], np.float32)
+    M, K, N = 128, 64, 96
+    g = np.resize(wl.bf16_bits_to_f32(wl.f32_to_bf16_bits(vals)), M).astype(np.float32)
+    x = np.zeros((M, K), np.uint16)
+    x[:, 0] = wl.f32_to_bf16_bits(g)
+    W = np.zeros((K, N), np.uint16)
+    W[0, :] = wl.f32_to_bf16_bits(np.ones(N, np.float32))
+    acc = np.repeat(g[:, None], N, 1)
+    for steps, q in ((0, 0.0), (po.PP_QUANT, 0.5)):
+        ref = po.pp(acc, steps, po.I8, q=q)
+        for Mrun in (M, 16):   # tile kernel and decode kernel
+            C = torch.zeros((Mrun, N), dtype=torch.int8, device="cuda")
+            mx.gemm(dev_bf16(x[:Mrun]), mx.repack_b(dev_bf16(W)), N, mx.Epilogue(C, steps, q_scale=q))
+            assert np.array_equal(host_bits(C), ref[:Mrun]), (mx.last_kernel(), steps)
