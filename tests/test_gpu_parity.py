@@ -540,3 +540,11 @@ def test_int8_store_rounding_and_saturation_edges(po):
             C = torch.zeros((Mrun, N), dtype=torch.int8, device="cuda")
             mx.gemm(dev_bf16(x[:Mrun]), mx.repack_b(dev_bf16(W)), N, mx.Epilogue(C, steps, q_scale=q))
             assert np.array_equal(host_bits(C), ref[:Mrun]), (mx.last_kernel(), steps)
+
+
+def test_llama_mlp_stack_demo():
+    """torch-ext/test.py:176-218 in small: a stack of RMSNorm + MLP through torch's linear layers and through
+    the fused MLP gives the same result up to bf16 rounding of the intermediates."""
+    from mm_amx_amd import mlp_llama
+    r = mlp_llama.perf_llama7b_MLP(M=40, num_layers=3, rounds=1, hidden_size=512, intermediate_size=1024, verbose=False)
+    assert r["rel_err_one_layer"] < 1e-2 and r["rel_err"] < 5e-2 and r["mm_amx_amd"]["per_layer_us"] > 0
