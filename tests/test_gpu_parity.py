@@ -548,3 +548,20 @@ def test_llama_mlp_stack_demo():
     from mm_amx_amd import mlp_llama
     r = mlp_llama.perf_llama7b_MLP(M=40, num_layers=3, rounds=1, hidden_size=512, intermediate_size=1024, verbose=False)
     assert r["rel_err_one_layer"] < 1e-2 and r["rel_err"] < 5e-2 and r["mm_amx_amd"]["per_layer_us"] > 0
+
+
+def test_packed_weight_file_round_trip(po, tmp_path):
+    """Packed int8 weights + per-channel scales written to a file, read back, used: same bits as before."""
+    from mm_amx_amd import packed_io
+    w = wl.decode_gemv_w8(M=4, K=512, N=200, seed=77)
+    packed = mx.repack_b(dev(w["W"]))
+    path = str(tmp_path / "w.safetensors")
+    packed_io.save_packed(path, packed, "int8", w["K"], w["N"], scales=dev(w["scale"]), extra={"name": "ffn_up"})
+    got = packed_io.load_packed(path)
+    assert got["dtype"] == "int8" and (got["K"], got["N"]) == (w["K"], w["N"]) and got["extra"] == {"name": "ffn_up"}
+    assert torch.equal(got["packed"], packed)
+    y = torch.zeros((4, w["N"]), dtype=torch.bfloat16, device="cuda")
+    mx.gemm(dev_bf16(w["x"]), got["packed"], w["N"], mx.Epilogue(y, mx.PP_DEQUANT, deq_scale_per_oc=got["scales"]), b_dtype=mx.I8)
+    assert np.array_equal(host_bits(y), po.gemv_w8(w["x"], w["W"], w["scale"]))
+    with pytest.raises(mx.MmxError):
+        packed_io.save_packed(path, packed[:-1], "int8", w["K"], w["N"])
