@@ -2,9 +2,11 @@
 //
 // Stands in for the large-M paths of amx_kernel::Matmul::operator()
 // (include/kernels_amx.hpp:1255-1313): the AMX 2x2 register blocking of 16x16 tiles becomes a
-// 2x2 grid of wavefronts, each owning a (BM/2)x(BN/2) block of 32x32 MFMA accumulators; the
-// per-32x32-block post-op through an L1 scratch tile (:1290-1294) becomes an epilogue applied
-// to the accumulators in registers and staged through LDS only to make the stores row-contiguous.
+// grid of four wavefronts (2x2, or 4x1 for the 64-column tile), each owning a block of 32x32 MFMA
+// accumulators; the per-32x32-block post-op through an L1 scratch tile (:1290-1294) becomes an
+// epilogue applied to the accumulators in registers: the weights are the first MFMA operand, so a
+// lane holds runs of four consecutive columns of one output row, and a swap between the wave's
+// halves turns them into 16 consecutive columns stored with 16-byte stores.
 //
 // Data movement per k-iteration (128 bytes of K per row: 64 bf16 or 128 int8):
 //   A  [BM rows x 128 B]  row-major in HBM -> LDS rows of 128 B, 16-byte chunks XOR-swizzled by
