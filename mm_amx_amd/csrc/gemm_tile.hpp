@@ -114,10 +114,12 @@ __device__ __forceinline__ u32x4 load_a_chunk_masked(const char* rowptr, int kby
 // LDS ring of the hand-scheduled pipeline: R half-stages of (BM + BN) rows x 64 bytes.
 template <int BM, int BN>
 struct Ring {
-    static constexpr int HS = (BM + BN) * 64;  // bytes per half-stage
-    static constexpr int AH = BM * 64;         // A part of a half-stage
-    static constexpr int R = (5 * HS <= 160 * 1024 - 4096) ? 5 : 4;
-    static constexpr int BYTES = R * HS;
+    static constexpr int A_ST = BM * 128;  // A: one stage = 128 bytes of K per row (whole cache lines)
+    static constexpr int BH = BN * 64;     // B: one half-stage = 64 bytes of K per column (two fragments per panel)
+    static constexpr int RA = 3;           // A stages in LDS
+    static constexpr int R = (RA * A_ST + 4 * BH <= 156 * 1024) ? 4 : 3;  // B half-stages in LDS (R <= 2 RA - 2)
+    static constexpr int B0 = RA * A_ST;   // the B ring follows the A ring
+    static constexpr int BYTES = B0 + R * BH;
 };
 
 template <typename TIn, int BM, int BN, int MODE, typename TOut>
@@ -223,34 +225,40 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         // drains into the LDS / address FIFOs.  So every MFMA is followed by at most one LDS read (for
         // the next k-step) and one HBM->LDS load, and the order is pinned.
         //
-        // LDS is a ring of R half-stages (64 bytes of K per row = two k-steps each).  While half-stage
-        // h is multiplied, the loads of half-stages h+1 .. h+R-1 are in flight: (R-1) x 768 MFMA
-        // cycles of prefetch distance, enough to cover an HBM miss.  One workgroup barrier per
-        // half-stage; it waits only for the loads of the NEXT half-stage (s_waitcnt vmcnt(N) with the
-        // younger loads still outstanding).
+        // A half-stage is 64 bytes of K per row = two k-steps.  B lives in a ring of R half-stage slots
+        // (two 1 KiB fragments per panel).  A lives in a ring of RA stage slots of 128 bytes per row: an
+        // A row is fetched in whole 128-byte cache lines, because the L1 cannot keep half a line until
+        // the next half-stage wants it and the L2 -> L1 path, not latency, is what limits this loop
+        // (with 64-byte pieces every A line crosses it twice).  The loads belonging to half-stage w
+        // ("window" w) are the B chunks of half-stage w and, of A, the rows-half (w+1)&1 of stage
+        // (w+1)>>1 - so both halves of a stage are complete when its first half-stage starts.
+        // While half-stage h is multiplied the windows h+1 .. h+R-1 are in flight.  One workgroup
+        // barrier per half-stage; it waits only for window h+1 (s_waitcnt vmcnt(N), the younger loads
+        // stay outstanding; loads return in order).
         using RG = Ring<BM, BN>;
-        constexpr int R = RG::R, HS = RG::HS, AH = RG::AH;
-        constexpr int A_IT2 = BM / 64, B_IT2 = BN / 64;   // 16-byte chunks per thread per half-stage
+        constexpr int R = RG::R, RA = RG::RA, BH = RG::BH, A_ST = RG::A_ST, B0 = RG::B0;
+        constexpr int A_IT2 = BM / 64, B_IT2 = BN / 64;   // 16-byte chunks per thread per window
         constexpr int MN = MI * NJ;                       // MFMAs per k-step
-        constexpr int NL = A_IT2 + B_IT2;                 // HBM->LDS loads per thread per half-stage
+        constexpr int NL = A_IT2 + B_IT2;                 // HBM->LDS loads per thread per window
         constexpr int H = (NL + 1) / 2;                   // issued in two groups, one load per MFMA slot
         constexpr int RPS = (MI + NJ + MN - 1) / MN;      // LDS reads per MFMA slot (1 unless the wave tile is tiny)
         static_assert(H <= MN, "not enough MFMA slots to spread the loads over");
-        static_assert((R - 2) * NL <= 63, "vmcnt is a 6-bit counter");
+        static_assert((R - 2) * NL + H <= 63, "vmcnt is a 6-bit counter");
+        static_assert(R >= 3 && R <= 2 * RA - 2, "an A stage slot must be free again when its next user is loaded");
 
-        // 64-byte rows: the 16-byte chunk c of row r sits at slot c ^ f(r), f chosen so that the 32 rows
-        // an MFMA operand touches spread over all banks whether 8 or 16 lanes are served per cycle
-        const auto swz = [](int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); };
-
-        uint32_t aoff[A_IT2], boff[B_IT2];
+        // A in LDS: rows of 128 bytes; the 16-byte chunk c of row r sits at position c ^ ((r >> 1) & 7), so
+        // the 16 rows x 16 bytes that one LDS cycle serves for an MFMA operand fall into 16 different
+        // bank groups.  A load instruction covers 8 rows x 128 bytes: lane -> (row, position).
+        uint32_t aoff[2][A_IT2], boff[B_IT2];
 #pragma unroll
-        for (int it = 0; it < A_IT2; it++) {
-            const int c = it * 256 + tid;
-            const int row = c >> 2, slot = c & 3;
-            int grow = m0 + row;
-            grow = grow < g.M ? grow : g.M - 1;
-            aoff[it] = (uint32_t)grow * (uint32_t)g.lda + (uint32_t)((slot ^ swz(row)) * 16);
-        }
+        for (int half = 0; half < 2; half++)
+#pragma unroll
+            for (int it = 0; it < A_IT2; it++) {
+                const int row = half * (BM / 2) + it * 32 + (tid >> 3);
+                int grow = m0 + row;
+                grow = grow < g.M ? grow : g.M - 1;
+                aoff[half][it] = (uint32_t)grow * (uint32_t)g.lda + (uint32_t)(((tid & 7) ^ ((tid >> 4) & 7)) * 16);
+            }
 #pragma unroll
         for (int it = 0; it < B_IT2; it++) {
             const int c = it * 256 + tid;
@@ -261,90 +269,115 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         const char* const b_base = g.Bp + (int64_t)panel0 * g.panel_stride;
         const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(
             (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)(smem + wave * 1024));
-        const int last_hs = 2 * g.nk - 1;
+        const int last_hs = 2 * g.nk - 1, last_st = g.nk - 1;
 
-        // load number q of half-stage hs into ring slot `buf` (B chunks first, then A chunks)
-        auto dma = [&](int q, int hs, int buf) {
-            hs = hs < last_hs ? hs : last_hs;  // past the end: re-fetch the last one into a free slot
+        // load number q of window w (B chunks first, then A rounds of 32 rows) into B slot bslot / A slot aslot;
+        // HALF must be (w + 1) & 1.  Past the end the last data are fetched again, into slots that are free.
+        auto dma = [&](int q, auto half_c, int w, int bslot, int aslot) {
+            constexpr int HALF = decltype(half_c)::value;
             uint32_t m0v, off;
             const char* base;
             if (q < B_IT2) {
-                m0v = lds_wave + buf * HS + AH + q * 4096;
+                const int hs = w < last_hs ? w : last_hs;
+                m0v = lds_wave + B0 + bslot * BH + q * 4096;
                 off = boff[q];
                 base = b_base + (int64_t)hs * 2048;
             } else {
-                m0v = lds_wave + buf * HS + (q - B_IT2) * 4096;
-                off = aoff[q - B_IT2];
-                base = g.A + (int64_t)hs * 64;
+                int st = (w + 1) >> 1;
+                st = st < last_st ? st : last_st;
+                m0v = lds_wave + aslot * A_ST + HALF * (BM / 2) * 128 + (q - B_IT2) * 4096;
+                off = aoff[HALF][q - B_IT2];
+                base = g.A + (int64_t)st * 128;
             }
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                          :
                          : "s"(m0v), "v"(off), "s"(base)
                          : "memory");
         };
-        const int a_row_off = (wm * WM + l32) * 64;
-        const int a_swz = swz(l32);
-        const int b_frag_off = AH + wn * NJ * 2 * 1024 + lane * 16;
+        // A operand of k-step s (0..3 within the stage): 16 bytes at position (2 s + g32) ^ ((row >> 1) & 7)
+        const int a_x0 = (wm * WM + l32) * 128 + ((g32 ^ ((l32 >> 1) & 7)) * 16);
+        const int b_frag_off = B0 + wn * NJ * 2 * 1024 + lane * 16;
 
-        // one k-step: MFMAs on (ca, cb); meanwhile fill (na, nb) with k-step RS of ring slot rbuf and
-        // issue loads [Q0, Q1) of half-stage fhs into ring slot fbuf
-        auto kstep = [&](const frag (&ca)[MI], const frag (&cb)[NJ], frag (&na)[MI], frag (&nb)[NJ], int rbuf,
-                         auto rs_c, auto q0_c, auto q1_c, int fhs, int fbuf) {
-            constexpr int RS = decltype(rs_c)::value, Q0 = decltype(q0_c)::value, Q1 = decltype(q1_c)::value;
-            const char* sA = smem + rbuf * HS + a_row_off + (((2 * RS + g32) ^ a_swz) * 16);
-            const char* sB = smem + rbuf * HS + b_frag_off + RS * 1024;
+        // one k-step: MFMAs on (ca, cb); meanwhile fill (na, nb) from sA / sB and issue loads [Q0, Q1) of window w
+        auto kstep = [&](const frag (&ca)[MI], const frag (&cb)[NJ], frag (&na)[MI], frag (&nb)[NJ], const char* sA,
+                         const char* sB, auto q0_c, auto q1_c, auto half_c, int w, int bslot, int aslot) {
+            constexpr int Q0 = decltype(q0_c)::value, Q1 = decltype(q1_c)::value;
 #pragma unroll
             for (int t = 0; t < MN; t++) {
                 acc[t / NJ][t % NJ] = MF::run(cb[t % NJ], ca[t / NJ], acc[t / NJ][t % NJ]);
 #pragma unroll
                 for (int rd = t * RPS; rd < (t + 1) * RPS; rd++) {
                     if (rd < NJ) nb[rd] = *reinterpret_cast<const frag*>(sB + rd * 2 * 1024);
-                    else if (rd < NJ + MI) na[rd - NJ] = *reinterpret_cast<const frag*>(sA + (rd - NJ) * 32 * 64);
+                    else if (rd < NJ + MI) na[rd - NJ] = *reinterpret_cast<const frag*>(sA + (rd - NJ) * 32 * 128);
                 }
-                if (Q0 + t < Q1) dma(Q0 + t, fhs, fbuf);
+                if (Q0 + t < Q1) dma(Q0 + t, half_c, w, bslot, aslot);
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
         using std::integral_constant;
         typedef integral_constant<int, 0> c0;
-        typedef integral_constant<int, 1> c1;
         typedef integral_constant<int, H> cH;
         typedef integral_constant<int, NL> cNL;
 
-        // prologue: half-stages 0 .. R-2 completely, and the first group of half-stage R-1
+        // prologue: the first rows-half of stage 0 (it belongs to no window), windows 0 .. R-2 completely,
+        // and the first group of window R-1
 #pragma unroll
-        for (int hs = 0; hs < R - 1; hs++)
+        for (int it = 0; it < A_IT2; it++) dma(B_IT2 + it, c0{}, -1, 0, 0);
+        static_for<0, R - 1>([&](auto w_c) {
+            constexpr int W = decltype(w_c)::value;
 #pragma unroll
-            for (int q = 0; q < NL; q++) dma(q, hs, hs);
+            for (int q = 0; q < NL; q++) dma(q, integral_constant<int, (W + 1) & 1>{}, W, W, ((W + 1) >> 1) % RA);
+        });
 #pragma unroll
-        for (int q = 0; q < H; q++) dma(q, R - 1, R - 1);
-        asm volatile("s_waitcnt vmcnt(%0)" : : "n"((R - 2) * NL + H) : "memory");  // half-stage 0 has landed
+        for (int q = 0; q < H; q++) dma(q, integral_constant<int, R & 1>{}, R - 1, R - 1, (R >> 1) % RA);
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"((R - 2) * NL + H) : "memory");  // window 0 and all before it have landed
         __syncthreads();
         {
-            const char* sA = smem + a_row_off + ((g32 ^ a_swz) * 16);
+            const char* sA = smem + a_x0;
             const char* sB = smem + b_frag_off;
 #pragma unroll
-            for (int i = 0; i < MI; i++) fa[0][i] = *reinterpret_cast<const frag*>(sA + i * 32 * 64);
+            for (int i = 0; i < MI; i++) fa[0][i] = *reinterpret_cast<const frag*>(sA + i * 32 * 128);
 #pragma unroll
             for (int j = 0; j < NJ; j++) fb[0][j] = *reinterpret_cast<const frag*>(sB + j * 2 * 1024);
         }
         __builtin_amdgcn_sched_barrier(0);
 
-        int buf = 0;  // ring slot of the half-stage being multiplied
-        for (int hs = 0; hs <= last_hs; hs++) {
-            const int nbuf = buf + 1 < R ? buf + 1 : 0;           // slot of half-stage hs+1
-            const int pbuf = buf == 0 ? R - 1 : buf - 1;          // slot of hs-1 == slot of hs+R-1
-            // k-step 0: read k-step 1 of this half-stage; second group of the loads of half-stage hs+R-1
-            kstep(fa[0], fb[0], fa[1], fb[1], buf, c1{}, cH{}, cNL{}, hs + R - 1, pbuf);
-            // every wave now holds all of half-stage hs in registers; half-stage hs+1 must have landed,
-            // the (R-2) younger ones may still be in flight
+        // half-stage h = 2 st + PAR: A stage slot as (the next stage's slot is nas), B slot bs
+        auto half_stage = [&](auto par_c, int h, int as, int nas, int bs) {
+            constexpr int PAR = decltype(par_c)::value;
+            const int nbs = bs + 1 < R ? bs + 1 : 0;   // slot of half-stage h+1
+            const int pbs = bs == 0 ? R - 1 : bs - 1;  // slot of h-1 == slot of h+R-1
+            // k-step 0: read k-step 1 of this half-stage; second group of the loads of window h+R-1
+            {
+                int as2 = as + ((PAR + R) >> 1);
+                as2 = as2 >= RA ? as2 - RA : as2;
+                kstep(fa[0], fb[0], fa[1], fb[1], smem + as * A_ST + (a_x0 ^ ((4 * PAR + 2) * 16)),
+                      smem + bs * BH + b_frag_off + 1024, cH{}, cNL{}, integral_constant<int, (PAR + R) & 1>{},
+                      h + R - 1, pbs, as2);
+            }
+            // every wave now holds all of half-stage h in registers; window h+1 must have landed, the
+            // (R-2) younger ones may still be in flight
             asm volatile("s_waitcnt vmcnt(%0)" : : "n"((R - 2) * NL) : "memory");
             __syncthreads();
             __builtin_amdgcn_sched_barrier(0);
-            // k-step 1: read k-step 0 of the next half-stage; first group of the loads of half-stage
-            // hs+R goes into the slot this half-stage has just vacated
-            kstep(fa[1], fb[1], fa[0], fb[0], nbuf, c0{}, c0{}, cH{}, hs + R, buf);
-            buf = nbuf;
+            // k-step 1: read k-step 0 of the next half-stage; first group of the loads of window h+R; its
+            // B chunks go into the slot this half-stage has just vacated
+            {
+                int as1 = as + ((PAR + R + 1) >> 1);
+                as1 = as1 >= RA ? as1 - RA : as1;
+                const char* sA = PAR == 0 ? smem + as * A_ST + (a_x0 ^ (4 * 16)) : smem + nas * A_ST + a_x0;
+                kstep(fa[1], fb[1], fa[0], fb[0], sA, smem + nbs * BH + b_frag_off, c0{}, cH{},
+                      integral_constant<int, (PAR + R + 1) & 1>{}, h + R, bs, as1);
+            }
+        };
+        int as = 0, bs = 0;
+        for (int st = 0; st <= last_st; st++) {
+            const int nas = as + 1 < RA ? as + 1 : 0;
+            half_stage(integral_constant<int, 0>{}, 2 * st, as, nas, bs);
+            bs = bs + 1 < R ? bs + 1 : 0;
+            half_stage(integral_constant<int, 1>{}, 2 * st + 1, as, nas, bs);
+            bs = bs + 1 < R ? bs + 1 : 0;
+            as = nas;
         }
         asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // the re-fetched slots past the end must land before the wave ends
     } else {
