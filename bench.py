@@ -148,7 +148,8 @@ def main():
         extra = {}
 
         def avg_ms(Ain, packs, Nn, epi, iters, **kw):
-            mx.time_gemm(Ain, packs, Nn, epi, max(3, iters // 10), **kw)
+            # a new shape needs about a hundred launches before its time settles (fresh buffers, clocks)
+            mx.time_gemm(Ain, packs, Nn, epi, max(100, iters // 2), **kw)
             return mx.time_gemm(Ain, packs, Nn, epi, iters, **kw)
 
         # bf16 256^3, fp32 out, no post-op (launch-latency bound; reported, not a roofline case)
@@ -165,7 +166,7 @@ def main():
             ws = wl.ffn_up_bias_gelu(M=Ms)
             As = dev_bf16(ws["A"])
             Cs = torch.zeros((Ms, N), dtype=torch.bfloat16, device="cuda")
-            ms = avg_ms(As, [Bp], N, mx.Epilogue(Cs, mx.PP_BIAS | mx.PP_GELU, bias=bias), 30)
+            ms = avg_ms(As, [Bp], N, mx.Epilogue(Cs, mx.PP_BIAS | mx.PP_GELU, bias=bias), 100)
             sweep[str(Ms)] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * Ms * N * K / ms / 1e9, 1),
                               "kernel": mx.last_kernel()}
             del As, Cs
@@ -207,16 +208,16 @@ def main():
         for Mm in (1, 2048):
             xm = dev_bf16(wm["x"][:Mm])
             ym = torch.zeros((Mm, wm["K"]), dtype=torch.bfloat16, device="cuda")
-            for _ in range(3):
+            for _ in range(60):
                 op.run(xm, ym)
             torch.cuda.synchronize()
             a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             a0.record()
-            for _ in range(20):
+            for _ in range(60):
                 op.run(xm, ym)
             a1.record()
             torch.cuda.synchronize()
-            ms = a0.elapsed_time(a1) / 20
+            ms = a0.elapsed_time(a1) / 60
             fl = 6.0 * Mm * wm["K"] * wm["N"]
             mlp[str(Mm)] = {"us": round(ms * 1e3, 1), "tflops": round(fl / ms / 1e9, 1),
                             "weight_GBps": round(3.0 * wm["K"] * wm["N"] * 2 / ms / 1e6, 0)}

@@ -9,14 +9,15 @@
 // halves turns them into 16 consecutive columns stored with 16-byte stores.
 //
 // Data movement per k-iteration (128 bytes of K per row: 64 bf16 or 128 int8):
-//   A  [BM rows x 128 B]  row-major in HBM -> LDS rows of 128 B, 16-byte chunks XOR-swizzled by
-//      (row & 7) so that the 32 rows an MFMA operand needs hit all LDS banks;
+//   A  [BM rows x 128 B]  row-major in HBM -> LDS rows of 128 B, 16-byte chunks XOR-swizzled by a
+//      function of the row so that the rows an MFMA operand needs spread over the LDS banks;
 //   B  [BN/32 panels x 4 fragments x 1 KiB] already in MFMA operand order in HBM -> copied
 //      verbatim, every ds_read_b128 of a fragment is lane-contiguous.
 // Three ways of bringing the tiles into LDS (template parameter MODE):
 //   MODE 2  the product path: global_load_lds_dwordx4 (HBM -> LDS without passing through VGPRs)
-//           issued from inline asm into a ring of half-stages, hand-scheduled against the MFMAs
-//           (see the comment at the pipeline);
+//           issued from inline asm into rings of LDS slots (A in whole 128-byte lines per row, B in
+//           half-stages of two fragments per panel), hand-scheduled against the MFMAs (see the
+//           comment at the pipeline);
 //   MODE 0  global -> VGPR -> LDS with 16-byte loads, two LDS stages, rows past M clamped to the
 //           last row: the fallback when A or the packed weights are too large for the 32-bit
 //           offsets MODE 2 addresses with, and a tested alternative;
@@ -271,65 +272,129 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)(smem + wave * 1024));
         const int last_hs = 2 * g.nk - 1, last_st = g.nk - 1;
 
-        // load number q of window w (B chunks first, then A rounds of 32 rows) into B slot bslot / A slot aslot;
-        // HALF must be (w + 1) & 1.  Past the end the last data are fetched again, into slots that are free.
-        auto dma = [&](int q, auto half_c, int w, int bslot, int aslot) {
-            constexpr int HALF = decltype(half_c)::value;
-            uint32_t m0v, off;
-            const char* base;
-            if (q < B_IT2) {
-                const int hs = w < last_hs ? w : last_hs;
-                m0v = lds_wave + B0 + bslot * BH + q * 4096;
-                off = boff[q];
-                base = b_base + (int64_t)hs * 2048;
-            } else {
-                int st = (w + 1) >> 1;
-                st = st < last_st ? st : last_st;
-                m0v = lds_wave + aslot * A_ST + HALF * (BM / 2) * 128 + (q - B_IT2) * 4096;
-                off = aoff[HALF][q - B_IT2];
-                base = g.A + (int64_t)st * 128;
-            }
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                         :
-                         : "s"(m0v), "v"(off), "s"(base)
-                         : "memory");
-        };
-        // A operand of k-step s (0..3 within the stage): 16 bytes at position (2 s + g32) ^ ((row >> 1) & 7)
-        const int a_x0 = (wm * WM + l32) * 128 + ((g32 ^ ((l32 >> 1) & 7)) * 16);
-        const int b_frag_off = B0 + wn * NJ * 2 * 1024 + lane * 16;
-
-        // one k-step: MFMAs on (ca, cb); meanwhile fill (na, nb) from sA / sB and issue loads [Q0, Q1) of window w
-        auto kstep = [&](const frag (&ca)[MI], const frag (&cb)[NJ], frag (&na)[MI], frag (&nb)[NJ], const char* sA,
-                         const char* sB, auto q0_c, auto q1_c, auto half_c, int w, int bslot, int aslot) {
-            constexpr int Q0 = decltype(q0_c)::value, Q1 = decltype(q1_c)::value;
-#pragma unroll
-            for (int t = 0; t < MN; t++) {
-                acc[t / NJ][t % NJ] = MF::run(cb[t % NJ], ca[t / NJ], acc[t / NJ][t % NJ]);
-#pragma unroll
-                for (int rd = t * RPS; rd < (t + 1) * RPS; rd++) {
-                    if (rd < NJ) nb[rd] = *reinterpret_cast<const frag*>(sB + rd * 2 * 1024);
-                    else if (rd < NJ + MI) na[rd - NJ] = *reinterpret_cast<const frag*>(sA + (rd - NJ) * 32 * 128);
-                }
-                if (Q0 + t < Q1) dma(Q0 + t, half_c, w, bslot, aslot);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        };
         using std::integral_constant;
         typedef integral_constant<int, 0> c0;
+        typedef integral_constant<int, 1> c1;
         typedef integral_constant<int, H> cH;
         typedef integral_constant<int, NL> cNL;
 
+        const int a_x0 = (wm * WM + l32) * 128 + ((g32 ^ ((l32 >> 1) & 7)) * 16);
+        const int b_frag_off = B0 + wn * NJ * 2 * 1024 + lane * 16;
+
+        // Everything a k-step needs besides its operands: where its LDS reads come from and where its
+        // loads go.  A wave issues in order and an MFMA slot is 32 cycles = about six instructions, so
+        // these values are computed, a few per slot, in the idle slots of the PREVIOUS k-step (and pinned
+        // there: left to the compiler the whole address arithmetic lands in front of the first load of the
+        // k-step, which holds up the MFMAs behind it by several slots).
+        struct KParams {
+            uint32_t m0B, m0A;   // LDS destinations of this wave's B chunk 0 / A round 0
+            const char* srcB;    // global sources (the lane offsets are boff / aoff)
+            const char* srcA;
+            uint32_t rdA, rdB;   // LDS byte offsets of this lane's first A / B fragment
+        };
+        // k-step KS (0/1) of half-stage h = 2 st + PAR; as/nas = A slot of this / the next stage, bs = B slot.
+        // k-step 0 issues the second group of window h+R-1, k-step 1 the first group of window h+R (its B
+        // chunks go into the slot this half-stage has just vacated).  Of A, window w carries the rows-half
+        // (w+1)&1 of stage (w+1)>>1.  Past the end the last data are fetched again, into slots that are free.
+        auto prepare = [&](auto part_c, KParams& n, auto par_c, auto ks_c, int h, int as, int nas, int bs) {
+            constexpr int PART = decltype(part_c)::value, PAR = decltype(par_c)::value, KS = decltype(ks_c)::value;
+            constexpr int HALF = (PAR + R + KS) & 1;
+            const int w = h + R - 1 + KS;
+            if constexpr (PART == 0) {
+                const int bslot = KS == 0 ? (bs == 0 ? R - 1 : bs - 1) : bs;
+                int aslot = as + ((PAR + R + KS) >> 1);
+                aslot = aslot >= RA ? aslot - RA : aslot;
+                n.m0B = lds_wave + B0 + bslot * BH;
+                n.m0A = lds_wave + aslot * A_ST + HALF * (BM / 2) * 128;
+                asm volatile("" : "+s"(n.m0B), "+s"(n.m0A));
+            } else if constexpr (PART == 1) {
+                const int hs = w < last_hs ? w : last_hs;
+                n.srcB = b_base + (int64_t)hs * 2048;
+                asm volatile("" : "+s"(n.srcB));
+            } else if constexpr (PART == 2) {
+                int st = (w + 1) >> 1;
+                st = st < last_st ? st : last_st;
+                n.srcA = g.A + (int64_t)st * 128;
+                asm volatile("" : "+s"(n.srcA));
+            } else {
+                // A operand of k-step s (0..3 within the stage): position (2 s + g32) ^ ((row >> 1) & 7) of the row
+                if constexpr (KS == 0) {  // reads k-step 1 of this half-stage
+                    n.rdA = as * A_ST + (a_x0 ^ ((4 * PAR + 2) * 16));
+                    n.rdB = bs * BH + b_frag_off + 1024;
+                } else {                  // reads k-step 0 of the next half-stage
+                    const int nbs = bs + 1 < R ? bs + 1 : 0;
+                    n.rdA = PAR == 0 ? as * A_ST + (a_x0 ^ (4 * 16)) : nas * A_ST + a_x0;
+                    n.rdB = nbs * BH + b_frag_off;
+                }
+                asm volatile("" : "+v"(n.rdA), "+v"(n.rdB));
+            }
+        };
+        // load number Q of a window: B chunks first, then A rounds of 32 rows
+        auto dma = [&](auto q_c, auto half_c, const KParams& kp) {
+            constexpr int Q = decltype(q_c)::value, HALF = decltype(half_c)::value;
+            if constexpr (Q < B_IT2) {
+                const uint32_t off = boff[Q];
+                asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                             :
+                             : "s"(kp.m0B), "v"(off), "s"(kp.srcB), "n"(Q * 4096)
+                             : "memory", "scc");
+            } else {
+                const uint32_t off = aoff[HALF][Q - B_IT2];
+                asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                             :
+                             : "s"(kp.m0A), "v"(off), "s"(kp.srcA), "n"((Q - B_IT2) * 4096)
+                             : "memory", "scc");
+            }
+        };
+
+        // one k-step: MFMAs on (ca, cb); meanwhile fill (na, nb) for the next k-step, issue loads [Q0, Q1)
+        // and let `prep(part)` work out the parameters of the next k-step in the last slots
+        auto kstep = [&](const frag (&ca)[MI], const frag (&cb)[NJ], frag (&na)[MI], frag (&nb)[NJ], const KParams& kp,
+                         auto q0_c, auto q1_c, auto half_c, auto&& prep) {
+            constexpr int Q0 = decltype(q0_c)::value, Q1 = decltype(q1_c)::value;
+            const char* sA = smem + kp.rdA;
+            const char* sB = smem + kp.rdB;
+            static_for<0, MN>([&](auto t_c) {
+                constexpr int t = decltype(t_c)::value;
+                acc[t / NJ][t % NJ] = MF::run(cb[t % NJ], ca[t / NJ], acc[t / NJ][t % NJ]);
+                static_for<t * RPS, (t + 1) * RPS>([&](auto rd_c) {
+                    constexpr int rd = decltype(rd_c)::value;
+                    if constexpr (rd < NJ) nb[rd] = *reinterpret_cast<const frag*>(sB + rd * 2 * 1024);
+                    else if constexpr (rd < NJ + MI) na[rd - NJ] = *reinterpret_cast<const frag*>(sA + (rd - NJ) * 32 * 128);
+                });
+                if constexpr (Q0 + t < Q1) dma(integral_constant<int, Q0 + t>{}, half_c, kp);
+                // four parts of the next k-step's parameters in the last four slots (all in the last one
+                // where a k-step has fewer)
+                static_for<0, 4>([&](auto part_c) {
+                    constexpr int part = decltype(part_c)::value;
+                    constexpr int slot = MN >= 4 ? MN - 4 + part : MN - 1;
+                    if constexpr (slot == t) prep(part_c);
+                });
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        };
         // prologue: the first rows-half of stage 0 (it belongs to no window), windows 0 .. R-2 completely,
         // and the first group of window R-1
-#pragma unroll
-        for (int it = 0; it < A_IT2; it++) dma(B_IT2 + it, c0{}, -1, 0, 0);
-        static_for<0, R - 1>([&](auto w_c) {
-            constexpr int W = decltype(w_c)::value;
-#pragma unroll
-            for (int q = 0; q < NL; q++) dma(q, integral_constant<int, (W + 1) & 1>{}, W, W, ((W + 1) >> 1) % RA);
-        });
-#pragma unroll
-        for (int q = 0; q < H; q++) dma(q, integral_constant<int, R & 1>{}, R - 1, R - 1, (R >> 1) % RA);
+        {
+            KParams kp;
+            kp.m0A = lds_wave;
+            kp.srcA = g.A;
+            static_for<0, A_IT2>([&](auto it_c) { dma(integral_constant<int, B_IT2 + decltype(it_c)::value>{}, c0{}, kp); });
+            static_for<0, R>([&](auto w_c) {
+                constexpr int W = decltype(w_c)::value;
+                constexpr int HALF = (W + 1) & 1;
+                const int hs = W < last_hs ? W : last_hs;
+                int st = (W + 1) >> 1;
+                st = st < last_st ? st : last_st;
+                kp.m0B = lds_wave + B0 + W * BH;
+                kp.m0A = lds_wave + (((W + 1) >> 1) % RA) * A_ST + HALF * (BM / 2) * 128;
+                kp.srcB = b_base + (int64_t)hs * 2048;
+                kp.srcA = g.A + (int64_t)st * 128;
+                static_for<0, (W < R - 1 ? NL : H)>([&](auto q_c) { dma(q_c, integral_constant<int, HALF>{}, kp); });
+            });
+        }
+        KParams kpa, kpb;  // parameters of the k-step being executed / of the one after it
+        static_for<0, 4>([&](auto part_c) { prepare(part_c, kpa, c0{}, c0{}, 0, 0, RA > 1 ? 1 : 0, 0); });
         asm volatile("s_waitcnt vmcnt(%0)" : : "n"((R - 2) * NL + H) : "memory");  // window 0 and all before it have landed
         __syncthreads();
         {
@@ -342,40 +407,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         }
         __builtin_amdgcn_sched_barrier(0);
 
-        // half-stage h = 2 st + PAR: A stage slot as (the next stage's slot is nas), B slot bs
+        // half-stage h = 2 st + PAR: A stage slot as (the next stage's slot is nas), B slot bs; on entry kpa
+        // describes its k-step 0, on exit k-step 0 of half-stage h+1
         auto half_stage = [&](auto par_c, int h, int as, int nas, int bs) {
             constexpr int PAR = decltype(par_c)::value;
-            const int nbs = bs + 1 < R ? bs + 1 : 0;   // slot of half-stage h+1
-            const int pbs = bs == 0 ? R - 1 : bs - 1;  // slot of h-1 == slot of h+R-1
             // k-step 0: read k-step 1 of this half-stage; second group of the loads of window h+R-1
-            {
-                int as2 = as + ((PAR + R) >> 1);
-                as2 = as2 >= RA ? as2 - RA : as2;
-                kstep(fa[0], fb[0], fa[1], fb[1], smem + as * A_ST + (a_x0 ^ ((4 * PAR + 2) * 16)),
-                      smem + bs * BH + b_frag_off + 1024, cH{}, cNL{}, integral_constant<int, (PAR + R) & 1>{},
-                      h + R - 1, pbs, as2);
-            }
+            kstep(fa[0], fb[0], fa[1], fb[1], kpa, cH{}, cNL{}, integral_constant<int, (PAR + R) & 1>{},
+                  [&](auto part_c) { prepare(part_c, kpb, par_c, c1{}, h, as, nas, bs); });
             // every wave now holds all of half-stage h in registers; window h+1 must have landed, the
             // (R-2) younger ones may still be in flight
             asm volatile("s_waitcnt vmcnt(%0)" : : "n"((R - 2) * NL) : "memory");
             __syncthreads();
             __builtin_amdgcn_sched_barrier(0);
-            // k-step 1: read k-step 0 of the next half-stage; first group of the loads of window h+R; its
-            // B chunks go into the slot this half-stage has just vacated
-            {
-                int as1 = as + ((PAR + R + 1) >> 1);
-                as1 = as1 >= RA ? as1 - RA : as1;
-                const char* sA = PAR == 0 ? smem + as * A_ST + (a_x0 ^ (4 * 16)) : smem + nas * A_ST + a_x0;
-                kstep(fa[1], fb[1], fa[0], fb[0], sA, smem + nbs * BH + b_frag_off, c0{}, cH{},
-                      integral_constant<int, (PAR + R + 1) & 1>{}, h + R, bs, as1);
+            // k-step 1: read k-step 0 of the next half-stage; first group of the loads of window h+R
+            const int nbs = bs + 1 < R ? bs + 1 : 0;
+            int as_n = as, nas_n = nas;  // slots as half-stage h+1 sees them
+            if constexpr (PAR == 1) {
+                as_n = nas;
+                nas_n = nas + 1 < RA ? nas + 1 : 0;
             }
+            kstep(fa[1], fb[1], fa[0], fb[0], kpb, c0{}, cH{}, integral_constant<int, (PAR + R + 1) & 1>{},
+                  [&](auto part_c) { prepare(part_c, kpa, integral_constant<int, 1 - PAR>{}, c0{}, h + 1, as_n, nas_n, nbs); });
         };
         int as = 0, bs = 0;
         for (int st = 0; st <= last_st; st++) {
             const int nas = as + 1 < RA ? as + 1 : 0;
-            half_stage(integral_constant<int, 0>{}, 2 * st, as, nas, bs);
+            half_stage(c0{}, 2 * st, as, nas, bs);
             bs = bs + 1 < R ? bs + 1 : 0;
-            half_stage(integral_constant<int, 1>{}, 2 * st + 1, as, nas, bs);
+            half_stage(c1{}, 2 * st + 1, as, nas, bs);
             bs = bs + 1 < R ? bs + 1 : 0;
             as = nas;
         }
