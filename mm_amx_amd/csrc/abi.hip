@@ -49,8 +49,10 @@ struct TileCfg {
 };
 static TileCfg g_forced = {0, 0};
 static int g_load_mode = 2;
+static int g_decode_halves = -1;
 TileCfg forced_tile() { return g_forced; }
 int load_mode() { return g_load_mode; }
+int decode_halves() { return g_decode_halves; }
 
 static int elesz_of(int dtype) { return dtype == MMX_BF16 ? 2 : dtype == MMX_I8 ? 1 : 0; }
 
@@ -237,6 +239,11 @@ int mmx_set_option(const char* name, int value) {
     if (name && !strcmp(name, "load_mode")) {
         if (value != 0 && value != 2) return set_error(MMX_E_INVALID, "mmx_set_option: load_mode is 0 or 2");
         g_load_mode = value;
+        return MMX_OK;
+    }
+    if (name && !strcmp(name, "decode_halves")) {
+        if (value < -1 || value > 1) return set_error(MMX_E_INVALID, "mmx_set_option: decode_halves is -1, 0 or 1");
+        g_decode_halves = value;
         return MMX_OK;
     }
     return set_error(MMX_E_INVALID, "mmx_set_option: unknown option");

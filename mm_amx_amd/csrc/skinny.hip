@@ -565,6 +565,193 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     skinny_finish<NP>(s, red, panel_first, tid, fin);
 }
 
+// Half-panel variant of the streaming kernel for 1-2 rows of x.  A list of 32-column panels that is only 1-2
+// per CU long leaves some CUs with twice the work of others (or idle), and how fast one CU can pull
+// weights in is what bounds this kernel.  Here a workgroup (four waves) multiplies HALF a panel
+// (16 columns, blockIdx.x = 2 * panel group + half): twice as many, half as large units, all resident at once.
+// A load covers the half-panel's part of TWO consecutive fragments (lanes 0-15/32-47: fragment 2u, lanes
+// 16-31/48-63: fragment 2u+1), so every lane still fetches its own 16 bytes.  As an MFMA operand that is 16
+// columns x two different k-ranges, so each load is multiplied twice, once with the x of either fragment,
+// into two accumulators: rows 0-15 of the first and rows 16-31 of the second are the two partial sums of
+// the 16 columns (the other rows are never looked at).  K * sizeof(T) is a multiple of 128 on this path,
+// so a panel has an even number of fragments.
+template <bool W8, int NP, bool ONE, int U>  // U: loads per panel per wave in flight at once (1 KiB each)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void skinny_half_kernel(const SkinnyArgs s, int zero_off) {
+    constexpr int NW = 4;
+    __shared__ float red[NW][NP][16][64];
+    extern __shared__ __attribute__((aligned(1024))) char xs[];  // [M][K] bf16, then at zero_off a row of zeros
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, g32 = lane >> 5;
+    const int half = blockIdx.x & 1;
+    const int panel_first = (s.n0 >> 5) + (int)(blockIdx.x >> 1) * NP;
+    const int panel_end = (s.n1 + 31) >> 5;
+    const int row_bytes = s.K * 2;
+    const int real_bytes = s.M * row_bytes;
+    const Epilogue& ep = s.ep;
+
+    {   // x -> LDS as in skinny_stream_kernel
+        const uint32_t lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)xs);
+        for (int off = wave * 1024; off < real_bytes; off += NW * 1024) {
+            int bo = off + lane * 16;
+            bo = bo < real_bytes ? bo : real_bytes - 16;
+            const int m = bo / row_bytes;
+            const char* src = s.x + (int64_t)m * s.ldx + (bo - m * row_bytes);
+            const uint32_t m0v = lds_base + off;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0v), "v"(src) : "memory");
+        }
+        for (int c = tid * 16; c < row_bytes; c += NW * 64 * 16) *reinterpret_cast<u32x4*>(xs + zero_off + c) = u32x4{0u, 0u, 0u, 0u};
+    }
+    // per-column operands of the post-op: thread -> (accumulator register v < 8, lane) -> column of the half-panel
+    float o_deq[2][NP], o_bias[2][NP], o_q[2][NP];
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int v = (tid + 256 * t) >> 6;
+        const int nloc = 16 * half + 8 * (v >> 2) + 4 * g32 + (v & 3);
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            const int n = ((panel_first + p) << 5) + nloc;
+            const bool ok = l32 < s.M && n < s.n1 && !(ep.steps & MMX_PP_SILU_GATE);
+            o_deq[t][p] = ep.deq;
+            o_bias[t][p] = 0.0f;
+            o_q[t][p] = ep.q;
+            if (ok && (ep.steps & MMX_PP_DEQUANT) && ep.deq_oc) o_deq[t][p] = ep.deq_oc[n];
+            if (ok && (ep.steps & MMX_PP_BIAS)) o_bias[t][p] = ep.bias[n];
+            if (ok && (ep.steps & MMX_PP_QUANT) && ep.q_oc) o_q[t][p] = ep.q_oc[n];
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    f32x16 acc[NP][2];
+#pragma unroll
+    for (int p = 0; p < NP; p++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[p][0][v] = acc[p][1][v] = 0.0f;
+
+    // wave w multiplies the fragment pairs [w*per_wave, (w+1)*per_wave); indices past the end are clamped
+    // for the load and paired with the zero row of x
+    const int npairs = s.nfrag >> 1;
+    const int per_wave = (npairs + NW - 1) / NW;
+    const int u_begin = wave * per_wave;
+    const int u_last = npairs - 1;
+    const char* wbase[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++) {
+        int panel = panel_first + p;
+        panel = (panel < panel_end && panel < s.npanels) ? panel : s.npanels - 1;  // columns past n1 are never stored
+        wbase[p] = s.Wp + (int64_t)panel * s.panel_stride + (l32 >> 4) * 1024 + (g32 * 32 + 16 * half + (l32 & 15)) * 16;
+    }
+    const char* zrow = xs + zero_off;
+    const char* xrow = l32 < s.M ? xs + l32 * row_bytes : zrow;
+    const int nbatch = (per_wave + U - 1) / U;  // same for every wave
+    u32x4 w[NP][U];
+#define MMX_REQUEST(BT, UU)                                                                                     \
+    do {                                                                                                        \
+        int u_ = u_begin + (BT) * U + (UU);                                                                     \
+        u_ = u_ < u_last ? u_ : u_last;                                                                         \
+        _Pragma("unroll") for (int p = 0; p < NP; p++)                                                          \
+            w[p][UU] = *reinterpret_cast<const u32x4*>(wbase[p] + (int64_t)u_ * 2048);                          \
+    } while (0)
+#define MMX_MULTIPLY(BT, UU)                                                                                    \
+    do {                                                                                                        \
+        const int u_ = u_begin + (BT) * U + (UU);                                                               \
+        const bool valid_ = (u_ - u_begin) < per_wave && u_ <= u_last; /* scalar */                             \
+        const int uc_ = u_ < u_last ? u_ : u_last;                                                              \
+        const char* xr_ = valid_ ? xrow : zrow;                                                                 \
+        if constexpr (W8) {                                                                                     \
+            const bf16x8 xa0_ = *reinterpret_cast<const bf16x8*>(xr_ + (64 * uc_ + 16 * g32) * 2);              \
+            const bf16x8 xa1_ = *reinterpret_cast<const bf16x8*>(xr_ + (64 * uc_ + 16 * g32 + 8) * 2);          \
+            const bf16x8 xb0_ = *reinterpret_cast<const bf16x8*>(xr_ + (64 * uc_ + 32 + 16 * g32) * 2);         \
+            const bf16x8 xb1_ = *reinterpret_cast<const bf16x8*>(xr_ + (64 * uc_ + 32 + 16 * g32 + 8) * 2);     \
+            _Pragma("unroll") for (int p = 0; p < NP; p++) {                                                    \
+                const bf16x8 lo_ = s8x8_to_bf16(w[p][UU].x, w[p][UU].y), hi_ = s8x8_to_bf16(w[p][UU].z, w[p][UU].w); \
+                acc[p][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lo_, xa0_, acc[p][0], 0, 0, 0);             \
+                acc[p][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(hi_, xa1_, acc[p][0], 0, 0, 0);             \
+                acc[p][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lo_, xb0_, acc[p][1], 0, 0, 0);             \
+                acc[p][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(hi_, xb1_, acc[p][1], 0, 0, 0);             \
+            }                                                                                                   \
+        } else {                                                                                                \
+            const bf16x8 xa_ = *reinterpret_cast<const bf16x8*>(xr_ + (32 * uc_ + 8 * g32) * 2);                \
+            const bf16x8 xb_ = *reinterpret_cast<const bf16x8*>(xr_ + (32 * uc_ + 16 + 8 * g32) * 2);           \
+            _Pragma("unroll") for (int p = 0; p < NP; p++) {                                                    \
+                acc[p][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w[p][UU]), xa_, acc[p][0], 0, 0, 0); \
+                acc[p][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w[p][UU]), xb_, acc[p][1], 0, 0, 0); \
+            }                                                                                                   \
+        }                                                                                                       \
+    } while (0)
+    {
+        // as in skinny_stream_kernel: a quarter of the first batch, then wait for x and publish it, then the rest
+        constexpr int U0 = U / 4;
+#pragma unroll
+        for (int u = 0; u < U0; u++) MMX_REQUEST(0, u);
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" : : "n"(U0 * NP) : "memory");
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = U0; u < U; u++) MMX_REQUEST(0, u);
+    }
+    if constexpr (ONE) {
+#pragma unroll
+        for (int u = 0; u < U; u++) MMX_MULTIPLY(0, u);
+    } else {
+        for (int bt = 0; bt + 1 < nbatch; bt++) {
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                MMX_MULTIPLY(bt, u);
+                MMX_REQUEST(bt + 1, u);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) MMX_MULTIPLY(nbatch - 1, u);
+    }
+#undef MMX_REQUEST
+#undef MMX_MULTIPLY
+
+    // accumulator register v of a lane is row 8 (v / 4) + 4 g32 + v % 4: rows 0-15 are v < 8
+#pragma unroll
+    for (int p = 0; p < NP; p++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) red[wave][p][v][lane] = v < 8 ? acc[p][0][v] : acc[p][1][v];
+    __syncthreads();
+
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int v = (tid + 256 * t) >> 6;
+        const int m = l32;
+        if (m >= s.M) continue;
+        const int nloc = 16 * half + 8 * (v >> 2) + 4 * g32 + (v & 3);
+        float sum[NP];
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            float a = 0.0f;
+#pragma unroll
+            for (int wv = 0; wv < NW; wv++) a += red[wv][p][v][lane] + red[wv][p][v + 8][lane];
+            sum[p] = a;
+        }
+        if (ep.steps & MMX_PP_SILU_GATE) {
+            if constexpr (NP == 2) {
+                const int n = ((panel_first >> 1) << 5) + nloc;  // output column (half width)
+                if (n < (s.n1 >> 1)) store_out(ep, m, n, silu(sum[0]) * sum[1]);
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                const int n = ((panel_first + p) << 5) + nloc;
+                if (n >= s.n1) continue;
+                float r = sum[p];
+                if (ep.steps & MMX_PP_DEQUANT) r = r * o_deq[t][p];
+                if (ep.steps & MMX_PP_BIAS) r = r + o_bias[t][p];
+                if (ep.steps & MMX_PP_GELU) r = gelu_erf_minimax(r);
+                if (ep.steps & MMX_PP_QUANT) r = r * o_q[t][p];
+                store_out(ep, m, n, r);
+            }
+        }
+    }
+}
+
+int decode_halves();
+
 int launch_skinny(bool w8, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
                   const Epilogue& ep, hipStream_t st) {
     SkinnyArgs s;
@@ -591,13 +778,29 @@ int launch_skinny(bool w8, const void* x, int64_t ldx, const void* Wp, int M, in
         if (pairs && (panels & 1)) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
         note_kernel(pairs ? "skinny_stream_bf16_gateup" : (w8 ? "skinny_stream_w8" : "skinny_stream_bf16"));
         const int per_wave = (s.nfrag + 7) / 8;
+        // Half-panel workgroups pay off for 1-2 rows of x (cheap to stage per workgroup), if all of them are
+        // resident at once (four waves each; LDS allows min(4, 160 KiB / (reduction scratch + x)) per CU) and
+        // each still has at least 128 KiB of weights to stream (measured: 64 KiB units lose more to the
+        // fixed cost of a workgroup than the better balance gains)
+        const int units = pairs ? panels / 2 : panels;
+        const int lds_wg = 16 * 1024 * (pairs ? 2 : 1) + xbytes;
+        const int wg_per_cu = (160 * 1024 / lds_wg) < 4 ? (160 * 1024 / lds_wg) : 4;
+        const int64_t unit_bytes = (int64_t)s.nfrag * 512 * (pairs ? 2 : 1);
+        const int force = decode_halves();  // -1: by the rule above, 0: never, 1: for every M <= 2 (tests pin the path with it)
+        const bool halves = M <= 2 && force != 0 && (force == 1 || (2 * units <= 256 * wg_per_cu && unit_bytes >= 128 * 1024));
+        const int per_wave_h = ((s.nfrag >> 1) + 3) / 4;
 #define MMX_STREAM(W8, NP, GRID)                                                                                     \
     do {                                                                                                             \
-        if (per_wave <= 16 / NP)                                                                                     \
+        if (halves && per_wave_h <= 16 / NP)                                                                         \
+            hipLaunchKernelGGL((skinny_half_kernel<W8, NP, true, 16 / NP>), dim3(2 * (GRID)), dim3(256), xbytes, st, s, zero_off); \
+        else if (halves) /* the rolling window holds fewer registers where two accumulator pairs need them */      \
+            hipLaunchKernelGGL((skinny_half_kernel<W8, NP, false, (NP == 2 ? 4 : (W8 ? 12 : 16))>), dim3(2 * (GRID)), dim3(256), xbytes, st, s, zero_off); \
+        else if (per_wave <= 16 / NP)                                                                                \
             hipLaunchKernelGGL((skinny_stream_kernel<W8, NP, true>), dim3(GRID), dim3(512), xbytes, st, s, zero_off); \
         else                                                                                                         \
             hipLaunchKernelGGL((skinny_stream_kernel<W8, NP, false>), dim3(GRID), dim3(512), xbytes, st, s, zero_off); \
     } while (0)
+        if (halves) note_kernel(pairs ? "skinny_half_bf16_gateup" : (w8 ? "skinny_half_w8" : "skinny_half_bf16"));
         if (pairs) MMX_STREAM(false, 2, panels / 2);
         else if (w8) MMX_STREAM(true, 1, panels);
         else MMX_STREAM(false, 1, panels);

@@ -292,6 +292,55 @@ def test_decode_small_shapes(po, shape, w8):
     assert np.linalg.norm(got - ref) <= 1e-3 * np.linalg.norm(ref)
 
 
+# the half-panel form of the streaming decode kernel (M <= 2), forced on: both weight types, the
+# all-at-once and the rolling window (K), ragged N, a column range, every post-op operand
+@pytest.mark.parametrize("shape", [(1, 256, 64), (2, 512, 100), (1, 4096, 352), (2, 2048, 96), (1, 11008, 160)])
+@pytest.mark.parametrize("w8", [False, True])
+def test_decode_half_panel_form(po, shape, w8):
+    M, K, N = shape
+    rng = np.random.default_rng(7 * sum(shape) + int(w8))
+    x = rand_bf16(rng, (M, K), 1.0)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    if w8:
+        W = np.clip(np.rint(rng.standard_normal((K, N)) * 40), -127, 127).astype(np.int8)
+        scale = rng.uniform(1e-3, 5e-3, N).astype(np.float32)
+        _, acc_ref = po.gemv_w8(x, W, scale, want_acc=True)
+        packed, steps, kw = mx.repack_b(dev(W)), mx.PP_DEQUANT | mx.PP_BIAS | mx.PP_GELU, {"b_dtype": mx.I8}
+    else:
+        W = rand_bf16(rng, (K, N), 0.05)
+        scale = None
+        acc_ref = po.gemm_bf16(x, W)
+        packed, steps, kw = mx.repack_b(dev_bf16(W)), mx.PP_BIAS | mx.PP_GELU, {}
+    n0, n1 = (32, N - 5) if N > 96 else (0, N)   # a column range that starts on a panel and ends inside one
+    mx.set_option("decode_halves", 1)
+    try:
+        y = torch.full((M, N), 7.0, dtype=torch.float32, device="cuda")
+        mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, steps, bias=dev(bias), deq_scale_per_oc=None if scale is None else dev(scale)),
+                n0=n0, n1=n1, **kw)
+        assert "skinny_half" in mx.last_kernel(), mx.last_kernel()
+        acc_gpu = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc_gpu, mx.PP_NONE), **kw)
+        assert "skinny_half" in mx.last_kernel()
+    finally:
+        mx.set_option("decode_halves", -1)
+    check_float_parity(host_bits(acc_gpu), acc_ref, f"half-panel accumulators {shape} w8={w8}")
+    posteps = (po.PP_DEQUANT if w8 else 0) | po.PP_BIAS | po.PP_GELU
+    again = po.pp(host_bits(acc_gpu), posteps, po.F32, bias=bias, deq_per_oc=scale)
+    got = host_bits(y)
+    assert np.array_equal(got[:, n0:n1].view(np.uint32), again[:, n0:n1].view(np.uint32))
+    assert np.all(got[:, :n0] == 7.0) and np.all(got[:, n1:] == 7.0)   # nothing outside the range is written
+    # the other form differs only in the order of the partial sums
+    acc2 = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    mx.set_option("decode_halves", 0)
+    try:
+        mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc2, mx.PP_NONE), **kw)
+        assert "half" not in mx.last_kernel()
+    finally:
+        mx.set_option("decode_halves", -1)
+    a, b = host_bits(acc_gpu).astype(np.float64), host_bits(acc2).astype(np.float64)
+    assert np.linalg.norm(a - b) <= 1e-5 * np.linalg.norm(b)
+
+
 @pytest.mark.parametrize("M", [4, 40])
 def test_weight_compressed_matmul(po, M):
     """Matmul<bf16,int8,float>: bf16 weights compressed per tensor inside the op (include/kernels_amx.hpp:1363-1379)."""
@@ -339,12 +388,28 @@ def _mlp_case(po, M, K, N, seed):
     # stage 1: h from the same x
     e1, f1 = check_float_parity(bf16_to_f32(h), bf16_to_f32(h_ref), f"mlp h M={M}")
     # the fused SiLU(gate)*up store equals the oracle's, bit for bit, on the accumulators the GPU produced
-    # (gate and up alternate in 32-column panels of the packed matrix)
-    acc = torch.zeros((M, 2 * N), dtype=torch.float32, device="cuda")
-    mx.gemm(dev_bf16(w["x"]), m.gate_up, 2 * N, mx.Epilogue(acc, mx.PP_NONE))
-    a = host_bits(acc).reshape(M, N // 32, 2, 32)
-    gate, up = np.ascontiguousarray(a[:, :, 0, :]).reshape(M, N), np.ascontiguousarray(a[:, :, 1, :]).reshape(M, N)
-    assert np.array_equal(h, po.silu_mul_bf16(gate, up))
+    # (gate and up alternate in 32-column panels of the packed matrix).  For M <= 2 the decode kernel has two
+    # forms that add the partial sums in different orders, chosen by the number of panels: pin the form so
+    # that the plain GEMM and the fused one go the same way, and check both.
+    forms = []
+    for halves in ((0, 1) if M <= 2 else (-1,)):
+        mx.set_option("decode_halves", halves)
+        try:
+            hh = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+            mx.gemm(dev_bf16(w["x"]), m.gate_up, 2 * N, mx.Epilogue(hh, mx.PP_SILU_GATE))
+            k_fused = mx.last_kernel()
+            acc = torch.zeros((M, 2 * N), dtype=torch.float32, device="cuda")
+            mx.gemm(dev_bf16(w["x"]), m.gate_up, 2 * N, mx.Epilogue(acc, mx.PP_NONE))
+            k_plain = mx.last_kernel()
+        finally:
+            mx.set_option("decode_halves", -1)
+        if M <= 2:
+            assert ("half" in k_fused) == (halves == 1) and ("half" in k_plain) == (halves == 1), (k_fused, k_plain)
+        a = host_bits(acc).reshape(M, N // 32, 2, 32)
+        gate, up = np.ascontiguousarray(a[:, :, 0, :]).reshape(M, N), np.ascontiguousarray(a[:, :, 1, :]).reshape(M, N)
+        assert np.array_equal(host_bits(hh), po.silu_mul_bf16(gate, up)), (halves, k_fused, k_plain)
+        forms.append(host_bits(hh))
+    assert any(np.array_equal(h, f) for f in forms)  # MLP.run above took one of them
     # stage 2: y from the SAME h the GPU produced (chained parity is not attainable by ulp: the
     # down projection is a cancelling sum, so one-ulp changes of h move small y by many ulps)
     y_ref = po.mlp_down(h, w["w_down"], split_k=True)
