@@ -27,11 +27,11 @@ PEAK_INT8_TOPS = 5000.0     # MI355X dense int8 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # HBM-side bytes per launch of the headline kernel, from two counter runs of this script under
-# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (KiB per dispatch: 81960 and 27920), each scaled by
+# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (KiB per dispatch: 81969 and 27913), each scaled by
 # what the same counter reads for the 256 MiB device copy of --calibrate-copy (factors 2.000 and 1.000);
 # the summary is profiles/gemm_bf16_256x192_ffn_up_M1024_hbm_traffic.txt.  Counters cannot be read from
 # inside the process, so the figure is only reported when the kernel that ran is the one profiled.
-MEASURED_TRAFFIC_BYTES = {"gemm_bf16_256x192_ring_out_bf16": (81960 * 2.000 + 27920 * 1.000) * 1024}
+MEASURED_TRAFFIC_BYTES = {"gemm_bf16_256x192_ring_out_bf16": (81969 * 2.000 + 27913 * 1.000) * 1024}
 
 
 def main():
@@ -181,6 +181,20 @@ def main():
         ms = avg_ms(Ai, [Bi], wi["N"], epi, 100)
         ops = 2.0 * wi["M"] * wi["K"] * wi["N"]
         extra["int8_fc_requant_M512_K4096_N4096"] = {
+            "us": round(ms * 1e3, 2), "tops": round(ops / ms / 1e9, 1), "frac_of_int8_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4),
+            "kernel": mx.last_kernel()}
+        del Ai, Bi, Ci
+        # the same int8 kernel on a shape large enough to fill the machine (the Llama-7B FFN shape at M=2048)
+        rng = np.random.default_rng(11)
+        Mi, Ki, Ni = 2048, 4096, 11008
+        Ai = torch.from_numpy(rng.integers(-127, 128, (Mi, Ki), dtype=np.int8)).cuda()
+        Bi = mx.repack_b(torch.from_numpy(rng.integers(-127, 128, (Ki, Ni), dtype=np.int8)).cuda())
+        Ci = torch.zeros((Mi, Ni), dtype=torch.int8, device="cuda")
+        epi = mx.Epilogue(Ci, mx.PP_DEQUANT | mx.PP_BIAS | mx.PP_QUANT, bias=torch.zeros(Ni, dtype=torch.float32, device="cuda"),
+                          deq_scale_per_oc=torch.full((Ni,), 1e-4, dtype=torch.float32, device="cuda"), q_scale=20.0)
+        ms = avg_ms(Ai, [Bi], Ni, epi, 100)
+        ops = 2.0 * Mi * Ki * Ni
+        extra["int8_fc_requant_M2048_K4096_N11008"] = {
             "us": round(ms * 1e3, 2), "tops": round(ops / ms / 1e9, 1), "frac_of_int8_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4),
             "kernel": mx.last_kernel()}
         del Ai, Bi, Ci
