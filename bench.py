@@ -236,6 +236,16 @@ def main():
             mlp[str(Mm)] = {"us": round(ms * 1e3, 1), "tflops": round(fl / ms / 1e9, 1),
                             "weight_GBps": round(3.0 * wm["K"] * wm["N"] * 2 / ms / 1e6, 0)}
         extra["llama7b_mlp_fused"] = mlp
+
+        # what the matrix pipes deliver with nothing else going on: an issue-bound loop of independent MFMAs,
+        # all-zero operands vs operands like the benchmark's (the clock under matrix load depends on the data)
+        ceil = {}
+        for key, dt, rnd in (("bf16_zero_operands", mx.BF16, 0), ("bf16_gaussian_operands", mx.BF16, 1),
+                             ("int8_zero_operands", mx.I8, 0), ("int8_uniform_operands", mx.I8, 1)):
+            mx.probe_mfma(dt, rnd, 20000)
+            rate, mhz = mx.probe_mfma(dt, rnd, 20000)
+            ceil[key] = {"rate": round(rate, 1), "unit": "TFLOP/s" if dt == mx.BF16 else "TOP/s", "shader_mhz": round(mhz)}
+        extra["mfma_issue_loop"] = ceil
         out["extra"] = extra
 
     print(json.dumps(out))

@@ -149,6 +149,13 @@ int mmx_set_option(const char* name, int value);
 int mmx_time_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* const* Bpacked_rot, int n_rot,
                   int M, int K, int N, int n0, int n1, const mmx_epilogue* ep, void* stream, int iters, float* ms_out);
 
+/* What an issue-bound loop of independent 32x32 MFMAs (dtype MMX_BF16 or MMX_I8) reaches on this device
+ * right now, with all-zero operands (random_operands = 0) or with random ones (bf16: N(0,1) x N(0,0.02);
+ * int8: uniform): *rate_out in Tflop/s or Top/s, *mhz_out the shader clock during the loop.  The clock of
+ * this part under matrix load depends on the operand data; benchmarks report this next to a GEMM's rate.
+ * scratch: 16 KiB of device memory.  Blocks until the loop has finished. */
+int mmx_probe_mfma(int dtype, int random_operands, int iters, void* scratch, void* stream, float* rate_out, float* mhz_out);
+
 #ifdef __cplusplus
 }
 #endif

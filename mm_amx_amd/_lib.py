@@ -17,7 +17,7 @@ _LIB_PATH = os.environ.get("MMX_LIB_PATH") or os.path.join(_HERE, "libmm_amx_amd
 
 EXPORTS = ["mmx_last_error", "mmx_init", "mmx_packed_b_bytes", "mmx_repack_b", "mmx_repack_gate_up",
            "mmx_quantize_weights", "mmx_dequant_packed", "mmx_gemm", "mmx_matvec", "mmx_mlp", "mmx_set_tile",
-           "mmx_set_option", "mmx_last_kernel", "mmx_time_gemm"]
+           "mmx_set_option", "mmx_last_kernel", "mmx_time_gemm", "mmx_probe_mfma"]
 
 
 class MmxError(RuntimeError):
@@ -66,6 +66,8 @@ def lib():
         l.mmx_time_gemm.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int64, C.POINTER(C.c_void_p), C.c_int, C.c_int,
                                     C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(_Epilogue), C.c_void_p, C.c_int,
                                     C.POINTER(C.c_float)]
+        l.mmx_probe_mfma.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.POINTER(C.c_float),
+                                     C.POINTER(C.c_float)]
         _lib = l
     return _lib
 
@@ -199,6 +201,15 @@ def time_gemm(A, Bpacked_list, N, ep, iters, b_dtype=None, n0=0, n1=None):
     _check(lib().mmx_time_gemm(a_dt, b_dt, A.data_ptr(), _row_stride_bytes(A), arr, len(Bpacked_list), M, K, N, n0,
                                n1, C.byref(s), _stream(), iters, C.byref(ms)))
     return ms.value
+
+
+def probe_mfma(dtype, random_operands, iters=20000):
+    """(Tflop/s or Top/s, shader MHz) of an issue-bound loop of independent MFMAs with zero or random operands."""
+    scratch = torch.zeros(16 * 1024, dtype=torch.uint8, device="cuda")
+    rate, mhz = C.c_float(0), C.c_float(0)
+    _check(lib().mmx_probe_mfma(dtype, int(bool(random_operands)), iters, scratch.data_ptr(), _stream(), C.byref(rate),
+                                C.byref(mhz)))
+    return rate.value, mhz.value
 
 
 def matvec(A, b, out=None):

@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmm_amx_amd.so")
-SOURCES = ["abi.hip", "gemm_bf16.hip", "gemm_i8.hip", "skinny.hip", "repack.hip"]
+SOURCES = ["abi.hip", "gemm_bf16.hip", "gemm_i8.hip", "skinny.hip", "repack.hip", "probe.hip"]
 # -ffp-contract=off: the epilogues reproduce the reference's separately rounded mul/add sequence;
 # fused operations are spelled fmaf().  Packed fp32 VALU instructions stay disabled.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-Wall", "-Wno-unused-function",

@@ -42,6 +42,7 @@ int launch_repack_gate_up(const void* wg, const void* wu, int64_t ldw, int K, in
 int launch_quantize(const void* W, int64_t ldw, int rows, int cols, void* Wq, int64_t ldq, float* scales_out,
                     uint32_t* scratch, hipStream_t st);
 int launch_dequant_packed(const void* in, int K, int N, void* out, hipStream_t st);
+int probe_mfma(bool i8, int random_operands, int iters, void* scratch, hipStream_t st, float* rate_out, float* mhz_out);
 int launch_matvec(bool i8, const void* A, int64_t lda, const void* b, void* c, int M, int K, hipStream_t st);
 
 struct TileCfg {
@@ -247,6 +248,12 @@ int mmx_set_option(const char* name, int value) {
         return MMX_OK;
     }
     return set_error(MMX_E_INVALID, "mmx_set_option: unknown option");
+}
+
+int mmx_probe_mfma(int dtype, int random_operands, int iters, void* scratch, void* stream, float* rate_out, float* mhz_out) {
+    if ((dtype != MMX_BF16 && dtype != MMX_I8) || iters <= 0 || !scratch || !rate_out || !mhz_out)
+        return set_error(MMX_E_INVALID, "mmx_probe_mfma: bad argument");
+    return probe_mfma(dtype == MMX_I8, random_operands, iters, scratch, static_cast<hipStream_t>(stream), rate_out, mhz_out);
 }
 
 int mmx_time_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* const* Bpacked_rot, int n_rot, int M,

@@ -630,3 +630,15 @@ def test_packed_weight_file_round_trip(po, tmp_path):
     assert np.array_equal(host_bits(y), po.gemv_w8(w["x"], w["W"], w["scale"]))
     with pytest.raises(mx.MmxError):
         packed_io.save_packed(path, packed[:-1], "int8", w["K"], w["N"])
+
+
+def test_mfma_issue_loop_probe():
+    # the measurement aid: rates are positive and below the datasheet peaks, zero operands are not slower than
+    # random ones (the clock under matrix load depends on the data), bad arguments are refused
+    z_rate, z_mhz = mx.probe_mfma(mx.BF16, 0, 4000)
+    r_rate, r_mhz = mx.probe_mfma(mx.BF16, 1, 4000)
+    assert 100 < r_rate <= z_rate * 1.05 < 2500 * 1.05 and 500 < r_mhz < 3000 and 500 < z_mhz < 3000
+    i_rate, _ = mx.probe_mfma(mx.I8, 1, 4000)
+    assert 200 < i_rate < 5000 * 1.05
+    with pytest.raises(mx.MmxError):
+        mx.probe_mfma(mx.F32, 0, 100)
