@@ -214,6 +214,23 @@ def main():
             del packs, Wg
         extra["decode_gemv_int8w_K4096_N11008"] = gemv
 
+        # the same GEMV over int4-compressed weights (22.5 MB), rotating over 24 copies (541 MB)
+        gemv4 = {}
+        wg = wl.decode_gemv_w8(M=4)
+        W4 = torch.randn((wg["K"], wg["N"]), dtype=torch.float32, device="cuda").mul_(0.02).to(torch.bfloat16)
+        P4, s4 = mx.quantize_pack_int4(W4)
+        packs = [P4] + [P4.clone() for _ in range(23)]
+        for Mg in (1, 4):
+            xg = dev_bf16(wg["x"][:Mg])
+            yg = torch.zeros((Mg, wg["N"]), dtype=torch.bfloat16, device="cuda")
+            epg = mx.Epilogue(yg, mx.PP_DEQUANT, deq_scale_per_oc=s4)
+            ms = avg_ms(xg, packs, wg["N"], epg, 240, b_dtype=mx.I4)
+            wbytes = float(wg["K"]) * wg["N"] / 2
+            gemv4[str(Mg)] = {"us": round(ms * 1e3, 2), "weight_GBps": round(wbytes / ms / 1e6, 0),
+                              "frac_of_hbm_peak": round(wbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "kernel": mx.last_kernel()}
+        del packs, P4, W4
+        extra["decode_gemv_int4w_K4096_N11008"] = gemv4
+
         # fused Llama-7B MLP
         mlp = {}
         wm = wl.llama_mlp(M=2048)

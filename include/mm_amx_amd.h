@@ -22,7 +22,7 @@ extern "C" {
 #endif
 
 /* element types */
-enum { MMX_F32 = 0, MMX_BF16 = 1, MMX_I8 = 2, MMX_I32 = 3 };
+enum { MMX_F32 = 0, MMX_BF16 = 1, MMX_I8 = 2, MMX_I32 = 3, MMX_I4 = 4 /* packed weights only */ };
 
 /* error codes */
 enum {
@@ -102,6 +102,20 @@ int mmx_repack_gate_up(const void* w_gate, const void* w_up, int64_t ldw_bytes, 
  * absmax_scratch is a device uint32 the call uses as scratch. */
 int mmx_quantize_weights(const void* W, int64_t ldw_bytes, int rows, int cols, void* Wq, int64_t ldq_bytes,
                          float* scales_out, uint32_t* absmax_scratch, void* stream);
+
+/* int4 weight compression.  The reference only times a stand-in that copies bytes
+ * (weight_compression/wcompress.hpp:90-134, README.md:216-244: "we haven't found efficient instructions to
+ * implement a fully-functional dequant() for INT4"); this is the real thing for the decode path.  Per output
+ * channel n, symmetric: a = max_k |w[k][n]|, q[k][n] = clamp(rint(w[k][n] * (7 / a)), -7, 7) in fp32 (q = 0 for
+ * a = 0), deq_scales_out[n] = a / 7.  W is [K, N] bf16 (transpose = 0) or [N, K] (transpose = 1, torch layout),
+ * row stride ldw_bytes.  packed receives mmx_packed_b_bytes(MMX_I4, K, N) bytes: 32-column panels of 1 KiB
+ * fragments, a fragment = 32 columns x 64 of k; the lane g * 32 + c (c = column in the panel, g = 0, 1) owns
+ * bytes [16 (g*32+c), +16): dword i holds k = 64 f + 32 g + 8 i + e in bits [4e, 4e+4), two's complement;
+ * K is padded with zeros to a multiple of 256.  Use: mmx_gemm(MMX_BF16, MMX_I4, ...) with M <= 32 and
+ * MMX_PP_DEQUANT with deq_scale_per_oc = deq_scales_out; the accumulators equal those of the bf16 GEMM on the
+ * (exactly representable) integers q. */
+int mmx_quantize_pack_int4(const void* W, int64_t ldw_bytes, int K, int N, int transpose, void* packed,
+                           float* deq_scales_out, void* stream);
 
 /* int8 packed weights -> bf16 packed weights (exact), the on-the-fly dequant of
  * include/kernels_amx.hpp:490-506 done once for the large-M weight-compressed path. */

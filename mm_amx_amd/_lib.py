@@ -8,7 +8,7 @@ import os
 
 import torch
 
-F32, BF16, I8, I32 = 0, 1, 2, 3
+F32, BF16, I8, I32, I4 = 0, 1, 2, 3, 4
 PP_NONE, PP_DEQUANT, PP_BIAS, PP_GELU, PP_QUANT, PP_SILU_GATE = 0, 1, 2, 4, 8, 16
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.environ.get("MMX_LIB_PATH") or os.path.join(_HERE, "libmm_amx_amd.so")
 
 EXPORTS = ["mmx_last_error", "mmx_init", "mmx_packed_b_bytes", "mmx_repack_b", "mmx_repack_gate_up",
-           "mmx_quantize_weights", "mmx_dequant_packed", "mmx_gemm", "mmx_matvec", "mmx_mlp", "mmx_set_tile",
+           "mmx_quantize_weights", "mmx_quantize_pack_int4", "mmx_dequant_packed", "mmx_gemm", "mmx_matvec", "mmx_mlp", "mmx_set_tile",
            "mmx_set_option", "mmx_last_kernel", "mmx_time_gemm", "mmx_probe_mfma"]
 
 
@@ -55,6 +55,8 @@ def lib():
         l.mmx_repack_gate_up.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
         l.mmx_quantize_weights.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p,
                                            C.c_void_p, C.c_void_p]
+        l.mmx_quantize_pack_int4.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
+                                             C.c_void_p]
         l.mmx_dequant_packed.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
         l.mmx_gemm.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
                                C.c_int, C.POINTER(_Epilogue), C.c_void_p]
@@ -168,6 +170,20 @@ def quantize_weights(W):
     _check(lib().mmx_quantize_weights(W.data_ptr(), _row_stride_bytes(W), W.shape[0], W.shape[1], Wq.data_ptr(),
                                       _row_stride_bytes(Wq), scales.data_ptr(), scratch.data_ptr(), _stream()))
     return Wq, scales
+
+
+def quantize_pack_int4(W, transpose=False):
+    """Per-output-channel symmetric int4 compression of a bf16 matrix W [K,N] (or [N,K] with transpose), packed for
+    gemm(..., b_dtype=I4) with M <= 32; returns (packed uint8, deq_scales fp32 [N])."""
+    _dev(W, "W")
+    if W.dtype != torch.bfloat16 or W.dim() != 2 or W.stride(1) != 1:
+        raise MmxError("W must be a 2-D bf16 tensor with unit column stride")
+    K, N = (W.shape[1], W.shape[0]) if transpose else W.shape
+    packed = torch.empty(packed_b_bytes(I4, K, N), dtype=torch.uint8, device=W.device)
+    deq = torch.empty(N, dtype=torch.float32, device=W.device)
+    _check(lib().mmx_quantize_pack_int4(W.data_ptr(), _row_stride_bytes(W), K, N, int(transpose), packed.data_ptr(),
+                                        deq.data_ptr(), _stream()))
+    return packed, deq
 
 
 def dequant_packed(packed_i8, K, N):

@@ -35,7 +35,7 @@ int launch_gemm_tiles_bf16(const void* A, int64_t lda, const void* Bp, int M, in
                            const Epilogue& ep, hipStream_t st);
 int launch_gemm_tiles_i8(const void* A, int64_t lda, const void* Bp, int M, int K, int N, int n0, int n1,
                          const Epilogue& ep, hipStream_t st);
-int launch_skinny(bool w8, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
+int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
                   const Epilogue& ep, hipStream_t st);
 int launch_repack(int elesz, const void* B, int64_t ldb, int K, int N, int transpose, void* out, hipStream_t st);
 int launch_repack_gate_up(const void* wg, const void* wu, int64_t ldw, int K, int N, void* out, hipStream_t st);
@@ -43,6 +43,8 @@ int launch_quantize(const void* W, int64_t ldw, int rows, int cols, void* Wq, in
                     uint32_t* scratch, hipStream_t st);
 int launch_dequant_packed(const void* in, int K, int N, void* out, hipStream_t st);
 int probe_mfma(bool i8, int random_operands, int iters, void* scratch, hipStream_t st, float* rate_out, float* mhz_out);
+int launch_quantize_pack_int4(const void* W, int64_t ldw, int K, int N, int transpose, void* packed, float* deq_out,
+                              hipStream_t st);
 int launch_matvec(bool i8, const void* A, int64_t lda, const void* b, void* c, int M, int K, hipStream_t st);
 
 struct TileCfg {
@@ -107,7 +109,8 @@ static int gemm_dispatch(int a_dtype, int b_dtype, const void* A, int64_t lda_by
     const bool bf = a_dtype == MMX_BF16 && b_dtype == MMX_BF16;
     const bool i8 = a_dtype == MMX_I8 && b_dtype == MMX_I8;
     const bool w8 = a_dtype == MMX_BF16 && b_dtype == MMX_I8;
-    if (!bf && !i8 && !w8) return set_error(MMX_E_INVALID, "mmx_gemm: dtype pair (%d, %d) not supported", a_dtype, b_dtype);
+    const bool w4 = a_dtype == MMX_BF16 && b_dtype == MMX_I4;
+    if (!bf && !i8 && !w8 && !w4) return set_error(MMX_E_INVALID, "mmx_gemm: dtype pair (%d, %d) not supported", a_dtype, b_dtype);
     if (n0 < 0 || n1 > N || n0 >= n1) return set_error(MMX_E_INVALID, "mmx_gemm: column range [%d, %d) outside [0, %d)", n0, n1, N);
     // the reference splits N in units of 32 (main.cpp:461-471)
     if (n0 % 32) return set_error(MMX_E_INVALID, "mmx_gemm: n0 = %d must be a multiple of 32", n0);
@@ -119,7 +122,8 @@ static int gemm_dispatch(int a_dtype, int b_dtype, const void* A, int64_t lda_by
     int rc = make_epilogue(ep_in, a_dtype, b_dtype, n0, &ep);
     if (rc) return rc;
     if ((ep.steps & MMX_PP_SILU_GATE) && ((n1 - n0) % 64)) return set_error(MMX_E_INVALID, "mmx_gemm: SILU_GATE needs (n1 - n0) %% 64 == 0");
-    if (M <= 32 && !i8) return launch_skinny(w8, A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st);
+    if (M <= 32 && !i8) return launch_skinny(w4 ? 2 : (w8 ? 1 : 0), A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st);
+    if (w4) return set_error(MMX_E_UNSUPPORTED, "mmx_gemm: bf16 x int4-weight is a decode path (M <= 32)");
     if (w8) return set_error(MMX_E_UNSUPPORTED, "mmx_gemm: bf16 x int8-weight with M > 32: convert the weights with mmx_dequant_packed and call the bf16 GEMM");
     return i8 ? launch_gemm_tiles_i8(A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st)
               : launch_gemm_tiles_bf16(A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st);
@@ -151,6 +155,10 @@ int mmx_init(int device) {
 }
 
 size_t mmx_packed_b_bytes(int dtype, int K, int N) {
+    if (dtype == MMX_I4) {  // 1 KiB fragments of 32 columns x 64 of k, four fragments at a time
+        if (K <= 0 || N <= 0) return 0;
+        return (size_t)((N + 31) / 32) * ((size_t)(K + 255) / 256 * 4) * 1024;
+    }
     const int es = elesz_of(dtype);
     if (!es || K <= 0 || N <= 0) return 0;
     const size_t kpad_bytes = ((size_t)K * es + 127) / 128 * 128;
@@ -183,6 +191,17 @@ int mmx_quantize_weights(const void* W, int64_t ldw_bytes, int rows, int cols, v
     if (rows <= 0 || cols <= 0 || ldw_bytes < (int64_t)cols * 2 || ldq_bytes < cols)
         return set_error(MMX_E_INVALID, "mmx_quantize_weights: bad shape or stride");
     return launch_quantize(W, ldw_bytes, rows, cols, Wq, ldq_bytes, scales_out, absmax_scratch, static_cast<hipStream_t>(stream));
+}
+
+int mmx_quantize_pack_int4(const void* W, int64_t ldw_bytes, int K, int N, int transpose, void* packed, float* deq_scales_out,
+                           void* stream) {
+    if (!W || !packed || !deq_scales_out) return set_error(MMX_E_INVALID, "mmx_quantize_pack_int4: NULL pointer");
+    if (K <= 0 || N <= 0) return set_error(MMX_E_INVALID, "mmx_quantize_pack_int4: K and N must be positive");
+    const int64_t min_ld = (int64_t)(transpose ? K : N) * 2;
+    if (ldw_bytes < min_ld || ldw_bytes % 2) return set_error(MMX_E_INVALID, "mmx_quantize_pack_int4: ldw_bytes %lld too small or odd", (long long)ldw_bytes);
+    if (reinterpret_cast<uintptr_t>(W) & 1) return set_error(MMX_E_INVALID, "mmx_quantize_pack_int4: W is not aligned to its element size");
+    if (reinterpret_cast<uintptr_t>(packed) & 15) return set_error(MMX_E_INVALID, "mmx_quantize_pack_int4: packed buffer must be 16-byte aligned");
+    return launch_quantize_pack_int4(W, ldw_bytes, K, N, transpose, packed, deq_scales_out, static_cast<hipStream_t>(stream));
 }
 
 int mmx_dequant_packed(const void* packed_i8, int K, int N, void* packed_bf16, void* stream) {

@@ -215,4 +215,62 @@ int launch_matvec(bool i8, const void* A, int64_t lda, const void* b, void* c, i
     return check_hip(hipGetLastError(), "matvec_kernel launch");
 }
 
+// ---- int4: per-column symmetric quantisation + packing in one pass per panel ---------------------------
+// One workgroup per 32-column panel.  Phase 1: column maxima of |w|; phase 2: every thread builds one dword
+// (8 values of one column) per fragment.  Not a hot path (done once per weight matrix).
+template <bool TRANSPOSED>
+__global__ __launch_bounds__(256) void quant4_pack_kernel(const char* W, int64_t ldw, int K, int N, char* out, int nfrag,
+                                                          float* deq_out) {
+    __shared__ float smax[8][32];
+    __shared__ float sscale[32];
+    const int t = threadIdx.x;
+    const int n0 = blockIdx.x * 32;
+    auto wval = [&](int k, int n) -> float {
+        if (k >= K || n >= N) return 0.0f;
+        const char* p = TRANSPOSED ? W + (int64_t)n * ldw + (int64_t)k * 2 : W + (int64_t)k * ldw + (int64_t)n * 2;
+        return from_bf16(*reinterpret_cast<const uint16_t*>(p));
+    };
+    {
+        const int c = t & 31, kr = t >> 5;
+        float m = 0.0f;
+        for (int k = kr; k < K; k += 8) m = fmaxf(m, fabsf(wval(k, n0 + c)));
+        smax[kr][c] = m;
+    }
+    __syncthreads();
+    if (t < 32) {
+        float a = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 8; r++) a = fmaxf(a, smax[r][t]);
+        sscale[t] = a > 0.0f ? 7.0f / a : 0.0f;
+        if (n0 + t < N) deq_out[n0 + t] = a / 7.0f;
+    }
+    __syncthreads();
+    const int i = t & 3, c = (t >> 2) & 31, g = t >> 7;
+    const float qs = sscale[c];
+    for (int f = 0; f < nfrag; f++) {
+        const int k0 = 64 * f + 32 * g + 8 * i;
+        uint32_t d = 0;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            float q = rintf(wval(k0 + e, n0 + c) * qs);
+            q = fminf(fmaxf(q, -7.0f), 7.0f);
+            d |= ((uint32_t)(int)q & 0xfu) << (4 * e);
+        }
+        *reinterpret_cast<uint32_t*>(out + ((int64_t)blockIdx.x * nfrag + f) * 1024 + t * 4) = d;
+    }
+}
+
+int launch_quantize_pack_int4(const void* W, int64_t ldw, int K, int N, int transpose, void* packed, float* deq_out,
+                              hipStream_t st) {
+    const int nfrag = (K + 255) / 256 * 4;
+    const int npanels = (N + 31) / 32;
+    if (transpose)
+        hipLaunchKernelGGL(quant4_pack_kernel<true>, dim3(npanels), dim3(256), 0, st, static_cast<const char*>(W), ldw, K, N,
+                           static_cast<char*>(packed), nfrag, deq_out);
+    else
+        hipLaunchKernelGGL(quant4_pack_kernel<false>, dim3(npanels), dim3(256), 0, st, static_cast<const char*>(W), ldw, K, N,
+                           static_cast<char*>(packed), nfrag, deq_out);
+    return check_hip(hipGetLastError(), "quant4_pack_kernel launch");
+}
+
 }  // namespace mmx

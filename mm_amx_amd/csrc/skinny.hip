@@ -49,6 +49,31 @@ __device__ __forceinline__ bf16x8 s8x8_to_bf16(uint32_t lo, uint32_t hi) {
     return r;
 }
 
+// 8 int4 (one dword, element e in bits 4e .. 4e+3, two's complement) -> 8 bf16 holding q / 16, exact.
+// v_cvt_off_f32_i4 maps the low nibble of its source to (signed nibble) / 16; its SDWA form picks the byte,
+// so the even nibbles come straight from the dword and the odd ones from the dword shifted by four:
+// 13 instructions per dword with the packing, against 20 for bit-field extract + int-to-float.  The
+// callers multiply the finished sums by 16 (exact).
+__device__ __forceinline__ bf16x8 s4x8_to_bf16_div16(uint32_t d) {
+    const uint32_t dh = d >> 4;
+    float f[8];
+#define MMX_CVT4(DST, SRC, BYTE) \
+    asm("v_cvt_off_f32_i4_sdwa %0, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:" BYTE : "=v"(DST) : "v"(SRC))
+    MMX_CVT4(f[0], d, "BYTE_0");
+    MMX_CVT4(f[1], dh, "BYTE_0");
+    MMX_CVT4(f[2], d, "BYTE_1");
+    MMX_CVT4(f[3], dh, "BYTE_1");
+    MMX_CVT4(f[4], d, "BYTE_2");
+    MMX_CVT4(f[5], dh, "BYTE_2");
+    MMX_CVT4(f[6], d, "BYTE_3");
+    MMX_CVT4(f[7], dh, "BYTE_3");
+#undef MMX_CVT4
+    bf16x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; e++) r[e] = (__bf16)f[e];
+    return r;
+}
+
 __device__ __forceinline__ void store_out(const Epilogue& ep, int m, int n, float r) {
     char* row = ep.C + (int64_t)m * ep.ldc;
     switch (ep.out_dtype) {
@@ -128,8 +153,10 @@ __device__ __forceinline__ void skinny_finish(const SkinnyArgs& s, const float (
     }
 }
 
-template <bool W8, int NP>
+// WK: weights are bf16 (0), int8 (1) or int4 (2); a 1 KiB fragment is 32 columns x 16, 32 or 64 of k
+template <int WK, int NP>
 __global__ __launch_bounds__(512) void skinny_kernel(const SkinnyArgs s) {
+    constexpr bool W8 = WK == 1, W4 = WK == 2;
     constexpr int U = 4;  // fragments in flight per wave
     __shared__ float red[8][NP][16][64];
 
@@ -155,7 +182,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(const SkinnyArgs s) {
 
     for (int f0 = f_begin; f0 < f_end; f0 += U) {
         u32x4 w[NP][U];
-        bf16x8 xa[U], xb[U];
+        bf16x8 xa[U], xb[U], xc[U], xd[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int f = f0 + u;
@@ -167,7 +194,13 @@ __global__ __launch_bounds__(512) void skinny_kernel(const SkinnyArgs s) {
                     w[p][u] = *reinterpret_cast<const u32x4*>(s.Wp + (int64_t)panel * s.panel_stride +
                                                               (int64_t)f * 1024 + lane * 16);
             }
-            if constexpr (W8) {
+            if constexpr (W4) {
+                const int k0 = 64 * f + 32 * g32;
+                xa[u] = load_x8(xrow, k0, s.K, live && f < f_end, s.x_vec_ok);
+                xb[u] = load_x8(xrow, k0 + 8, s.K, live && f < f_end, s.x_vec_ok);
+                xc[u] = load_x8(xrow, k0 + 16, s.K, live && f < f_end, s.x_vec_ok);
+                xd[u] = load_x8(xrow, k0 + 24, s.K, live && f < f_end, s.x_vec_ok);
+            } else if constexpr (W8) {
                 const int k0 = 32 * f + 16 * g32;
                 xa[u] = load_x8(xrow, k0, s.K, live && f < f_end, s.x_vec_ok);
                 xb[u] = load_x8(xrow, k0 + 8, s.K, live && f < f_end, s.x_vec_ok);
@@ -179,7 +212,12 @@ __global__ __launch_bounds__(512) void skinny_kernel(const SkinnyArgs s) {
         for (int u = 0; u < U; u++) {
 #pragma unroll
             for (int p = 0; p < NP; p++) {
-                if constexpr (W8) {
+                if constexpr (W4) {
+                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s4x8_to_bf16_div16(w[p][u].x), xa[u], acc[p], 0, 0, 0);
+                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s4x8_to_bf16_div16(w[p][u].y), xb[u], acc[p], 0, 0, 0);
+                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s4x8_to_bf16_div16(w[p][u].z), xc[u], acc[p], 0, 0, 0);
+                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s4x8_to_bf16_div16(w[p][u].w), xd[u], acc[p], 0, 0, 0);
+                } else if constexpr (W8) {
                     acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(w[p][u].x, w[p][u].y), xa[u], acc[p], 0, 0, 0);
                     acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(w[p][u].z, w[p][u].w), xb[u], acc[p], 0, 0, 0);
                 } else {
@@ -192,7 +230,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(const SkinnyArgs s) {
 #pragma unroll
     for (int p = 0; p < NP; p++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) red[wave][p][v][lane] = acc[p][v];
+        for (int v = 0; v < 16; v++) red[wave][p][v][lane] = W4 ? acc[p][v] * 16.0f : acc[p][v];  // int4 operands were q / 16
     __syncthreads();
 
     skinny_finish<NP>(s, red, panel_first, tid, fin);
@@ -443,9 +481,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 // 128 VGPRs at most: two workgroups per CU, so that every panel of an 11008-column matrix is resident at once.
 // ONE: every wave's share of K is a single batch (the common decode shapes); a variant of its own so that
 // each kernel holds one code path and stays within its registers.
-template <bool W8, int NP, bool ONE>
+template <int WK, int NP, bool ONE>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void skinny_stream_kernel(const SkinnyArgs s, int zero_off) {
-    constexpr int U = 16 / NP;  // fragments per panel per wave in flight at once (16 KiB of weights)
+    constexpr bool W8 = WK == 1, W4 = WK == 2;
+    // fragments per panel per wave in flight at once (16 KiB of weights; int4: 8 KiB, a fragment holds 64 of k
+    // and unpacking it costs more than streaming it)
+    constexpr int U = (W4 ? 8 : 16) / NP;
     __shared__ float red[8][NP][16][64];
     extern __shared__ __attribute__((aligned(1024))) char xs[];  // [M][K] bf16, then at zero_off a row of zeros
 
@@ -513,7 +554,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         const bool valid_ = (f_ - f_begin) < per_wave && f_ <= f_last; /* scalar */                             \
         const int fc_ = f_ < f_last ? f_ : f_last;                                                              \
         const char* xr_ = valid_ ? xrow : zrow;                                                                 \
-        if constexpr (W8) {                                                                                     \
+        if constexpr (W4) {                                                                                     \
+            _Pragma("unroll") for (int i_ = 0; i_ < 4; i_++) {                                                  \
+                const bf16x8 xq_ = *reinterpret_cast<const bf16x8*>(xr_ + (64 * fc_ + 32 * g32 + 8 * i_) * 2);  \
+                _Pragma("unroll") for (int p = 0; p < NP; p++)                                                  \
+                    acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s4x8_to_bf16_div16(w[p][UU][i_]), xq_, acc[p], 0, 0, 0); \
+            }                                                                                                   \
+        } else if constexpr (W8) {                                                                              \
             const bf16x8 xa_ = *reinterpret_cast<const bf16x8*>(xr_ + (32 * fc_ + 16 * g32) * 2);               \
             const bf16x8 xb_ = *reinterpret_cast<const bf16x8*>(xr_ + (32 * fc_ + 16 * g32 + 8) * 2);           \
             _Pragma("unroll") for (int p = 0; p < NP; p++) {                                                    \
@@ -560,7 +607,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #pragma unroll
     for (int p = 0; p < NP; p++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) red[wave][p][v][lane] = acc[p][v];
+        for (int v = 0; v < 16; v++) red[wave][p][v][lane] = W4 ? acc[p][v] * 16.0f : acc[p][v];  // int4 operands were q / 16
     __syncthreads();
     skinny_finish<NP>(s, red, panel_first, tid, fin);
 }
@@ -752,8 +799,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 
 int decode_halves();
 
-int launch_skinny(bool w8, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
+// wk: weights are bf16 (0), int8 (1) or int4 (2)
+int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
                   const Epilogue& ep, hipStream_t st) {
+    const bool w8 = wk == 1;
     SkinnyArgs s;
     s.x = static_cast<const char*>(x);
     s.ldx = ldx;
@@ -761,7 +810,7 @@ int launch_skinny(bool w8, const void* x, int64_t ldx, const void* Wp, int M, in
     s.M = M;
     s.K = K;
     const int kbytes_pad = ((K * (w8 ? 1 : 2)) + 127) / 128 * 128;
-    s.nfrag = kbytes_pad / 32;  // 32 bytes of K per column per fragment
+    s.nfrag = wk == 2 ? (K + 255) / 256 * 4 : kbytes_pad / 32;  // 32 bytes of K per column per fragment
     s.panel_stride = (int64_t)s.nfrag * 1024;
     s.npanels = (N + 31) / 32;
     s.n0 = n0;
@@ -770,6 +819,23 @@ int launch_skinny(bool w8, const void* x, int64_t ldx, const void* Wp, int M, in
     s.ep = ep;
     const int panels = ((n1 + 31) >> 5) - (n0 >> 5);
     const bool pairs = (ep.steps & MMX_PP_SILU_GATE) != 0;
+    if (wk == 2) {
+        // int4 weights: the streaming kernel if x fits in LDS and K fills whole fragments, else the general one
+        if (pairs) return set_error(MMX_E_UNSUPPORTED, "SILU_GATE over int4 weights is not built");
+        const int zoff = (M * K * 2 + 1023) & ~1023;
+        const int xb = zoff + K * 2;
+        if (s.nfrag * 64 == K && xb <= 46 * 1024 && s.x_vec_ok) {
+            note_kernel("skinny_stream_w4");
+            if ((s.nfrag + 7) / 8 <= 8)
+                hipLaunchKernelGGL((skinny_stream_kernel<2, 1, true>), dim3(panels), dim3(512), xb, st, s, zoff);
+            else
+                hipLaunchKernelGGL((skinny_stream_kernel<2, 1, false>), dim3(panels), dim3(512), xb, st, s, zoff);
+            return check_hip(hipGetLastError(), "skinny_stream_kernel launch");
+        }
+        note_kernel("skinny_w4");
+        hipLaunchKernelGGL((skinny_kernel<2, 1>), dim3(panels), dim3(512), 0, st, s);
+        return check_hip(hipGetLastError(), "skinny_kernel launch");
+    }
     const int kpad = kbytes_pad / (w8 ? 1 : 2);  // elements of K the packed weights cover
     const int zero_off = (M * K * 2 + 1023) & ~1023;
     const int xbytes = zero_off + K * 2;  // x, a gap up to the next KiB, one row of zeros

@@ -187,6 +187,45 @@ float orc_quantize_weights(const uint16_t* W, int64_t ldw, int rows, int cols, i
     return dq;
 }
 
+/* int4 weight compression.  The reference has no algorithm to restate here: weight_compression/wcompress.hpp:90-134
+ * and README.md:216-244 only time a stand-in that copies bytes ("we haven't found efficient instructions to
+ * implement a fully-functional dequant() for INT4").  This is the definition the device code is held to:
+ * per output channel n, a = max_k |w[k][n]|, q = clamp(rne(w * (7 / a)), -7, 7) in fp32 (0 for a = 0),
+ * deq[n] = a / 7.  W is [K][N] (transpose = 0) or [N][K] (transpose = 1), ldw in elements; q is [K][N]. */
+void orc_quantize_int4(const uint16_t* W, int64_t ldw, int K, int N, int transpose, int8_t* q, float* deq) {
+    for (int n = 0; n < N; n++) {
+        float a = 0.0f;
+        for (int k = 0; k < K; k++) {
+            const float v = fabsf(orc_bf16_to_f32(transpose ? W[(size_t)n * ldw + k] : W[(size_t)k * ldw + n]));
+            if (v > a) a = v;
+        }
+        const float qs = a > 0.0f ? 7.0f / a : 0.0f;
+        deq[n] = a / 7.0f;
+        for (int k = 0; k < K; k++) {
+            float r = rintf(orc_bf16_to_f32(transpose ? W[(size_t)n * ldw + k] : W[(size_t)k * ldw + n]) * qs);
+            r = r < -7.0f ? -7.0f : (r > 7.0f ? 7.0f : r);
+            q[(size_t)k * N + n] = (int8_t)r;
+        }
+    }
+}
+
+/* This project's packed int4 layout (no reference counterpart): 32-column panels of 1 KiB fragments, a fragment
+ * = 32 columns x 64 of k; lane g*32 + c owns 16 bytes, its dword i holds k = 64 f + 32 g + 8 i + e in bits
+ * [4e, 4e+4) as two's complement; K is padded with zeros to a multiple of 256. */
+size_t orc_pack_int4_bytes(int K, int N) { return (size_t)((N + 31) / 32) * ((size_t)(K + 255) / 256 * 4) * 1024; }
+
+void orc_pack_int4(const int8_t* q, int K, int N, uint8_t* out) {
+    const size_t nfrag = (size_t)(K + 255) / 256 * 4;
+    memset(out, 0, orc_pack_int4_bytes(K, N));
+    for (int n = 0; n < N; n++)
+        for (int k = 0; k < K; k++) {
+            const int f = k / 64, g = (k % 64) / 32, i = (k % 32) / 8, e = k % 8;
+            const size_t byte = ((size_t)(n / 32) * nfrag + f) * 1024 + (size_t)(g * 32 + n % 32) * 16 + i * 4 + e / 2;
+            const uint8_t nib = (uint8_t)q[(size_t)k * N + n] & 0xf;
+            out[byte] |= (e & 1) ? (uint8_t)(nib << 4) : nib;
+        }
+}
+
 /* weight_compression/fc16m.cpp:451-502 (matmul16m_Wint8B) and include/kernels_amx.hpp:1381-1441:
  * int8 weights are converted to bf16 exactly (|w| <= 128 needs 8 significant bits;
  * include/kernels_amx.hpp:490-506, fc16m.cpp:309-333) and fed to the same tdpbf16ps chain, the

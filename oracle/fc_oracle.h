@@ -25,6 +25,11 @@
  *                                    counterpart); checked to be a bijection + zero pad
  *   orc_quantize_weights   pinned  — against the compiled reference Matmul<bf16,int8>
  *   orc_gemv_w8            pinned  — through orc_gemm_bf16 on exactly converted weights
+ *   orc_quantize_int4,     spec    — PARITY UNPINNED against the reference, which has no int4 algorithm (it
+ *   orc_pack_int4                    only times a byte-copying stand-in): these define what the device code
+ *                                    must produce; checked by what the mathematics fixes (|w - q deq| <=
+ *                                    deq/2, |q| <= 7, the column maximum maps to +-7, zero columns, the
+ *                                    layout is a bijection with zero padding)
  *   orc_matvec_*           pinned  — against the compiled reference MatmulVector/GemAvB
  *                                    for ceil(K/kStep) <= 4 (the reference is wrong beyond)
  *   orc_rcp14              pinned  — against the vrcp14ps instruction itself on all 2^32 inputs
@@ -114,6 +119,12 @@ float orc_quantize_weights(const uint16_t* W, int64_t ldw, int rows, int cols,
 /* y[M,N] (bf16) = bf16( (x[M,K] bf16 · float(Wq[K,N] int8)) * scale[n] ), fp32 AMX-order
  * accumulation.  Wq is [K,N] (transW=0) or [N,K] (transW=1).  If acc_out != NULL the raw
  * fp32 accumulators are also returned. */
+/* int4 weight compression (definition of this project; the reference only times a stand-in,
+ * weight_compression/wcompress.hpp:90-134) and its packed layout */
+void orc_quantize_int4(const uint16_t* W, int64_t ldw, int K, int N, int transpose, int8_t* q, float* deq);
+size_t orc_pack_int4_bytes(int K, int N);
+void orc_pack_int4(const int8_t* q, int K, int N, uint8_t* out);
+
 void orc_gemv_w8(const uint16_t* x, int64_t ldx, const int8_t* Wq, int64_t ldw, int transW,
                  const float* scale, uint16_t* y, int64_t ldy, float* acc_out, int M, int K, int N,
                  int nthreads);

@@ -158,6 +158,25 @@ def quantize_weights(W):
     return Wq, float(dq), float(qs.value)
 
 
+def quantize_int4(W, transpose=False):
+    """W bf16 bits [K,N] (or [N,K] with transpose) -> (q int8 [K,N] in [-7,7], deq fp32 [N])"""
+    W = _c(W, np.uint16)
+    K, N = (W.shape[1], W.shape[0]) if transpose else W.shape
+    q = np.empty((K, N), np.int8)
+    deq = np.empty(N, np.float32)
+    lib().orc_quantize_int4(_p(W), C.c_int64(W.shape[1]), K, N, int(transpose), _p(q), _p(deq))
+    return q, deq
+
+
+def pack_int4(q):
+    q = _c(q, np.int8)
+    K, N = q.shape
+    lib().orc_pack_int4_bytes.restype = C.c_size_t
+    out = np.empty(lib().orc_pack_int4_bytes(K, N), np.uint8)
+    lib().orc_pack_int4(_p(q), K, N, _p(out))
+    return out
+
+
 def gemv_w8(x, Wq, scale, transW=False, nthreads=0, want_acc=False):
     M, K = x.shape
     N = Wq.shape[0] if transW else Wq.shape[1]

@@ -642,3 +642,77 @@ def test_mfma_issue_loop_probe():
     assert 200 < i_rate < 5000 * 1.05
     with pytest.raises(mx.MmxError):
         mx.probe_mfma(mx.F32, 0, 100)
+
+
+# ---- int4-compressed weights (decode path; defined by the oracle, the reference only times a stand-in) ------
+@pytest.mark.parametrize("shape", [(64, 32), (300, 45), (256, 96), (4096, 64), (70, 33)])
+@pytest.mark.parametrize("transpose", [False, True])
+def test_int4_quantise_and_pack_match_the_definition(po, shape, transpose):
+    K, N = shape
+    rng = np.random.default_rng(K + N)
+    Wf = (rng.standard_normal((K, N)) * 0.03).astype(np.float32)
+    if N > 1:
+        Wf[:, 1] = 0.0
+    W = po.f32_to_bf16(Wf)
+    q, deq = po.quantize_int4(W)
+    want = po.pack_int4(q)
+    src = np.ascontiguousarray(W.T) if transpose else W
+    wide = torch.zeros((src.shape[0], src.shape[1] + 8), dtype=torch.bfloat16, device="cuda")   # a padded row stride
+    wide[:, :src.shape[1]] = dev_bf16(src)
+    packed, deq_gpu = mx.quantize_pack_int4(wide[:, :src.shape[1]], transpose=transpose)
+    assert packed.numel() == want.size == mx.packed_b_bytes(mx.I4, K, N)
+    assert np.array_equal(host_bits(deq_gpu).view(np.uint32), deq.view(np.uint32))
+    assert np.array_equal(host_bits(packed), want)
+
+
+@pytest.mark.parametrize("shape", [(1, 256, 64), (3, 320, 100), (16, 337, 96), (32, 2560, 192), (2, 4096, 352), (4, 8192, 64)])
+def test_int4_decode_shapes(po, shape):
+    M, K, N = shape
+    rng = np.random.default_rng(sum(shape))
+    x = rand_bf16(rng, (M, K), 1.0)
+    W = rand_bf16(rng, (K, N), 0.05)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    q, deq = po.quantize_int4(W)
+    _, acc_ref = po.gemv_w8(x, q, deq, want_acc=True)     # exact conversion of the integers, then the bf16 GEMM
+    packed, deq_gpu = mx.quantize_pack_int4(dev_bf16(W))
+    y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_DEQUANT | mx.PP_BIAS | mx.PP_GELU, bias=dev(bias),
+                                                deq_scale_per_oc=deq_gpu), b_dtype=mx.I4)
+    assert "w4" in mx.last_kernel()
+    stream_ok = K % 256 == 0 and (M + 1) * K * 2 <= 45 * 1024
+    assert ("stream" in mx.last_kernel()) == stream_ok, (mx.last_kernel(), shape)
+    acc_gpu = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc_gpu, mx.PP_NONE), b_dtype=mx.I4)
+    check_float_parity(host_bits(acc_gpu), acc_ref, f"int4 decode accumulators {shape}")
+    again = po.pp(host_bits(acc_gpu), po.PP_DEQUANT | po.PP_BIAS | po.PP_GELU, po.F32, bias=bias, deq_per_oc=deq)
+    assert np.array_equal(host_bits(y).view(np.uint32), again.view(np.uint32))
+    ref = po.pp(acc_ref, po.PP_DEQUANT | po.PP_BIAS | po.PP_GELU, po.F32, bias=bias, deq_per_oc=deq)
+    assert np.linalg.norm(host_bits(y) - ref) <= 1e-3 * np.linalg.norm(ref)
+
+
+@pytest.mark.parametrize("M", [1, 4])
+def test_int4_gemv_full_size(po, M):
+    w = wl.decode_gemv_w8(M=M)      # x of the int8 case; the weights come from a bf16 matrix here
+    rng = np.random.default_rng(44)
+    W = rand_bf16(rng, (w["K"], w["N"]), 0.02)
+    q, deq = po.quantize_int4(W)
+    ref = po.gemv_w8(w["x"], q, deq)
+    packed, deq_gpu = mx.quantize_pack_int4(dev_bf16(W))
+    assert np.array_equal(host_bits(deq_gpu).view(np.uint32), deq.view(np.uint32))
+    y = torch.zeros((M, w["N"]), dtype=torch.bfloat16, device="cuda")
+    mx.gemm(dev_bf16(w["x"]), packed, w["N"], mx.Epilogue(y, mx.PP_DEQUANT, deq_scale_per_oc=deq_gpu), b_dtype=mx.I4)
+    assert mx.last_kernel() == "skinny_stream_w4"
+    err, frac = check_float_parity(bf16_to_f32(host_bits(y)), bf16_to_f32(ref), f"gemv_w4 M={M}")
+    print(f"gemv_w4 M={M}: rel_fro={err:.2e} within_1ulp={frac * 100:.4f}%")
+
+
+def test_int4_is_a_decode_path_only():
+    x = torch.zeros((40, 256), dtype=torch.bfloat16, device="cuda")
+    packed, deq = mx.quantize_pack_int4(torch.zeros((256, 64), dtype=torch.bfloat16, device="cuda"))
+    y = torch.zeros((40, 64), dtype=torch.float32, device="cuda")
+    with pytest.raises(mx.MmxError, match="decode path"):
+        mx.gemm(x, packed, 64, mx.Epilogue(y, mx.PP_NONE), b_dtype=mx.I4)
+    with pytest.raises(mx.MmxError):
+        mx.gemm(x[:4], packed, 64, mx.Epilogue(y[:4, :32], mx.PP_SILU_GATE), b_dtype=mx.I4)
+    with pytest.raises(mx.MmxError):
+        mx.quantize_pack_int4(torch.zeros((256, 64), dtype=torch.float32, device="cuda"))

@@ -105,6 +105,46 @@ def test_quantize_weights_properties(po):
     assert np.max(np.abs(Wq * np.float32(dq) - Wf)) <= 0.5 * dq * 1.001
 
 
+def test_int4_quantiser_and_layout_properties(po):
+    # the int4 compression has no counterpart in the reference (it only times a byte-copying stand-in), so its
+    # definition is checked by what the mathematics fixes
+    rng = np.random.default_rng(12)
+    for K, N in ((64, 32), (300, 45), (256, 96), (70, 33)):
+        Wf = (rng.standard_normal((K, N)) * 0.03).astype(np.float32)
+        Wf[:, 1] = 0.0                      # a column of zeros
+        Wf[3, 2] = -1.0                     # a dominant negative maximum
+        W = po.f32_to_bf16(Wf)
+        Wf = po.bf16_to_f32(W)
+        q, deq = po.quantize_int4(W)
+        amax = np.abs(Wf).max(axis=0)
+        assert np.array_equal(deq, (amax / np.float32(7)).astype(np.float32))
+        assert q.min() >= -7 and q.max() <= 7
+        assert np.all(q[:, 1] == 0) and deq[1] == 0
+        assert q[3, 2] == -7
+        # the maximum of every non-zero column maps to +-7, and every value is within half a step
+        nz = amax > 0
+        assert np.all(np.abs(q).max(axis=0)[nz] == 7)
+        assert np.all(np.abs(q * deq[None, :] - Wf) <= 0.5 * deq[None, :] * 1.001 + 1e-12)
+        # brute force of the rounding rule in fp32
+        qs = np.where(nz, np.float32(7) / np.where(nz, amax, 1).astype(np.float32), np.float32(0)).astype(np.float32)
+        want = np.clip(np.rint((Wf * qs[None, :]).astype(np.float32)), -7, 7).astype(np.int8)
+        assert np.array_equal(q, want)
+        # the transposed source gives the same result
+        qT, deqT = po.quantize_int4(np.ascontiguousarray(W.T), transpose=True)
+        assert np.array_equal(qT, q) and np.array_equal(deqT, deq)
+        # layout: zero-padded bijection, nibble (k, n) where the documented index says
+        packed = po.pack_int4(q)
+        nfrag = -(-K // 256) * 4
+        assert packed.size == -(-N // 32) * nfrag * 1024
+        lo, hi = packed & 0xF, packed >> 4
+        nib = np.stack([lo, hi], axis=1).reshape(-1)          # nibble e of a byte stream: byte e//2, low first
+        assert np.count_nonzero(nib) == np.count_nonzero(q)
+        for k, n in ((0, 0), (K - 1, N - 1), (K // 2, N // 3), (37 % K, 5), (63, 31 % N)):
+            f, g, i, e = k // 64, (k % 64) // 32, (k % 32) // 8, k % 8
+            idx = (((n // 32) * nfrag + f) * 1024 + (g * 32 + n % 32) * 16 + i * 4) * 2 + e
+            assert nib[idx] == (int(q[k, n]) & 0xF)
+
+
 def test_gemv_w8_is_exact_conversion_then_gemm(po):
     rng = np.random.default_rng(3)
     M, K, N = 3, 128, 40
