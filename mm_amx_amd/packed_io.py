@@ -16,15 +16,15 @@ from safetensors.torch import save_file
 from . import _lib as L
 
 FORMAT = "mm_amx_amd.packed_b/1"
-_DT = {"bf16": L.BF16, "int8": L.I8}
+_DT = {"bf16": L.BF16, "int8": L.I8, "int4": L.I4}
 
 
 def save_packed(path, packed, dtype, K, N, scales=None, layout="b", extra=None):
-    """packed: uint8 tensor from repack_b / repack_gate_up; dtype 'bf16' or 'int8'; K, N: the logical [K, N]
+    """packed: uint8 tensor from repack_b / repack_gate_up / quantize_pack_int4; dtype 'bf16', 'int8' or 'int4'; K, N: the logical [K, N]
     of the packed matrix (for a gate/up pair N is 2 x the projection width, layout='gate_up');
     scales: optional fp32 [N] per-output-channel dequantisation scales."""
     if dtype not in _DT:
-        raise L.MmxError("dtype must be 'bf16' or 'int8'")
+        raise L.MmxError("dtype must be 'bf16', 'int8' or 'int4'")
     if packed.dtype != torch.uint8 or packed.numel() != L.packed_b_bytes(_DT[dtype], K, N):
         raise L.MmxError("packed does not have the size of a packed [K, N] matrix of this dtype")
     tensors = {"packed": packed.detach().cpu().contiguous()}
