@@ -45,7 +45,7 @@ def main():
                     help="also run a 256 MiB device-to-device copy: a kernel of known traffic to scale profiler byte counters by")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on ONE GPU (the path shards over N by column panels; see DESIGN.md); "
+        sys.exit("bench.py: this build runs on ONE GPU (the path would shard over N by column panels, nothing here does); "
                  "--gpus must be 1")
 
     import numpy as np

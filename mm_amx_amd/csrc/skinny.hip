@@ -1,4 +1,4 @@
-// Decode-regime FC (M <= 32): y = PP(x · W[:, n0:n1]) over bf16 or int8-compressed weights.
+// Decode-regime FC (M <= 32): y = PP(x · W[:, n0:n1]) over bf16, int8-compressed or int4-compressed weights.
 //
 // Stands in for the M<=16 / M<=32 branches of amx_kernel::Matmul (include/kernels_amx.hpp:1216-1253,
 // 1297-1302), for Matmul<bf16,int8,float> at small M (:1381-1441) and for matmul16m_Wint8B
@@ -6,8 +6,9 @@
 // exactly once, in 1 KiB lane-contiguous fragments of the same packed layout the tile GEMM uses.
 // The few activations ride in the other MFMA operand (32 columns, only M of them live), so the
 // matrix core does the multiply-accumulate while the vector ALU only converts int8 -> bf16
-// (exact: |w| <= 128 has at most 8 significant bits, as in include/kernels_amx.hpp:490-506).
-// K is split across the 8 wavefronts of a workgroup; partial 32x32 blocks are summed through LDS.
+// (exact: |w| <= 128 has at most 8 significant bits, as in include/kernels_amx.hpp:490-506) or int4 -> bf16
+// (the reference has no int4 dequant, only a byte-copying stand-in: weight_compression/wcompress.hpp:90-134).
+// K is split across the wavefronts of a workgroup; partial 32x32 blocks are summed through LDS.
 #include "common.hpp"
 
 namespace mmx {
@@ -112,7 +113,7 @@ __device__ __forceinline__ void skinny_prefetch(const SkinnyArgs& s, int panel_f
     }
 }
 
-// cross-wave reduction of the partial 32x32 blocks + post-op + store (shared by both decode kernels)
+// cross-wave reduction of the partial 32x32 blocks + post-op + store (shared by the 8-wave decode kernels)
 template <int NP>
 __device__ __forceinline__ void skinny_finish(const SkinnyArgs& s, const float (&red)[8][NP][16][64], int panel_first, int tid,
                                               const FinishOperands<NP>& o) {
