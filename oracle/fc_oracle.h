@@ -29,7 +29,8 @@
  *   orc_pack_int4                    only times a byte-copying stand-in): these define what the device code
  *                                    must produce; checked by what the mathematics fixes (|w - q deq| <=
  *                                    deq/2, |q| <= 7, the column maximum maps to +-7, zero columns, the
- *                                    layout is a bijection with zero padding)
+ *                                    layout is a bijection with zero padding) and by answers worked
+ *                                    out by hand (ties to even, one packed dword)
  *   orc_matvec_*           pinned  — against the compiled reference MatmulVector/GemAvB
  *                                    for ceil(K/kStep) <= 4 (the reference is wrong beyond)
  *   orc_rcp14              pinned  — against the vrcp14ps instruction itself on all 2^32 inputs

@@ -145,6 +145,23 @@ def test_int4_quantiser_and_layout_properties(po):
             assert nib[idx] == (int(q[k, n]) & 0xF)
 
 
+def test_int4_known_answers(po):
+    # by hand: a column whose largest magnitude is 7 has quantisation scale 1, so q = rne(w) with ties to even,
+    # and deq = 1; the first dword of the packed column spells the nibbles out
+    col = np.array([7.0, -3.5, 2.5, 0.5, -0.5, 6.5, -7.0, 1.0] + [0.0] * 56, np.float32)
+    W = np.zeros((64, 32), np.float32)
+    W[:, 0] = col
+    W[:, 5] = col * 0.25          # the same column at another scale: same q, deq = 1/4
+    q, deq = po.quantize_int4(po.f32_to_bf16(W))
+    assert q[:8, 0].tolist() == [7, -4, 2, 0, 0, 6, -7, 1] and deq[0] == 1.0
+    assert q[:8, 5].tolist() == [7, -4, 2, 0, 0, 6, -7, 1] and deq[5] == 0.25
+    packed = po.pack_int4(q).view(np.uint32)
+    assert packed.size == 4 * 256                       # 4 fragments (K padded to 256) of 256 dwords
+    assert packed[0] == 0x196002C7                      # lane 0 (column 0, k 0..7)
+    assert packed[5 * 4] == 0x196002C7                  # lane 5 (column 5)
+    assert np.count_nonzero(packed) == 2
+
+
 def test_gemv_w8_is_exact_conversion_then_gemm(po):
     rng = np.random.default_rng(3)
     M, K, N = 3, 128, 40
