@@ -167,7 +167,7 @@ int mmx_time_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, co
  * right now, with all-zero operands (random_operands = 0) or with random ones (bf16: N(0,1) x N(0,0.02);
  * int8: uniform): *rate_out in Tflop/s or Top/s, *mhz_out the shader clock during the loop.  The clock of
  * this part under matrix load depends on the operand data; benchmarks report this next to a GEMM's rate.
- * scratch: 16 KiB of device memory.  Blocks until the loop has finished. */
+ * scratch: 16 KiB of device memory.  Blocks until the loop has finished; not thread-safe. */
 int mmx_probe_mfma(int dtype, int random_operands, int iters, void* scratch, void* stream, float* rate_out, float* mhz_out);
 
 #ifdef __cplusplus
