@@ -107,8 +107,12 @@ def dtype_code(t):
 
 
 def _row_stride_bytes(t):
-    if t.dim() != 2 or t.stride(1) != 1:
+    # torch leaves the stride of a dimension of size 1 arbitrary: a single column is contiguous whatever
+    # stride(1) says, and a single row has no row stride to speak of
+    if t.dim() != 2 or (t.stride(1) != 1 and t.shape[1] != 1):
         raise MmxError("expected a 2-D tensor with unit stride in its last dimension")
+    if t.shape[0] == 1:
+        return t.shape[1] * t.element_size()
     return t.stride(0) * t.element_size()
 
 
@@ -176,7 +180,7 @@ def quantize_pack_int4(W, transpose=False):
     """Per-output-channel symmetric int4 compression of a bf16 matrix W [K,N] (or [N,K] with transpose), packed for
     gemm(..., b_dtype=I4) with M <= 32; returns (packed uint8, deq_scales fp32 [N])."""
     _dev(W, "W")
-    if W.dtype != torch.bfloat16 or W.dim() != 2 or W.stride(1) != 1:
+    if W.dtype != torch.bfloat16 or W.dim() != 2:
         raise MmxError("W must be a 2-D bf16 tensor with unit column stride")
     K, N = (W.shape[1], W.shape[0]) if transpose else W.shape
     packed = torch.empty(packed_b_bytes(I4, K, N), dtype=torch.uint8, device=W.device)
