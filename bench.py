@@ -254,6 +254,32 @@ def main():
                             "weight_GBps": round(3.0 * wm["K"] * wm["N"] * 2 / ms / 1e6, 0)}
         extra["llama7b_mlp_fused"] = mlp
 
+        # the MLP's two GEMMs on their own, with their roofline fractions; at M=1 the weights are rotated
+        # (3 copies of gate/up = 541 MB, 6 of down) so that nothing is served from the 256 MB cache
+        from mm_amx_amd import _lib as L
+        stages = {}
+        Km, Nm = wm["K"], wm["N"]
+        gu = [L.repack_gate_up(dev_bf16(wm["w_gate"]), dev_bf16(wm["w_up"])) for _ in range(3)]
+        dn = [L.repack_b(dev_bf16(wm["w_down"]), transpose=True) for _ in range(6)]
+        for Mm in (1, 2048):
+            xm = dev_bf16(wm["x"][:Mm])
+            hm = torch.zeros((Mm, Nm), dtype=torch.bfloat16, device="cuda")
+            ym = torch.zeros((Mm, Km), dtype=torch.bfloat16, device="cuda")
+            t1 = avg_ms(xm, gu, 2 * Nm, mx.Epilogue(hm, mx.PP_SILU_GATE), 120)
+            k1 = mx.last_kernel()
+            t2 = avg_ms(hm, dn, Km, mx.Epilogue(ym, mx.PP_NONE), 120)
+            k2 = mx.last_kernel()
+            if Mm == 1:
+                stages[str(Mm)] = {
+                    "gate_up": {"us": round(t1 * 1e3, 1), "frac_of_hbm_peak": round(4.0 * Km * Nm / t1 / 1e6 / PEAK_HBM_GBS, 4), "kernel": k1},
+                    "down": {"us": round(t2 * 1e3, 1), "frac_of_hbm_peak": round(2.0 * Km * Nm / t2 / 1e6 / PEAK_HBM_GBS, 4), "kernel": k2}}
+            else:
+                stages[str(Mm)] = {
+                    "gate_up": {"us": round(t1 * 1e3, 1), "frac_of_bf16_peak": round(4.0 * Mm * Km * Nm / t1 / 1e9 / PEAK_BF16_TFLOPS, 4), "kernel": k1},
+                    "down": {"us": round(t2 * 1e3, 1), "frac_of_bf16_peak": round(2.0 * Mm * Km * Nm / t2 / 1e9 / PEAK_BF16_TFLOPS, 4), "kernel": k2}}
+        del gu, dn
+        extra["llama7b_mlp_stages"] = stages
+
         # what the matrix pipes deliver with nothing else going on: an issue-bound loop of independent MFMAs,
         # all-zero operands vs operands like the benchmark's (the clock under matrix load depends on the data)
         ceil = {}
