@@ -716,3 +716,37 @@ def test_int4_is_a_decode_path_only():
         mx.gemm(x[:4], packed, 64, mx.Epilogue(y[:4, :32], mx.PP_SILU_GATE), b_dtype=mx.I4)
     with pytest.raises(mx.MmxError):
         mx.quantize_pack_int4(torch.zeros((256, 64), dtype=torch.float32, device="cuda"))
+
+
+@pytest.mark.parametrize("M", [1, 64])
+def test_mlp_replays_from_a_hip_graph(M):
+    # the entry points allocate nothing and never synchronise, so a caller may capture them: the fused MLP (two
+    # launches) is captured once and replayed with new inputs, eager work and synchronisations in between; every
+    # replay must give the eager result
+    w = wl.llama_mlp(M=M, K=512, N=768, seed=77)
+    m = mx.MLP()
+    m.setup(dev_bf16(w["w_gate"]), dev_bf16(w["w_up"]), dev_bf16(w["w_down"]))
+    x = dev_bf16(w["x"]).clone()
+    y = torch.zeros((M, 512), dtype=torch.bfloat16, device="cuda")
+    m.run(x, y)                        # allocates the intermediate outside the capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        m.run(x, y)                    # warm-up on the capture stream
+        side.synchronize()
+        with torch.cuda.graph(g, stream=side):
+            m.run(x, y)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(5)
+    for rep in range(4):
+        x.copy_(dev_bf16(rand_bf16(rng, (M, 512), 1.0)))
+        y.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        got = host_bits(y).copy()
+        y2 = torch.zeros_like(y)
+        m.run(x, y2)                   # eager, between the replays
+        torch.cuda.synchronize()
+        assert np.array_equal(got, host_bits(y2)), rep
