@@ -214,6 +214,18 @@ def main():
             del packs, Wg
         extra["decode_gemv_int8w_K4096_N11008"] = gemv
 
+        # int8 activations x int8 weights at M=1 (int32 sums), same weights and rotation
+        w8b = wl.decode_gemv_w8(M=1)
+        Wi = mx.repack_b(dev(w8b["W"]))
+        packs = [Wi] + [Wi.clone() for _ in range(11)]
+        xi = torch.randint(-127, 128, (1, w8b["K"]), dtype=torch.int8, device="cuda")
+        yi = torch.zeros((1, w8b["N"]), dtype=torch.bfloat16, device="cuda")
+        ms = avg_ms(xi, packs, w8b["N"], mx.Epilogue(yi, mx.PP_DEQUANT, deq_scale_per_oc=dev(w8b["scale"])), 240)
+        extra["decode_gemv_int8x_int8w_K4096_N11008"] = {"1": {
+            "us": round(ms * 1e3, 2), "weight_GBps": round(float(w8b["K"]) * w8b["N"] / ms / 1e6, 0),
+            "frac_of_hbm_peak": round(float(w8b["K"]) * w8b["N"] / ms / 1e6 / PEAK_HBM_GBS, 4), "kernel": mx.last_kernel()}}
+        del packs, Wi
+
         # the same GEMV over int4-compressed weights (22.5 MB), rotating over 24 copies (541 MB)
         gemv4 = {}
         wg = wl.decode_gemv_w8(M=4)

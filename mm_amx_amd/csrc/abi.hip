@@ -35,6 +35,7 @@ int launch_gemm_tiles_bf16(const void* A, int64_t lda, const void* Bp, int M, in
                            const Epilogue& ep, hipStream_t st);
 int launch_gemm_tiles_i8(const void* A, int64_t lda, const void* Bp, int M, int K, int N, int n0, int n1,
                          const Epilogue& ep, hipStream_t st);
+bool skinny_i8_eligible(const void* x, int64_t ldx, int M, int K);
 int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
                   const Epilogue& ep, hipStream_t st);
 int launch_repack(int elesz, const void* B, int64_t ldb, int K, int N, int transpose, void* out, hipStream_t st);
@@ -123,6 +124,8 @@ static int gemm_dispatch(int a_dtype, int b_dtype, const void* A, int64_t lda_by
     if (rc) return rc;
     if ((ep.steps & MMX_PP_SILU_GATE) && ((n1 - n0) % 64)) return set_error(MMX_E_INVALID, "mmx_gemm: SILU_GATE needs (n1 - n0) %% 64 == 0");
     if (M <= 32 && !i8) return launch_skinny(w4 ? 2 : (w8 ? 1 : 0), A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st);
+    if (i8 && skinny_i8_eligible(A, lda_bytes, M, K) && forced_tile().bm == 0)
+        return launch_skinny(3, A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st);
     if (w4) return set_error(MMX_E_UNSUPPORTED, "mmx_gemm: bf16 x int4-weight is a decode path (M <= 32)");
     if (w8) return set_error(MMX_E_UNSUPPORTED, "mmx_gemm: bf16 x int8-weight with M > 32: convert the weights with mmx_dequant_packed and call the bf16 GEMM");
     return i8 ? launch_gemm_tiles_i8(A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st)

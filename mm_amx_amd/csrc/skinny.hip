@@ -114,7 +114,7 @@ __device__ __forceinline__ void skinny_prefetch(const SkinnyArgs& s, int panel_f
 }
 
 // cross-wave reduction of the partial 32x32 blocks + post-op + store (shared by the 8-wave decode kernels)
-template <int NP>
+template <int NP, bool ISUM = false>  // ISUM: the partial sums are int32 (int8 activations), stored as bits
 __device__ __forceinline__ void skinny_finish(const SkinnyArgs& s, const float (&red)[8][NP][16][64], int panel_first, int tid,
                                               const FinishOperands<NP>& o) {
     const Epilogue& ep = s.ep;
@@ -126,14 +126,29 @@ __device__ __forceinline__ void skinny_finish(const SkinnyArgs& s, const float (
         if (m >= s.M) continue;
         const int nloc = 8 * (v >> 2) + 4 * (ln >> 5) + (v & 3);
         float sum[NP];
+        int isum[NP];
 #pragma unroll
         for (int p = 0; p < NP; p++) {
-            float acc = 0.0f;
+            if constexpr (ISUM) {
+                int acc = 0;
 #pragma unroll
-            for (int w8 = 0; w8 < 8; w8++) acc += red[w8][p][v][ln];
-            sum[p] = acc;
+                for (int w8 = 0; w8 < 8; w8++) acc += reinterpret_cast<const int*>(&red[w8][p][v][ln])[0];
+                isum[p] = acc;
+                sum[p] = (float)acc;  // vcvtdq2ps, round to nearest even (include/kernels_amx.hpp:631-634)
+            } else {
+                float acc = 0.0f;
+#pragma unroll
+                for (int w8 = 0; w8 < 8; w8++) acc += red[w8][p][v][ln];
+                sum[p] = acc;
+            }
         }
-        if (ep.steps & MMX_PP_SILU_GATE) {
+        if (ISUM && ep.out_dtype == MMX_I32) {  // raw accumulators (steps == 0)
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                const int n = ((panel_first + p) << 5) + nloc;
+                if (n < s.n1) reinterpret_cast<int*>(ep.C + (int64_t)m * ep.ldc)[n] = isum[p];
+            }
+        } else if (ep.steps & MMX_PP_SILU_GATE) {
             if constexpr (NP == 2) {
                 const int n = ((panel_first >> 1) << 5) + nloc;  // output column (half width)
                 if (n < (s.n1 >> 1)) store_out(ep, m, n, silu(sum[0]) * sum[1]);
@@ -484,7 +499,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 // each kernel holds one code path and stays within its registers.
 template <int WK, int NP, bool ONE>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void skinny_stream_kernel(const SkinnyArgs s, int zero_off) {
-    constexpr bool W8 = WK == 1, W4 = WK == 2;
+    constexpr bool W8 = WK == 1, W4 = WK == 2, I8A = WK == 3;  // 3: int8 weights AND int8 activations, int32 sums
+    using accv = std::conditional_t<I8A, i32x16, f32x16>;
     // fragments per panel per wave in flight at once (16 KiB of weights; int4: 8 KiB, a fragment holds 64 of k
     // and unpacking it costs more than streaming it)
     constexpr int U = (W4 ? 8 : 16) / NP;
@@ -496,7 +512,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const int l32 = lane & 31, g32 = lane >> 5;
     const int panel_first = (s.n0 >> 5) + blockIdx.x * NP;
     const int panel_end = (s.n1 + 31) >> 5;
-    const int row_bytes = s.K * 2;
+    const int row_bytes = s.K * (I8A ? 1 : 2);
     const int real_bytes = s.M * row_bytes;
 
     // x -> LDS, 1 KiB per wave per instruction; the lanes past the end of x re-read its last 16 bytes
@@ -518,11 +534,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     skinny_prefetch<NP>(s, panel_first, tid, fin);
     __builtin_amdgcn_sched_barrier(0);
 
-    f32x16 acc[NP];
+    accv acc[NP];
 #pragma unroll
     for (int p = 0; p < NP; p++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) acc[p][v] = 0.0f;
+        for (int v = 0; v < 16; v++) acc[p][v] = 0;
 
     // wave w multiplies fragments [w*per_wave, (w+1)*per_wave); indices past the end are clamped for the
     // load and paired with the zero row of x
@@ -555,7 +571,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         const bool valid_ = (f_ - f_begin) < per_wave && f_ <= f_last; /* scalar */                             \
         const int fc_ = f_ < f_last ? f_ : f_last;                                                              \
         const char* xr_ = valid_ ? xrow : zrow;                                                                 \
-        if constexpr (W4) {                                                                                     \
+        if constexpr (I8A) {                                                                                    \
+            const i32x4 xq_ = *reinterpret_cast<const i32x4*>(xr_ + 32 * fc_ + 16 * g32);                       \
+            _Pragma("unroll") for (int p = 0; p < NP; p++)                                                      \
+                acc[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, w[p][UU]), xq_, acc[p], 0, 0, 0); \
+        } else if constexpr (W4) {                                                                              \
             _Pragma("unroll") for (int i_ = 0; i_ < 4; i_++) {                                                  \
                 const bf16x8 xq_ = *reinterpret_cast<const bf16x8*>(xr_ + (64 * fc_ + 32 * g32 + 8 * i_) * 2);  \
                 _Pragma("unroll") for (int p = 0; p < NP; p++)                                                  \
@@ -608,9 +628,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #pragma unroll
     for (int p = 0; p < NP; p++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) red[wave][p][v][lane] = W4 ? acc[p][v] * 16.0f : acc[p][v];  // int4 operands were q / 16
+        for (int v = 0; v < 16; v++) {
+            if constexpr (I8A) reinterpret_cast<int*>(&red[wave][p][v][lane])[0] = acc[p][v];  // the sums travel as bits
+            else red[wave][p][v][lane] = W4 ? acc[p][v] * 16.0f : acc[p][v];  // int4 operands were q / 16
+        }
     __syncthreads();
-    skinny_finish<NP>(s, red, panel_first, tid, fin);
+    skinny_finish<NP, I8A>(s, red, panel_first, tid, fin);
 }
 
 // Half-panel variant of the streaming kernel for 1-2 rows of x.  A list of 32-column panels that is only 1-2
@@ -800,7 +823,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 
 int decode_halves();
 
-// wk: weights are bf16 (0), int8 (1) or int4 (2)
+// int8 x int8 at M <= 32 can use the streaming decode kernel if x fits in LDS, is 16-byte aligned and K fills whole
+// 128-byte groups of the packed weights
+bool skinny_i8_eligible(const void* x, int64_t ldx, int M, int K) {
+    const int zoff = (M * K + 1023) & ~1023;
+    return M <= 32 && K % 128 == 0 && zoff + K <= 46 * 1024 && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) && ((ldx & 15) == 0);
+}
+
+// wk: weights are bf16 (0), int8 (1) or int4 (2); 3: int8 weights and int8 activations
 int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
                   const Epilogue& ep, hipStream_t st) {
     const bool w8 = wk == 1;
@@ -810,7 +840,7 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
     s.Wp = static_cast<const char*>(Wp);
     s.M = M;
     s.K = K;
-    const int kbytes_pad = ((K * (w8 ? 1 : 2)) + 127) / 128 * 128;
+    const int kbytes_pad = ((K * ((wk == 1 || wk == 3) ? 1 : 2)) + 127) / 128 * 128;
     s.nfrag = wk == 2 ? (K + 255) / 256 * 4 : kbytes_pad / 32;  // 32 bytes of K per column per fragment
     s.panel_stride = (int64_t)s.nfrag * 1024;
     s.npanels = (N + 31) / 32;
@@ -820,6 +850,17 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
     s.ep = ep;
     const int panels = ((n1 + 31) >> 5) - (n0 >> 5);
     const bool pairs = (ep.steps & MMX_PP_SILU_GATE) != 0;
+    if (wk == 3) {
+        // int8 activations x int8 weights (int32 sums): only the streaming form exists; the caller has checked
+        // skinny_i8_eligible and uses the tile kernel otherwise
+        const int zoff = (M * K + 1023) & ~1023;
+        note_kernel("skinny_stream_i8");
+        if ((s.nfrag + 7) / 8 <= 16)
+            hipLaunchKernelGGL((skinny_stream_kernel<3, 1, true>), dim3(panels), dim3(512), zoff + K, st, s, zoff);
+        else
+            hipLaunchKernelGGL((skinny_stream_kernel<3, 1, false>), dim3(panels), dim3(512), zoff + K, st, s, zoff);
+        return check_hip(hipGetLastError(), "skinny_stream_kernel launch");
+    }
     if (wk == 2) {
         // int4 weights: the streaming kernel if x fits in LDS and K fills whole fragments, else the general one
         if (pairs) return set_error(MMX_E_UNSUPPORTED, "SILU_GATE over int4 weights is not built");

@@ -750,3 +750,43 @@ def test_mlp_replays_from_a_hip_graph(M):
         m.run(x, y2)                   # eager, between the replays
         torch.cuda.synchronize()
         assert np.array_equal(got, host_bits(y2)), rep
+
+
+# ---- int8 activations at M <= 32: the streaming decode form (int32 sums, order-free) --------------------------
+@pytest.mark.parametrize("shape", [(1, 128, 64), (5, 1024, 100), (32, 1152, 192), (4, 4096, 352), (9, 4096, 33),
+                                   (2, 8192, 96)])
+def test_int8_decode_form(po, shape):
+    M, K, N = shape
+    rng = np.random.default_rng(3 * sum(shape))
+    A = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    deq = (np.float32(0.02) * rng.uniform(1e-3, 1e-2, N).astype(np.float32)).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    qoc = rng.uniform(5, 40, N).astype(np.float32)
+    acc_ref = po.gemm_i8(A, B)
+    packed = mx.repack_b(dev(B))
+    wide = torch.zeros((M, K + 16), dtype=torch.int8, device="cuda")    # a padded (16-byte aligned) row stride
+    wide[:, :K] = dev(A)
+    Ad = wide[:, :K]
+    eligible = (M * K + 1023) // 1024 * 1024 + K <= 46 * 1024
+    n0, n1 = (32, N - 3) if N > 96 else (0, N)
+    C = torch.full((M, N), -7, dtype=torch.int32, device="cuda")
+    mx.gemm(Ad, packed, N, mx.Epilogue(C, mx.PP_NONE), n0=n0, n1=n1)
+    assert (mx.last_kernel() == "skinny_stream_i8") == eligible, (mx.last_kernel(), shape)
+    got = host_bits(C)
+    assert np.array_equal(got[:, n0:n1], acc_ref[:, n0:n1])
+    assert np.all(got[:, :n0] == -7) and np.all(got[:, n1:] == -7)
+    # every post-op step, int8 and bf16 stores
+    out8 = torch.zeros((M, N), dtype=torch.int8, device="cuda")
+    mx.gemm(Ad, packed, N, mx.Epilogue(out8, 15, bias=dev(bias), deq_scale_per_oc=dev(deq), q_scale_per_oc=dev(qoc)))
+    assert np.array_equal(host_bits(out8), po.pp(acc_ref, 15, po.I8, bias=bias, deq_per_oc=deq, q_per_oc=qoc))
+    outb = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    mx.gemm(Ad, packed, N, mx.Epilogue(outb, mx.PP_DEQUANT | mx.PP_BIAS, bias=dev(bias), deq_scale_per_oc=dev(deq)))
+    assert np.array_equal(host_bits(outb), po.pp(acc_ref, po.PP_DEQUANT | po.PP_BIAS, po.BF16, bias=bias, deq_per_oc=deq))
+    # an unaligned x falls back to the tile kernels with the same result
+    odd = torch.zeros((M, K + 3), dtype=torch.int8, device="cuda")
+    odd[:, :K] = dev(A)
+    C2 = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    mx.gemm(odd[:, :K], packed, N, mx.Epilogue(C2, mx.PP_NONE))
+    assert "skinny" not in mx.last_kernel() or M == 1
+    assert np.array_equal(host_bits(C2), acc_ref)
