@@ -27,11 +27,11 @@ PEAK_INT8_TOPS = 5000.0     # MI355X dense int8 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # HBM-side bytes per launch of the headline kernel, from two counter runs of this script under
-# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (KiB per dispatch: 81969 and 27913), each scaled by
+# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (KiB per dispatch: 81969 and 27915), each scaled by
 # what the same counter reads for the 256 MiB device copy of --calibrate-copy (factors 2.000 and 1.000);
 # the summary is profiles/gemm_bf16_256x192_ffn_up_M1024_hbm_traffic.txt.  Counters cannot be read from
 # inside the process, so the figure is only reported when the kernel that ran is the one profiled.
-MEASURED_TRAFFIC_BYTES = {"gemm_bf16_256x192_ring_out_bf16": (81969 * 2.000 + 27913 * 1.000) * 1024}
+MEASURED_TRAFFIC_BYTES = {"gemm_bf16_256x192_ring_out_bf16": (81969 * 2.000 + 27915 * 1.000) * 1024}
 
 
 def main():
