@@ -374,6 +374,44 @@ struct Matmul<bfloat16, int8_t, float> {
     }
 };
 
+// Decode-path Matmul over int4-compressed weights.  The reference has no such class: it only times a stand-in
+// that copies bytes in place of an int4 dequant (weight_compression/wcompress.hpp:90-134).  Same call shape as
+// Matmul<bfloat16, int8_t, float>: takes the bf16 weights, compresses them per output channel to [-7, 7] at the
+// first call and points the post-op's dequant step at the per-channel scales.  M <= 32 only.
+struct MatmulW4 {
+    device_vector<uint8_t> internalB4;      // packed nibbles
+    device_vector<float> dequant_scales_B;  // [N]
+    bool constB;
+    bool transposeB;
+
+    MatmulW4(bool constB = false, bool transposeB = false) : constB(constB), transposeB(transposeB) {}
+
+    template <typename P>
+    void operator()(tensor2D<bfloat16>& matA, tensor2D<bfloat16>& matB, P ppkernel, hipStream_t stream = nullptr) {
+        (*this)(matA, matB, 0, matB.dims[transposeB ? 0 : 1], ppkernel, stream);
+    }
+
+    template <typename P>
+    void operator()(tensor2D<bfloat16>& matA, tensor2D<bfloat16>& matB, int n0, int n1, P ppkernel,
+                    hipStream_t stream = nullptr) {
+        const int M = matA.dims[0], K = matA.dims[1];
+        const int N = matB.dims[transposeB ? 0 : 1];
+        require(K == matB.dims[transposeB ? 1 : 0], "MatmulW4: K of A and B differ");
+        require(M <= 32, "MatmulW4: int4 weights are a decode path (M <= 32)");
+        if (!constB || !internalB4.data) {
+            // (freeing the previous buffers waits for the launches that still read them)
+            internalB4 = device_vector<uint8_t>(mmx_packed_b_bytes(MMX_I4, K, N));
+            dequant_scales_B = device_vector<float>(N);
+            check(mmx_quantize_pack_int4(matB.data, matB.stride, K, N, transposeB ? 1 : 0, internalB4.data,
+                                         dequant_scales_B.data, stream),
+                  "MatmulW4: quantize");
+        }
+        ppkernel.set_deq_scale(dequant_scales_B.data);
+        const mmx_epilogue e = ppkernel.descriptor();
+        check(mmx_gemm(MMX_BF16, MMX_I4, matA.data, matA.stride, internalB4.data, M, K, N, n0, n1, &e, stream), "MatmulW4");
+    }
+};
+
 // ---- MatmulVector (include/kernels_amx.hpp:833-1043): c[M] = A[M, K] · b[K] ------------------------
 // vB and vC are device pointers.  The reference admits kStep <= K <= 6 kStep (966); this kernel
 // takes any K >= 1, the same bounds are not enforced.

@@ -200,6 +200,33 @@ static void test_matmul_weight_int8(int M, int K, int N) {
     EXPECT(e.fro <= 1e-3 && e.within >= 0.999, "rel Frobenius %.3e, %.3f%% within 1 bf16 ulp", e.fro, e.within * 100);
 }
 
+// ---- MatmulW4: int4 weight compression inside the op (no reference counterpart beyond a timing stand-in) ----
+static void test_matmul_weight_int4(int M, int K, int N) {
+    std::printf("  MatmulW4 (weights compressed to int4 per output channel) M=%d K=%d N=%d\n", M, K, N);
+    auto hA = rand_bf16(static_cast<size_t>(M) * K, 1.0f), hB = rand_bf16(static_cast<size_t>(K) * N, 0.05f);
+    tensor2D<bfloat16> A(M, K), B(K, N);
+    tensor2D<float> C(M, N);
+    A.upload(hA.data());
+    B.upload(hB.data());
+    MatmulW4 mm(true, false);
+    mm(A, B, PP::BiasGeluStore<float, PP::DEQUANT>(C));
+    mm(A, B, PP::BiasGeluStore<float, PP::DEQUANT>(C));  // second call: the cached packed weights
+    check_hip(hipDeviceSynchronize(), "sync");
+    std::vector<float> got(static_cast<size_t>(M) * N);
+    C.download(got.data());
+
+    std::vector<int8_t> q(static_cast<size_t>(K) * N);
+    std::vector<float> deq(N);
+    orc_quantize_int4(bits(hB), N, K, N, 0, q.data(), deq.data());
+    EXPECT(mm.dequant_scales_B.to_host() == deq, "per-channel scales differ from the definition");
+    std::vector<float> acc(got.size()), ref(got.size()), ones(N, 1.0f);
+    std::vector<uint16_t> ydummy(got.size());
+    orc_gemv_w8(bits(hA), K, q.data(), N, 0, ones.data(), ydummy.data(), N, acc.data(), M, K, N, 0);
+    for (size_t i = 0; i < ref.size(); i++) ref[i] = acc[i] * deq[i % N];
+    const Err e = compare(got, ref);
+    EXPECT(e.fro <= 1e-3 && e.within >= 0.999, "rel Frobenius %.3e, %.3f%% within 1 bf16 ulp", e.fro, e.within * 100);
+}
+
 // ---- MatmulVector / GemAvB, reference shapes main.cpp:884-885 ----
 static void test_matvec(int M, int K) {
     std::printf("  MatmulVector / GemAvB M=%d K=%d\n", M, K);
@@ -319,6 +346,8 @@ int main() {
         test_matmul_i8_requant(77, 200, 95);
         test_matmul_weight_int8(2, 2560, 192);  // fc16m.cpp:749
         test_matmul_weight_int8(160, 512, 256);
+        test_matmul_weight_int4(1, 4096, 352);
+        test_matmul_weight_int4(7, 300, 77);
         test_matvec(901, 80);  // main.cpp:884
         test_matvec(901, 96);  // main.cpp:885
         test_linear_nxn(32, 32, 32);  // torch-ext/test.py:35
