@@ -365,10 +365,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 // the row so that the 32 rows an operand reads spread over the banks.
 // Lanes of rows >= M read row 0 (their output columns are never stored); fragments past the end of K
 // get zero weights and a clamped (finite) x.
-template <bool W8, int NP, int FPW, int XD>  // XD: 16-byte x loads per thread per chunk (8 KiB of x each)
+// WK: weights are bf16 (0), int8 (1) or int4 (2); XD: 16-byte x loads per thread per chunk (8 KiB of x each)
+template <int WK, int NP, int FPW, int XD>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void skinny_chunk_kernel(const SkinnyArgs s) {
-    constexpr int W = (FPW == 2 && (W8 || NP == 2)) ? 2 : 3;  // chunks in flight (what 128 registers hold)
-    constexpr int XB = W8 ? 64 : 32;     // bytes of a row of x one fragment covers
+    constexpr bool W8 = WK == 1, W4 = WK == 2;
+    // chunks in flight (what 128 registers hold)
+    constexpr int W = W4 ? (XD >= 4 ? 2 : 3) : ((FPW == 2 && (W8 || NP == 2)) ? 2 : 3);
+    constexpr int XB = W4 ? 128 : (W8 ? 64 : 32);  // bytes of a row of x one fragment covers
     constexpr int FC = 8 * FPW;          // fragments per chunk
     constexpr int RB = FC * XB;          // bytes of a row of x per chunk
     constexpr int BUF = 8 * XD * 1024;   // one LDS buffer: BUF / RB rows of x (the launcher checks M against it)
@@ -443,7 +446,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             const int fl_ = wave * FPW + u;                                                                    \
             const bool valid_ = (C) * FC + fl_ <= f_last; /* scalar */                                         \
             const char* xb_ = xread + ((C) & 1) * BUF;                                                         \
-            if constexpr (W8) {                                                                                \
+            if constexpr (W4) {                                                                                \
+                const int c0_ = fl_ * 8 + g32 * 4;                                                             \
+                _Pragma("unroll") for (int i_ = 0; i_ < 4; i_++) {                                             \
+                    const bf16x8 xq_ = *reinterpret_cast<const bf16x8*>(xb_ + (((c0_ + i_) ^ xswz) * 16));     \
+                    _Pragma("unroll") for (int p = 0; p < NP; p++) {                                           \
+                        const u32x4 wv_ = valid_ ? w[J][u][p] : u32x4{0u, 0u, 0u, 0u};                         \
+                        acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s4x8_to_bf16_div16(wv_[i_]), xq_, acc[p], 0, 0, 0); \
+                    }                                                                                          \
+                }                                                                                              \
+            } else if constexpr (W8) {                                                                         \
                 const int c0_ = fl_ * 4 + g32 * 2;                                                             \
                 const bf16x8 xa_ = *reinterpret_cast<const bf16x8*>(xb_ + ((c0_ ^ xswz) * 16));                \
                 const bf16x8 xc_ = *reinterpret_cast<const bf16x8*>(xb_ + (((c0_ + 1) ^ xswz) * 16));          \
@@ -490,7 +502,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #pragma unroll
     for (int p = 0; p < NP; p++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) red[wave][p][v][lane] = acc[p][v];
+        for (int v = 0; v < 16; v++) red[wave][p][v][lane] = W4 ? acc[p][v] * 16.0f : acc[p][v];  // int4 operands were q / 16
     __syncthreads();
     skinny_finish<NP>(s, red, panel_first, tid, fin);
 }
@@ -883,6 +895,13 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
             else
                 hipLaunchKernelGGL((skinny_stream_kernel<2, 1, false>), dim3(panels), dim3(512), xb, st, s, zoff);
             return check_hip(hipGetLastError(), "skinny_stream_kernel launch");
+        }
+        if (s.nfrag * 64 == K && s.x_vec_ok) {
+            // x too large for LDS: through LDS chunk by chunk (two buffers of 16 or 32 rows x 1 KiB)
+            note_kernel("skinny_chunk_w4");
+            if (M <= 16) hipLaunchKernelGGL((skinny_chunk_kernel<2, 1, 1, 2>), dim3(panels), dim3(512), 2 * 8 * 2 * 1024, st, s);
+            else hipLaunchKernelGGL((skinny_chunk_kernel<2, 1, 1, 4>), dim3(panels), dim3(512), 2 * 8 * 4 * 1024, st, s);
+            return check_hip(hipGetLastError(), "skinny_chunk_kernel launch");
         }
         note_kernel("skinny_w4");
         hipLaunchKernelGGL((skinny_kernel<2, 1>), dim3(panels), dim3(512), 0, st, s);

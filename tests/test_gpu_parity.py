@@ -665,7 +665,8 @@ def test_int4_quantise_and_pack_match_the_definition(po, shape, transpose):
     assert np.array_equal(host_bits(packed), want)
 
 
-@pytest.mark.parametrize("shape", [(1, 256, 64), (3, 320, 100), (16, 337, 96), (32, 2560, 192), (2, 4096, 352), (4, 8192, 64)])
+@pytest.mark.parametrize("shape", [(1, 256, 64), (3, 320, 100), (16, 337, 96), (32, 2560, 192), (2, 4096, 352), (4, 8192, 64),
+                                   (8, 4096, 352), (20, 1024, 100), (16, 11008, 64)])
 def test_int4_decode_shapes(po, shape):
     M, K, N = shape
     rng = np.random.default_rng(sum(shape))
@@ -681,6 +682,7 @@ def test_int4_decode_shapes(po, shape):
     assert "w4" in mx.last_kernel()
     stream_ok = K % 256 == 0 and (M + 1) * K * 2 <= 45 * 1024
     assert ("stream" in mx.last_kernel()) == stream_ok, (mx.last_kernel(), shape)
+    assert ("chunk" in mx.last_kernel()) == (K % 256 == 0 and not stream_ok), (mx.last_kernel(), shape)
     acc_gpu = torch.zeros((M, N), dtype=torch.float32, device="cuda")
     mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc_gpu, mx.PP_NONE), b_dtype=mx.I4)
     check_float_parity(host_bits(acc_gpu), acc_ref, f"int4 decode accumulators {shape}")
