@@ -262,7 +262,8 @@ __global__ __launch_bounds__(512) void skinny_kernel(const SkinnyArgs s) {
     skinny_finish<NP>(s, red, panel_first, tid, fin);
 }
 
-// ---- direct variant for aligned operands whose x does not fit in LDS, few rows (4 < M <= 8) ----------
+// ---- direct variant for aligned operands whose x does not fit in LDS, few rows (4 < M <= 8); launched for
+// plain bf16 weights only (for int8 weights and gate/up pairs the chunked variant below measured faster) ----
 // Every lane reads its own 16 (bf16 weights) or 32 (int8 weights) bytes of x per fragment straight from
 // global memory (served by L2: all workgroups read the same x) together with the fragment, U of
 // them in flight per wave as a rolling window.  Lanes of rows >= M read row 0: in the MFMA an output
@@ -944,13 +945,11 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
 #undef MMX_STREAM
         return check_hip(hipGetLastError(), "skinny_stream_kernel launch");
     }
-    if (kpad == K && s.x_vec_ok && !(pairs && w8) && M <= 8) {
-        // aligned, x too large for LDS, few rows: every lane reads its own part of x
-        if (pairs && (panels & 1)) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
-        note_kernel(pairs ? "skinny_direct_bf16_gateup" : (w8 ? "skinny_direct_w8" : "skinny_direct_bf16"));
-        if (pairs) hipLaunchKernelGGL((skinny_direct_kernel<false, 2>), dim3(panels / 2), dim3(512), 0, st, s);
-        else if (w8) hipLaunchKernelGGL((skinny_direct_kernel<true, 1>), dim3(panels), dim3(512), 0, st, s);
-        else hipLaunchKernelGGL((skinny_direct_kernel<false, 1>), dim3(panels), dim3(512), 0, st, s);
+    if (kpad == K && s.x_vec_ok && !w8 && !pairs && M <= 8) {
+        // aligned, x too large for LDS, few rows, plain bf16 weights: every lane reads its own part of x
+        // (measured: for int8 weights and for gate/up pairs the chunked kernel below is faster at these M too)
+        note_kernel("skinny_direct_bf16");
+        hipLaunchKernelGGL((skinny_direct_kernel<false, 1>), dim3(panels), dim3(512), 0, st, s);
         return check_hip(hipGetLastError(), "skinny_direct_kernel launch");
     }
     if (kpad == K && s.x_vec_ok && !(pairs && w8)) {
