@@ -366,13 +366,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 // the row so that the 32 rows an operand reads spread over the banks.
 // Lanes of rows >= M read row 0 (their output columns are never stored); fragments past the end of K
 // get zero weights and a clamped (finite) x.
-// WK: weights are bf16 (0), int8 (1) or int4 (2); XD: 16-byte x loads per thread per chunk (8 KiB of x each)
+// WK: weights are bf16 (0), int8 (1) or int4 (2), 3: int8 weights and int8 activations (int32 sums);
+// XD: 16-byte x loads per thread per chunk (8 KiB of x each)
 template <int WK, int NP, int FPW, int XD>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void skinny_chunk_kernel(const SkinnyArgs s) {
-    constexpr bool W8 = WK == 1, W4 = WK == 2;
+    constexpr bool W8 = WK == 1, W4 = WK == 2, I8A = WK == 3;
+    using accv = std::conditional_t<I8A, i32x16, f32x16>;
     // chunks in flight (what 128 registers hold)
     constexpr int W = W4 ? (XD >= 4 ? 2 : 3) : ((FPW == 2 && (W8 || NP == 2)) ? 2 : 3);
-    constexpr int XB = W4 ? 128 : (W8 ? 64 : 32);  // bytes of a row of x one fragment covers
+    constexpr int XB = W4 ? 128 : (W8 ? 64 : 32);  // bytes of a row of x one fragment covers (int8 x int8: 32)
     constexpr int FC = 8 * FPW;          // fragments per chunk
     constexpr int RB = FC * XB;          // bytes of a row of x per chunk
     constexpr int BUF = 8 * XD * 1024;   // one LDS buffer: BUF / RB rows of x (the launcher checks M against it)
@@ -390,15 +392,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     FinishOperands<NP> fin;
     skinny_prefetch<NP>(s, panel_first, tid, fin);
 
-    f32x16 acc[NP];
+    accv acc[NP];
 #pragma unroll
     for (int p = 0; p < NP; p++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) acc[p][v] = 0.0f;
+        for (int v = 0; v < 16; v++) acc[p][v] = 0;
 
     const int f_last = s.nfrag - 1;
     const int nchunk = (s.nfrag + FC - 1) / FC;
-    const int row_bytes = s.K * 2;
+    const int row_bytes = s.K * (I8A ? 1 : 2);
     const char* wbase[NP];
 #pragma unroll
     for (int p = 0; p < NP; p++) {
@@ -447,7 +449,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             const int fl_ = wave * FPW + u;                                                                    \
             const bool valid_ = (C) * FC + fl_ <= f_last; /* scalar */                                         \
             const char* xb_ = xread + ((C) & 1) * BUF;                                                         \
-            if constexpr (W4) {                                                                                \
+            if constexpr (I8A) {                                                                               \
+                const int c0_ = fl_ * 2 + g32;                                                                 \
+                const i32x4 xq_ = *reinterpret_cast<const i32x4*>(xb_ + ((c0_ ^ xswz) * 16));                  \
+                _Pragma("unroll") for (int p = 0; p < NP; p++) {                                               \
+                    const u32x4 wv_ = valid_ ? w[J][u][p] : u32x4{0u, 0u, 0u, 0u};                             \
+                    acc[p] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, wv_), xq_, acc[p], 0, 0, 0); \
+                }                                                                                              \
+            } else if constexpr (W4) {                                                                         \
                 const int c0_ = fl_ * 8 + g32 * 4;                                                             \
                 _Pragma("unroll") for (int i_ = 0; i_ < 4; i_++) {                                             \
                     const bf16x8 xq_ = *reinterpret_cast<const bf16x8*>(xb_ + (((c0_ + i_) ^ xswz) * 16));     \
@@ -503,9 +512,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #pragma unroll
     for (int p = 0; p < NP; p++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) red[wave][p][v][lane] = W4 ? acc[p][v] * 16.0f : acc[p][v];  // int4 operands were q / 16
+        for (int v = 0; v < 16; v++) {
+            if constexpr (I8A) reinterpret_cast<int*>(&red[wave][p][v][lane])[0] = acc[p][v];  // the sums travel as bits
+            else red[wave][p][v][lane] = W4 ? acc[p][v] * 16.0f : acc[p][v];  // int4 operands were q / 16
+        }
     __syncthreads();
-    skinny_finish<NP>(s, red, panel_first, tid, fin);
+    skinny_finish<NP, I8A>(s, red, panel_first, tid, fin);
 }
 
 // ---- streaming variant for the smallest M -----------------------------------------------------------
@@ -846,11 +858,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 
 int decode_halves();
 
-// int8 x int8 at M <= 32 can use the streaming decode kernel if x fits in LDS, is 16-byte aligned and K fills whole
-// 128-byte groups of the packed weights
+// int8 x int8 at M <= 32 can use the decode kernels if x is 16-byte aligned and K fills whole 128-byte groups of
+// the packed weights: the streaming form if x fits in LDS, else the chunked one, which walks K in chunks of 256
 bool skinny_i8_eligible(const void* x, int64_t ldx, int M, int K) {
     const int zoff = (M * K + 1023) & ~1023;
-    return M <= 32 && K % 128 == 0 && zoff + K <= 46 * 1024 && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) && ((ldx & 15) == 0);
+    return M <= 32 && K % 128 == 0 && (zoff + K <= 46 * 1024 || K % 256 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
+           ((ldx & 15) == 0);
 }
 
 // wk: weights are bf16 (0), int8 (1) or int4 (2); 3: int8 weights and int8 activations
@@ -874,9 +887,14 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
     const int panels = ((n1 + 31) >> 5) - (n0 >> 5);
     const bool pairs = (ep.steps & MMX_PP_SILU_GATE) != 0;
     if (wk == 3) {
-        // int8 activations x int8 weights (int32 sums): only the streaming form exists; the caller has checked
-        // skinny_i8_eligible and uses the tile kernel otherwise
+        // int8 activations x int8 weights (int32 sums): the caller has checked skinny_i8_eligible and uses the tile
+        // kernel otherwise
         const int zoff = (M * K + 1023) & ~1023;
+        if (zoff + K > 46 * 1024) {  // x does not fit in LDS: through LDS chunk by chunk (32 rows x 256 bytes per buffer)
+            note_kernel("skinny_chunk_i8");
+            hipLaunchKernelGGL((skinny_chunk_kernel<3, 1, 1, 1>), dim3(panels), dim3(512), 8 * 1 * 16 * 64 * 4, st, s);
+            return check_hip(hipGetLastError(), "skinny_chunk_kernel launch");
+        }
         note_kernel("skinny_stream_i8");
         if ((s.nfrag + 7) / 8 <= 16)
             hipLaunchKernelGGL((skinny_stream_kernel<3, 1, true>), dim3(panels), dim3(512), zoff + K, st, s, zoff);
