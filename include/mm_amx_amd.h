@@ -153,7 +153,7 @@ const char* mmx_last_kernel(void);
  * 2 (default) direct HBM->LDS loads in a hand-scheduled ring pipeline, 0 through registers (the
  * fallback for operands beyond 32-bit offsets).  Shapes whose K tail or alignment need masked
  * loads use a masked kernel whatever this is set to.  "decode_halves": whether the streaming decode
- * kernel for M <= 2 splits every 32-column panel over two workgroups — -1 (default) where that fills the
+ * kernel for M <= 4 splits every 32-column panel over two workgroups — -1 (default) where that fills the
  * CUs better, 0 never, 1 always (the two forms add the partial sums in different orders). */
 int mmx_set_option(const char* name, int value);
 /* HIP-event timing of `iters` back-to-back launches of the given gemm on `stream`, launch i

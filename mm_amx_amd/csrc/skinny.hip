@@ -671,7 +671,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     skinny_finish<NP, I8A>(s, red, panel_first, tid, fin);
 }
 
-// Half-panel variant of the streaming kernel for 1-2 rows of x.  A list of 32-column panels that is only 1-2
+// Half-panel variant of the streaming kernel for 1-4 rows of x.  A list of 32-column panels that is only 1-2
 // per CU long leaves some CUs with twice the work of others (or idle), and how fast one CU can pull
 // weights in is what bounds this kernel.  Here a workgroup (four waves) multiplies HALF a panel
 // (16 columns, blockIdx.x = 2 * panel group + half): twice as many, half as large units, all resident at once.
@@ -934,7 +934,7 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         if (pairs && (panels & 1)) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
         note_kernel(pairs ? "skinny_stream_bf16_gateup" : (w8 ? "skinny_stream_w8" : "skinny_stream_bf16"));
         const int per_wave = (s.nfrag + 7) / 8;
-        // Half-panel workgroups pay off for 1-2 rows of x (cheap to stage per workgroup) if each still has at least
+        // Half-panel workgroups pay off for up to 4 rows of x (cheap enough to stage per workgroup) if each still has at least
         // 128 KiB of weights to stream (measured: 64 KiB units lose more to the fixed cost of a workgroup than the
         // better balance gains) and the list is short enough for balance to matter: at most two rounds of resident
         // workgroups (four waves each; LDS allows min(4, 160 KiB / (reduction scratch + x)) per CU)
@@ -942,8 +942,8 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         const int lds_wg = 16 * 1024 * (pairs ? 2 : 1) + xbytes;
         const int wg_per_cu = (160 * 1024 / lds_wg) < 4 ? (160 * 1024 / lds_wg) : 4;
         const int64_t unit_bytes = (int64_t)s.nfrag * 512 * (pairs ? 2 : 1);
-        const int force = decode_halves();  // -1: by the rule above, 0: never, 1: for every M <= 2 (tests pin the path with it)
-        const bool halves = M <= 2 && force != 0 && (force == 1 || (2 * units <= 2 * 256 * wg_per_cu && unit_bytes >= 128 * 1024));
+        const int force = decode_halves();  // -1: by the rule above, 0: never, 1: for every M <= 4 (tests pin the path with it)
+        const bool halves = M <= 4 && force != 0 && (force == 1 || (2 * units <= 2 * 256 * wg_per_cu && unit_bytes >= 128 * 1024));
         const int per_wave_h = ((s.nfrag >> 1) + 3) / 4;
 #define MMX_STREAM(W8, NP, GRID)                                                                                     \
     do {                                                                                                             \

@@ -292,9 +292,10 @@ def test_decode_small_shapes(po, shape, w8):
     assert np.linalg.norm(got - ref) <= 1e-3 * np.linalg.norm(ref)
 
 
-# the half-panel form of the streaming decode kernel (M <= 2), forced on: both weight types, the
+# the half-panel form of the streaming decode kernel (M <= 4), forced on: both weight types, the
 # all-at-once and the rolling window (K), ragged N, a column range, every post-op operand
-@pytest.mark.parametrize("shape", [(1, 256, 64), (2, 512, 100), (1, 4096, 352), (2, 2048, 96), (1, 11008, 160)])
+@pytest.mark.parametrize("shape", [(1, 256, 64), (2, 512, 100), (1, 4096, 352), (2, 2048, 96), (1, 11008, 160), (4, 1024, 224),
+                                   (3, 4096, 64)])
 @pytest.mark.parametrize("w8", [False, True])
 def test_decode_half_panel_form(po, shape, w8):
     M, K, N = shape
@@ -388,11 +389,11 @@ def _mlp_case(po, M, K, N, seed):
     # stage 1: h from the same x
     e1, f1 = check_float_parity(bf16_to_f32(h), bf16_to_f32(h_ref), f"mlp h M={M}")
     # the fused SiLU(gate)*up store equals the oracle's, bit for bit, on the accumulators the GPU produced
-    # (gate and up alternate in 32-column panels of the packed matrix).  For M <= 2 the decode kernel has two
+    # (gate and up alternate in 32-column panels of the packed matrix).  For M <= 4 the decode kernel has two
     # forms that add the partial sums in different orders, chosen by the number of panels: pin the form so
     # that the plain GEMM and the fused one go the same way, and check both.
     forms = []
-    for halves in ((0, 1) if M <= 2 else (-1,)):
+    for halves in ((0, 1) if M <= 4 else (-1,)):
         mx.set_option("decode_halves", halves)
         try:
             hh = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
@@ -403,7 +404,7 @@ def _mlp_case(po, M, K, N, seed):
             k_plain = mx.last_kernel()
         finally:
             mx.set_option("decode_halves", -1)
-        if M <= 2:
+        if M <= 4:
             assert ("half" in k_fused) == (halves == 1) and ("half" in k_plain) == (halves == 1), (k_fused, k_plain)
         a = host_bits(acc).reshape(M, N // 32, 2, 32)
         gate, up = np.ascontiguousarray(a[:, :, 0, :]).reshape(M, N), np.ascontiguousarray(a[:, :, 1, :]).reshape(M, N)
@@ -451,7 +452,7 @@ def test_silu_gate_special_values(po, M):
     assert np.array_equal(got[~nan], want[~nan]), (mx.last_kernel(), g[np.flatnonzero((got != want).any(1))][:8])
 
 
-@pytest.mark.parametrize("M", [1, 5, 48, 300])
+@pytest.mark.parametrize("M", [1, 3, 5, 48, 300])
 def test_mlp_small(po, M):
     _mlp_case(po, M, 512, 768, seed=20 + M)
 
