@@ -861,8 +861,9 @@ int decode_halves();
 // int8 x int8 at M <= 32 can use the decode kernels if x is 16-byte aligned and K fills whole 128-byte groups of
 // the packed weights: the streaming form if x fits in LDS, else the chunked one, which walks K in chunks of 256
 bool skinny_i8_eligible(const void* x, int64_t ldx, int M, int K) {
+    if (M > 32 || K > (1 << 24)) return false;
     const int zoff = (M * K + 1023) & ~1023;
-    return M <= 32 && K % 128 == 0 && (zoff + K <= 46 * 1024 || K % 256 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
+    return K % 128 == 0 && (zoff + K <= 46 * 1024 || K % 256 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
            ((ldx & 15) == 0);
 }
 
@@ -870,6 +871,8 @@ bool skinny_i8_eligible(const void* x, int64_t ldx, int M, int K) {
 int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
                   const Epilogue& ep, hipStream_t st) {
     const bool w8 = wk == 1;
+    // the byte counts below are 32-bit: M <= 32 rows of at most 2^24 elements
+    if (M > 32 || K > (1 << 24)) return set_error(MMX_E_UNSUPPORTED, "decode kernels take M <= 32 and K <= 2^24 (got M = %d, K = %d)", M, K);
     SkinnyArgs s;
     s.x = static_cast<const char*>(x);
     s.ldx = ldx;
