@@ -292,6 +292,27 @@ def main():
         del gu, dn
         extra["llama7b_mlp_stages"] = stages
 
+        # q against a cache of keys (the mat-vec of test_qk.cpp): 2^21 tokens x head size 128, bf16, 537 MB
+        # (more than the 256 MB last-level cache holds)
+        T, D = 1 << 21, 128
+        keys = torch.randn((T, D), dtype=torch.float32, device="cuda").to(torch.bfloat16)
+        q = torch.randn((D,), dtype=torch.float32, device="cuda").to(torch.bfloat16)
+        sc = torch.empty(T, dtype=torch.float32, device="cuda")
+        mv = mx.MatmulVector()
+        for _ in range(20):
+            mv(keys, q, sc)
+        torch.cuda.synchronize()
+        a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a0.record()
+        for _ in range(20):
+            mv(keys, q, sc)
+        a1.record()
+        torch.cuda.synchronize()
+        ms = a0.elapsed_time(a1) / 20
+        extra["qk_matvec_bf16_T2097152_D128"] = {"us": round(ms * 1e3, 1), "GBps": round(T * D * 2 / ms / 1e6, 0),
+                                                 "frac_of_hbm_peak": round(T * D * 2 / ms / 1e6 / PEAK_HBM_GBS, 4)}
+        del keys, sc
+
         # what the matrix pipes deliver with nothing else going on: an issue-bound loop of independent MFMAs,
         # all-zero operands vs operands like the benchmark's (the clock under matrix load depends on the data)
         ceil = {}

@@ -362,7 +362,10 @@ def test_weight_compressed_matmul(po, M):
 
 
 # ---- mat-vec ---------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("shape", [(901, 80), (901, 96), (64, 4096), (37, 33)])
+# (256, 128) is the q x K-cache case of test_qk.cpp:483-484; (5000, 128) a longer cache; the others cover rows of
+# 4 / 16 / 64 lanes, tails after the last whole 16 bytes and rows shorter than 16 bytes.
+@pytest.mark.parametrize("shape", [(901, 80), (901, 96), (64, 4096), (37, 33), (256, 128), (5000, 128), (77, 24), (300, 200),
+                                   (19, 1000), (3, 7), (1, 4096)])
 def test_matvec(po, shape):
     M, K = shape
     rng = np.random.default_rng(16)
@@ -376,6 +379,29 @@ def test_matvec(po, shape):
     bi = rng.integers(-127, 128, K, dtype=np.int8)
     ci = mx.MatmulVector()(dev(Ai), dev(bi))
     assert np.array_equal(host_bits(ci), po.matvec_i8(Ai, bi))
+
+
+def test_matvec_row_views_and_alignment(po):
+    """Rows taken out of a wider cache (a head of a [tokens, heads x head_size] tensor) and operands that are
+    not 16-byte aligned go through the same call and give the same numbers."""
+    rng = np.random.default_rng(17)
+    T, H, D = 333, 4, 128
+    cache = rand_bf16(rng, (T, H * D), 1.0)
+    q = rand_bf16(rng, (D,), 1.0)
+    dcache = dev_bf16(cache)
+    for h in (0, 3):
+        c = mx.MatmulVector()(dcache[:, h * D:(h + 1) * D], dev_bf16(q))
+        ref = po.matvec_bf16(np.ascontiguousarray(cache[:, h * D:(h + 1) * D]), q)
+        assert np.linalg.norm(host_bits(c) - ref) <= 1e-5 * np.linalg.norm(ref)
+    # a view that starts 2 bytes into a row: the element-wise form
+    c = mx.MatmulVector()(dcache[:, 1:1 + D], dev_bf16(q))
+    ref = po.matvec_bf16(np.ascontiguousarray(cache[:, 1:1 + D]), q)
+    assert np.linalg.norm(host_bits(c) - ref) <= 1e-5 * np.linalg.norm(ref)
+    Ai = rng.integers(-127, 128, (T, H * D), dtype=np.int8)
+    bi = rng.integers(-127, 128, D, dtype=np.int8)
+    for off in (0, 128, 3):
+        ci = mx.MatmulVector()(dev(Ai)[:, off:off + D], dev(bi))
+        assert np.array_equal(host_bits(ci), po.matvec_i8(np.ascontiguousarray(Ai[:, off:off + D]), bi))
 
 
 # ---- fused MLP ---------------------------------------------------------------------------------------------
