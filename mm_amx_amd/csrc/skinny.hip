@@ -13,6 +13,11 @@
 
 namespace mmx {
 
+// Packed weights are read exactly once per launch: nontemporal loads keep them from displacing x, the
+// per-column operands and each other in the caches (int8 GEMV 4096x11008: 11.2 -> 10.5 us; MLP gate/up at
+// M=1: 36.3 -> 33.4 us).
+#define MMX_WLOAD(ptr) __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(ptr))
+
 struct SkinnyArgs {
     const char* x;
     int64_t ldx;  // bytes
@@ -217,8 +222,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(const SkinnyArgs s) {
                 const int panel = panel_first + p;
                 w[p][u] = u32x4{0u, 0u, 0u, 0u};
                 if (f < f_end && panel < panel_end && panel < s.npanels)
-                    w[p][u] = *reinterpret_cast<const u32x4*>(s.Wp + (int64_t)panel * s.panel_stride +
-                                                              (int64_t)f * 1024 + lane * 16);
+                    w[p][u] = MMX_WLOAD(s.Wp + (int64_t)panel * s.panel_stride + (int64_t)f * 1024 + lane * 16);
             }
             if constexpr (W4) {
                 const int k0 = 64 * f + 32 * g32;
@@ -311,7 +315,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         int f_ = f_begin + (BT) * U + (UU);                                                 \
         f_ = f_ < f_last ? f_ : f_last;                                                     \
         _Pragma("unroll") for (int p = 0; p < NP; p++)                                      \
-            w[p][UU] = *reinterpret_cast<const u32x4*>(wbase[p] + (int64_t)f_ * 1024);      \
+            w[p][UU] = MMX_WLOAD(wbase[p] + (int64_t)f_ * 1024);                         \
         xa[UU] = *reinterpret_cast<const bf16x8*>(xlane + (int64_t)f_ * XB);                \
         if constexpr (W8) xb[UU] = *reinterpret_cast<const bf16x8*>(xlane + (int64_t)f_ * XB + 16); \
     } while (0)
@@ -437,7 +441,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             int f_ = (C) * FC + wave * FPW + u;                                                                \
             f_ = f_ < f_last ? f_ : f_last;                                                                    \
             _Pragma("unroll") for (int p = 0; p < NP; p++)                                                     \
-                w[J][u][p] = *reinterpret_cast<const u32x4*>(wbase[p] + (int64_t)f_ * 1024);                   \
+                w[J][u][p] = MMX_WLOAD(wbase[p] + (int64_t)f_ * 1024);                                      \
         }                                                                                                      \
     } while (0)
 #define MMX_CHUNK(C, J)                                                                                        \
@@ -598,7 +602,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         int f_ = f_begin + (BT) * U + (UU);                                                                     \
         f_ = f_ < f_last ? f_ : f_last;                                                                         \
         _Pragma("unroll") for (int p = 0; p < NP; p++)                                                          \
-            w[p][UU] = *reinterpret_cast<const u32x4*>(wbase[p] + (int64_t)f_ * 1024);                          \
+            w[p][UU] = MMX_WLOAD(wbase[p] + (int64_t)f_ * 1024);                                             \
     } while (0)
 #define MMX_MULTIPLY(BT, UU)                                                                                    \
     do {                                                                                                        \
@@ -757,7 +761,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         int u_ = u_begin + (BT) * U + (UU);                                                                     \
         u_ = u_ < u_last ? u_ : u_last;                                                                         \
         _Pragma("unroll") for (int p = 0; p < NP; p++)                                                          \
-            w[p][UU] = *reinterpret_cast<const u32x4*>(wbase[p] + (int64_t)u_ * 2048);                          \
+            w[p][UU] = MMX_WLOAD(wbase[p] + (int64_t)u_ * 2048);                                             \
     } while (0)
 #define MMX_MULTIPLY(BT, UU)                                                                                    \
     do {                                                                                                        \
