@@ -313,6 +313,35 @@ def main():
                                                  "frac_of_hbm_peak": round(T * D * 2 / ms / 1e6 / PEAK_HBM_GBS, 4)}
         del keys, sc
 
+        # What a kernel that only streams the same number of bytes takes, launch after launch: the mat-vec kernel
+        # over key caches of the size of the decode weights (45 / 90 / 180 MB, rotated over 541 MB), replayed
+        # from a HIP graph so that no host time is in the figure.  The decode kernels are judged against this.
+        floor = {}
+        for label, Tf in (("45MB", 176128), ("90MB", 352256), ("180MB", 704512)):
+            ks = [torch.randn((Tf, D), dtype=torch.float32, device="cuda").to(torch.bfloat16) for _ in range(12 * 176128 // Tf)]
+            scf = torch.empty(Tf, dtype=torch.float32, device="cuda")
+            nl = len(ks) * 10
+            for i in range(nl):
+                mv(ks[i % len(ks)], q, scf)
+            torch.cuda.synchronize()
+            gr, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+            with torch.cuda.stream(side):
+                with torch.cuda.graph(gr, stream=side):
+                    for i in range(nl):
+                        mv(ks[i % len(ks)], q, scf)
+            torch.cuda.synchronize()
+            gr.replay()
+            torch.cuda.synchronize()
+            a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a0.record()
+            gr.replay()
+            a1.record()
+            torch.cuda.synchronize()
+            us = a0.elapsed_time(a1) / nl * 1e3
+            floor[label] = {"us": round(us, 2), "GBps": round(Tf * D * 2 / us / 1e3, 0)}
+            del gr, ks, scf
+        extra["streaming_read_floor"] = floor
+
         # what the matrix pipes deliver with nothing else going on: an issue-bound loop of independent MFMAs,
         # all-zero operands vs operands like the benchmark's (the clock under matrix load depends on the data)
         ceil = {}
