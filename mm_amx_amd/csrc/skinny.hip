@@ -16,6 +16,15 @@ namespace mmx {
 // Packed weights are read exactly once per launch: nontemporal loads keep them from displacing x, the
 // per-column operands and each other in the caches (int8 GEMV 4096x11008: 11.2 -> 10.5 us; MLP gate/up at
 // M=1: 36.3 -> 33.4 us).
+// compile-time loop: f(integral_constant<int, B>) ... f(integral_constant<int, E-1>)
+template <int B, int E, typename F>
+__device__ __forceinline__ void skinny_static_for(F&& f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        skinny_static_for<B + 1, E>(f);
+    }
+}
+
 #define MMX_WLOAD(ptr) __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(ptr))
 
 struct SkinnyArgs {
@@ -363,7 +372,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 // to LDS and read from there as MFMA operands: fetched per lane straight from global memory, the 32
 // rows of an operand make every load touch 32 cache lines, and the CU's vector cache becomes the
 // bottleneck (19 us instead of 12 for the 4096 x 11008 int8 GEMV at M = 16).
-// Weights and x of chunk c+W are requested while chunk c is multiplied (W = 3 chunks in flight; all
+// Weights and x of chunk c+W are requested while chunk c is multiplied (W = 3 chunks in flight, more
+// measured no faster; all
 // loads are ordinary loads, so the compiler's own counting of outstanding loads places the waits).
 // Two LDS buffers: chunk c+1 is written while slower waves still read chunk c; the barrier of chunk
 // c+1 is what allows chunk c+2 to overwrite chunk c.  16-byte pieces of a row are XOR-swizzled with
@@ -489,28 +499,21 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         }                                                                                                      \
     } while (0)
 
-    if (0 < nchunk) MMX_LOAD(0, 0);
-    if (1 < nchunk) MMX_LOAD(1, 1);
-    if constexpr (W == 3) {
-        if (2 < nchunk) MMX_LOAD(2, 2);
-    }
+    skinny_static_for<0, W>([&](auto j_c) {
+        constexpr int J = decltype(j_c)::value;
+        if (J < nchunk) MMX_LOAD(J, J);
+    });
     for (int c0 = 0; c0 < nchunk; c0 += W) {
-        MMX_CHUNK(c0, 0);
-        if (c0 + W < nchunk) MMX_LOAD(c0 + W, 0);
-        if (c0 + 1 < nchunk) {
-            MMX_CHUNK(c0 + 1, 1);
-            if (c0 + 1 + W < nchunk) MMX_LOAD(c0 + 1 + W, 1);
-        }
-        if constexpr (W == 3) {
-            if (c0 + 2 < nchunk) {
-                MMX_CHUNK(c0 + 2, 2);
-                if (c0 + 2 + W < nchunk) MMX_LOAD(c0 + 2 + W, 2);
+        skinny_static_for<0, W>([&](auto j_c) {
+            constexpr int J = decltype(j_c)::value;
+            if (c0 + J < nchunk) {
+                MMX_CHUNK(c0 + J, J);
+                if (c0 + J + W < nchunk) MMX_LOAD(c0 + J + W, J);
             }
-        }
+        });
     }
 #undef MMX_LOAD
 #undef MMX_CHUNK
-    static_assert(W == 2 || W == 3, "the loop above is unrolled by hand");
 
     __syncthreads();  // all reads of x are done: the buffers become the reduction scratch
 #pragma unroll
