@@ -747,6 +747,16 @@ def test_int4_is_a_decode_path_only():
         mx.quantize_pack_int4(torch.zeros((256, 64), dtype=torch.float32, device="cuda"))
 
 
+def test_decode_rejects_k_beyond_its_32_bit_byte_counts():
+    # buffers of the real size, so that nothing could be read out of bounds even if the call went through
+    K, N = (1 << 24) + 256, 32
+    x = torch.empty((1, K), dtype=torch.bfloat16, device="cuda")
+    packed = torch.empty(mx.packed_b_bytes(mx.BF16, K, N), dtype=torch.uint8, device="cuda")
+    y = torch.zeros((1, N), dtype=torch.float32, device="cuda")
+    with pytest.raises(mx.MmxError, match="K <= 2\\^24"):
+        mx.gemm(x, packed, N, mx.Epilogue(y, mx.PP_NONE))
+
+
 @pytest.mark.parametrize("M", [1, 64])
 def test_mlp_replays_from_a_hip_graph(M):
     # the entry points allocate nothing and never synchronise, so a caller may capture them: the fused MLP (two
