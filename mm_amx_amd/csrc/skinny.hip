@@ -939,6 +939,29 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
     const int kpad = kbytes_pad / (w8 ? 1 : 2);  // elements of K the packed weights cover
     const int zero_off = (M * K * 2 + 1023) & ~1023;
     const int xbytes = zero_off + K * 2;  // x, a gap up to the next KiB, one row of zeros
+    if (kpad == K && s.x_vec_ok && !w8 && !pairs && M >= 2 && M <= 4 && xbytes > 46 * 1024 && xbytes <= 128 * 1024 &&
+        decode_halves() != 0 && panels <= 256 && (int64_t)s.nfrag * 512 >= 128 * 1024) {
+        // A few rows of a long x (the MLP's down projection at M = 2-4: 66-110 KiB with the zero row) and at
+        // most one half-panel per CU: the half-panel form with one workgroup per CU still has all of x in LDS.
+        typedef void (*HalfKernel)(const SkinnyArgs, int);
+        static bool attr_done = false;
+        if (!attr_done) {
+            const HalfKernel kernels[2] = {skinny_half_kernel<false, 1, true, 16>, skinny_half_kernel<false, 1, false, 16>};
+            for (HalfKernel k : kernels) {
+                const int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                             128 * 1024),
+                                         "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+                if (rc) return rc;
+            }
+            attr_done = true;
+        }
+        note_kernel("skinny_half_bf16");
+        if (((s.nfrag >> 1) + 3) / 4 <= 16)
+            hipLaunchKernelGGL((skinny_half_kernel<false, 1, true, 16>), dim3(2 * panels), dim3(256), xbytes, st, s, zero_off);
+        else
+            hipLaunchKernelGGL((skinny_half_kernel<false, 1, false, 16>), dim3(2 * panels), dim3(256), xbytes, st, s, zero_off);
+        return check_hip(hipGetLastError(), "skinny_half_kernel launch");
+    }
     if (kpad == K && xbytes <= 46 * 1024 && s.x_vec_ok && !(pairs && w8)) {  // LDS: 2 x (this + 32 KiB) per CU
         // the activations fit in LDS: streaming variant
         if (pairs && (panels & 1)) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");

@@ -342,6 +342,37 @@ def test_decode_half_panel_form(po, shape, w8):
     assert np.linalg.norm(a - b) <= 1e-5 * np.linalg.norm(b)
 
 
+# 2-4 rows of a long x (the MLP's down projection: K = 11008) still go whole into LDS for the half-panel form when
+# there is at most one half-panel per CU; "decode_halves" = 0 gives the per-lane form to compare with
+@pytest.mark.parametrize("shape", [(2, 11008, 256), (3, 11008, 100), (4, 11008, 4096), (4, 8192, 160)])
+def test_decode_half_panel_form_long_x(po, shape):
+    M, K, N = shape
+    rng = np.random.default_rng(9 * sum(shape))
+    x, W = rand_bf16(rng, (M, K), 1.0), rand_bf16(rng, (K, N), 0.05)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    packed = mx.repack_b(dev_bf16(W))
+    n0, n1 = (32, N - 5) if N > 96 and N < 4096 else (0, N)
+    out = {}
+    try:
+        for halves in (-1, 0):
+            mx.set_option("decode_halves", halves)
+            y = torch.full((M, N), 7.0, dtype=torch.float32, device="cuda")
+            mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_BIAS | mx.PP_GELU, bias=dev(bias)), n0=n0, n1=n1)
+            k1 = mx.last_kernel()
+            acc = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+            mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc, mx.PP_NONE))
+            assert ("skinny_half" in k1) == (halves == -1) and ("skinny_half" in mx.last_kernel()) == (halves == -1), k1
+            out[halves] = (host_bits(y), host_bits(acc))
+    finally:
+        mx.set_option("decode_halves", -1)
+    acc_ref = po.gemm_bf16(x, W)
+    for halves, (got, acc) in out.items():
+        check_float_parity(acc, acc_ref, f"long-x accumulators {shape} halves={halves}")
+        again = po.pp(acc, po.PP_BIAS | po.PP_GELU, po.F32, bias=bias)
+        assert np.array_equal(got[:, n0:n1].view(np.uint32), again[:, n0:n1].view(np.uint32))
+        assert np.all(got[:, :n0] == 7.0) and np.all(got[:, n1:] == 7.0)
+
+
 @pytest.mark.parametrize("M", [4, 40])
 def test_weight_compressed_matmul(po, M):
     """Matmul<bf16,int8,float>: bf16 weights compressed per tensor inside the op (include/kernels_amx.hpp:1363-1379)."""
