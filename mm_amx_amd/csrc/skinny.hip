@@ -546,8 +546,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     // fragments per panel per wave in flight at once (16 KiB of weights; int4: 8 KiB, a fragment holds 64 of k
     // and unpacking it costs more than streaming it)
     constexpr int U = (W4 ? 8 : 16) / NP;
-    __shared__ float red[8][NP][16][64];
-    extern __shared__ __attribute__((aligned(1024))) char xs[];  // [M][K] bf16, then at zero_off a row of zeros
+    // [M][K] bf16, then at zero_off a row of zeros; once x has been used up, the cross-wave reduction scratch
+    // (the launcher allocates the larger of the two: stream_lds_bytes)
+    extern __shared__ __attribute__((aligned(1024))) char xs[];
+    typedef float Red[8][NP][16][64];
+    Red& red = *reinterpret_cast<Red*>(xs);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: keeps the control flow below uniform
@@ -667,6 +670,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #undef MMX_REQUEST
 #undef MMX_MULTIPLY
 
+    __syncthreads();  // every wave has read its last x: the buffer becomes the reduction scratch
 #pragma unroll
     for (int p = 0; p < NP; p++)
 #pragma unroll
@@ -867,6 +871,9 @@ int decode_halves();
 
 // int8 x int8 at M <= 32 can use the decode kernels if x is 16-byte aligned and K fills whole 128-byte groups of
 // the packed weights: the streaming form if x fits in LDS, else the chunked one, which walks K in chunks of 256
+// dynamic LDS of skinny_stream_kernel: x + the zero row, reused afterwards as the reduction scratch (32 KiB per panel)
+static inline int stream_lds_bytes(int xbytes, int np) { return xbytes > 32768 * np ? xbytes : 32768 * np; }
+
 bool skinny_i8_eligible(const void* x, int64_t ldx, int M, int K) {
     if (M > 32 || K > (1 << 24)) return false;
     const int zoff = (M * K + 1023) & ~1023;
@@ -907,9 +914,9 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         }
         note_kernel("skinny_stream_i8");
         if ((s.nfrag + 7) / 8 <= 16)
-            hipLaunchKernelGGL((skinny_stream_kernel<3, 1, true>), dim3(panels), dim3(512), zoff + K, st, s, zoff);
+            hipLaunchKernelGGL((skinny_stream_kernel<3, 1, true>), dim3(panels), dim3(512), stream_lds_bytes(zoff + K, 1), st, s, zoff);
         else
-            hipLaunchKernelGGL((skinny_stream_kernel<3, 1, false>), dim3(panels), dim3(512), zoff + K, st, s, zoff);
+            hipLaunchKernelGGL((skinny_stream_kernel<3, 1, false>), dim3(panels), dim3(512), stream_lds_bytes(zoff + K, 1), st, s, zoff);
         return check_hip(hipGetLastError(), "skinny_stream_kernel launch");
     }
     if (wk == 2) {
@@ -920,9 +927,9 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         if (s.nfrag * 64 == K && xb <= 46 * 1024 && s.x_vec_ok) {
             note_kernel("skinny_stream_w4");
             if ((s.nfrag + 7) / 8 <= 8)
-                hipLaunchKernelGGL((skinny_stream_kernel<2, 1, true>), dim3(panels), dim3(512), xb, st, s, zoff);
+                hipLaunchKernelGGL((skinny_stream_kernel<2, 1, true>), dim3(panels), dim3(512), stream_lds_bytes(xb, 1), st, s, zoff);
             else
-                hipLaunchKernelGGL((skinny_stream_kernel<2, 1, false>), dim3(panels), dim3(512), xb, st, s, zoff);
+                hipLaunchKernelGGL((skinny_stream_kernel<2, 1, false>), dim3(panels), dim3(512), stream_lds_bytes(xb, 1), st, s, zoff);
             return check_hip(hipGetLastError(), "skinny_stream_kernel launch");
         }
         if (s.nfrag * 64 == K && s.x_vec_ok) {
@@ -962,7 +969,26 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
             hipLaunchKernelGGL((skinny_half_kernel<false, 1, false, 16>), dim3(2 * panels), dim3(256), xbytes, st, s, zero_off);
         return check_hip(hipGetLastError(), "skinny_half_kernel launch");
     }
-    if (kpad == K && xbytes <= 46 * 1024 && s.x_vec_ok && !(pairs && w8)) {  // LDS: 2 x (this + 32 KiB) per CU
+    // The streaming form needs all of x in LDS and at least two workgroups per CU (344 panels of N = 11008 must all
+    // be resident): 80 KiB of x each (4096 x 11008 int8 GEMV at M = 5-8: 13.0-13.4 -> 11.5-12.0 us against the chunked
+    // form; with one workgroup per CU, M = 12-16, it loses: 16.6-17.7 against 13.7-14.5 us).
+    const bool bigx = !pairs && xbytes > 46 * 1024 && xbytes <= 80 * 1024;
+    if (bigx) {
+        typedef void (*StreamKernel)(const SkinnyArgs, int);
+        static bool attr_done = false;
+        if (!attr_done) {
+            const StreamKernel kernels[4] = {skinny_stream_kernel<0, 1, true>, skinny_stream_kernel<0, 1, false>,
+                                             skinny_stream_kernel<1, 1, true>, skinny_stream_kernel<1, 1, false>};
+            for (StreamKernel k : kernels) {
+                const int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                             80 * 1024),
+                                         "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+                if (rc) return rc;
+            }
+            attr_done = true;
+        }
+    }
+    if (kpad == K && (xbytes <= 46 * 1024 || bigx) && s.x_vec_ok && !(pairs && w8)) {
         // the activations fit in LDS: streaming variant
         if (pairs && (panels & 1)) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
         note_kernel(pairs ? "skinny_stream_bf16_gateup" : (w8 ? "skinny_stream_w8" : "skinny_stream_bf16"));
@@ -976,7 +1002,7 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         const int wg_per_cu = (160 * 1024 / lds_wg) < 4 ? (160 * 1024 / lds_wg) : 4;
         const int64_t unit_bytes = (int64_t)s.nfrag * 512 * (pairs ? 2 : 1);
         const int force = decode_halves();  // -1: by the rule above, 0: never, 1: for every M <= 4 (tests pin the path with it)
-        const bool halves = M <= 4 && force != 0 && (force == 1 || (2 * units <= 2 * 256 * wg_per_cu && unit_bytes >= 128 * 1024));
+        const bool halves = M <= 4 && !bigx && force != 0 && (force == 1 || (2 * units <= 2 * 256 * wg_per_cu && unit_bytes >= 128 * 1024));
         const int per_wave_h = ((s.nfrag >> 1) + 3) / 4;
 #define MMX_STREAM(W8, NP, GRID)                                                                                     \
     do {                                                                                                             \
@@ -985,9 +1011,9 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         else if (halves) /* the rolling window holds fewer registers where two accumulator pairs need them */      \
             hipLaunchKernelGGL((skinny_half_kernel<W8, NP, false, (NP == 2 ? 4 : (W8 ? 12 : 16))>), dim3(2 * (GRID)), dim3(256), xbytes, st, s, zero_off); \
         else if (per_wave <= 16 / NP)                                                                                \
-            hipLaunchKernelGGL((skinny_stream_kernel<W8, NP, true>), dim3(GRID), dim3(512), xbytes, st, s, zero_off); \
+            hipLaunchKernelGGL((skinny_stream_kernel<W8, NP, true>), dim3(GRID), dim3(512), stream_lds_bytes(xbytes, NP), st, s, zero_off); \
         else                                                                                                         \
-            hipLaunchKernelGGL((skinny_stream_kernel<W8, NP, false>), dim3(GRID), dim3(512), xbytes, st, s, zero_off); \
+            hipLaunchKernelGGL((skinny_stream_kernel<W8, NP, false>), dim3(GRID), dim3(512), stream_lds_bytes(xbytes, NP), st, s, zero_off); \
     } while (0)
         if (halves) note_kernel(pairs ? "skinny_half_bf16_gateup" : (w8 ? "skinny_half_w8" : "skinny_half_bf16"));
         if (pairs) MMX_STREAM(false, 2, panels / 2);

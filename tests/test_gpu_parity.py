@@ -256,7 +256,9 @@ def test_decode_gemv_w8_full_size(po, M):
     print(f"gemv_w8 M={M}: rel_fro={err:.2e} within_1ulp={frac * 100:.4f}%")
 
 
-@pytest.mark.parametrize("shape", [(1, 256, 64), (3, 320, 100), (16, 337, 96), (32, 2560, 192), (7, 70, 45)])
+# the last three: 46-80 KiB of x, which the streaming form still holds in LDS (the reduction scratch reuses the space)
+@pytest.mark.parametrize("shape", [(1, 256, 64), (3, 320, 100), (16, 337, 96), (32, 2560, 192), (7, 70, 45),
+                                   (8, 4096, 96), (9, 4096, 160), (5, 6144, 64)])
 @pytest.mark.parametrize("w8", [False, True])
 def test_decode_small_shapes(po, shape, w8):
     M, K, N = shape
@@ -281,6 +283,8 @@ def test_decode_small_shapes(po, shape, w8):
         y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
         mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_BIAS | mx.PP_GELU, bias=dev(bias)))
     assert "skinny" in mx.last_kernel()
+    if K >= 4096:
+        assert "skinny_stream" in mx.last_kernel(), mx.last_kernel()
     # raw accumulators through the same kernel, then the oracle's post-op on them must give y's bits
     acc_gpu = torch.zeros((M, N), dtype=torch.float32, device="cuda")
     mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc_gpu, mx.PP_NONE), b_dtype=mx.I8 if w8 else None)
