@@ -154,7 +154,8 @@ const char* mmx_last_kernel(void);
  * fallback for operands beyond 32-bit offsets).  Shapes whose K tail or alignment need masked
  * loads use a masked kernel whatever this is set to.  "decode_halves": whether the streaming decode
  * kernel for M <= 4 splits every 32-column panel over two workgroups — -1 (default) where that fills the
- * CUs better, 0 never, 1 always (the two forms add the partial sums in different orders). */
+ * CUs better, 0 never, 1 always while x takes at most 46 KiB of LDS (the two forms add the partial sums in
+ * different orders). */
 int mmx_set_option(const char* name, int value);  /* process-wide, like mmx_set_tile: set them before the threads start */
 /* HIP-event timing of `iters` back-to-back launches of the given gemm on `stream`, launch i
  * using the packed weights Bpacked_rot[i % n_rot] (rotate over several copies so that a
