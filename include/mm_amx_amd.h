@@ -76,7 +76,8 @@ typedef struct mmx_epilogue {
 /* message for the last failing call made by this thread ("" if none) */
 const char* mmx_last_error(void);
 
-/* Selects `device`, checks that it is a gfx950, raises kernel LDS limits.  Idempotent.
+/* Selects `device` and checks that it is a gfx950.  Idempotent, callable from any thread.  (Kernels that need
+ * more than 64 KiB of LDS have their limit raised at their first launch on a device, under a lock.)
  * Stands in for initXTILE() (include/misc.hpp:376-396), the reference's one-time set-up. */
 int mmx_init(int device);
 
@@ -132,6 +133,29 @@ int mmx_dequant_packed(const void* packed_i8, int K, int N, void* packed_bf16, v
 int mmx_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* Bpacked, int M, int K,
              int N, int n0, int n1, const mmx_epilogue* ep, void* stream);
 
+/* ---- the same product with K split over several workgroups per output tile ---------------------------------
+ * AMX_MLP::Linear (tests/amx-mlp.cpp:560-593) gives each half of the K blocks of `down` to its own core and lets
+ * the one that finishes last add the two fp32 partial results and round to bf16 (:648-682).  Here a tile's K range
+ * is cut into k_splits slices of whole 512-byte blocks of K per row (256 bf16, the reference's K block; slice s
+ * takes blocks [s*q, (s+1)*q), q = ceil(blocks / k_splits), so k_splits = 2 is the reference's partition), one
+ * workgroup each; each parks its fp32 / int32 partial tile in `workspace`, and the workgroup that arrives last
+ * adds them in slice order (so the result does not depend on the arrival order) and applies the post-op.  It
+ * pays where a shape has fewer tiles than the GPU has CUs, or tiles bound by the bytes a CU can pull in.
+ *   k_splits  0 = the library chooses (possibly no split), 1 = none, 2..4 = exactly that many slices
+ *             (MMX_E_INVALID if K is too short or the workspace too small, MMX_E_UNSUPPORTED for M <= 32,
+ *             SILU_GATE, unaligned A or K * sizeof(T) not a multiple of 128).
+ *   workspace device memory, 256-byte aligned, mmx_gemm_workspace_bytes() or more (64 MiB + 16 KiB always
+ *             suffices for k_splits = 0; with less, the choice is restricted to what fits).  Its first 16 KiB are
+ *             arrival counters: zero them once after allocation; every call leaves them zero.  Calls that share
+ *             a workspace must not overlap in time (different streams need different workspaces).
+ * With workspace = NULL this is mmx_gemm. */
+int mmx_gemm_splitk(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* Bpacked, int M, int K,
+                    int N, int n0, int n1, const mmx_epilogue* ep, int k_splits, void* workspace,
+                    size_t workspace_bytes, void* stream);
+/* Workspace the call above would use for this shape (0 if it would not split).  steps = the post-op steps. */
+size_t mmx_gemm_workspace_bytes(int a_dtype, int b_dtype, int M, int K, int N, int n0, int n1, uint32_t steps,
+                                int k_splits);
+
 /* ---- c[M] = A[M, K] · b[K]: amx_kernel::MatmulVector::operator() (include/kernels_amx.hpp:959)
  * and amx_kernel::GemAvB::operator() (:1534).  dtype MMX_BF16 (c fp32) or MMX_I8 (c int32). */
 int mmx_matvec(int dtype, const void* A, int64_t lda_bytes, const void* b, void* c, int M, int K, void* stream);
@@ -144,8 +168,16 @@ int mmx_matvec(int dtype, const void* A, int64_t lda_bytes, const void* b, void*
 int mmx_mlp(const void* x, int64_t ldx_bytes, const void* w_gate_up, const void* w_down, void* h, int64_t ldh_bytes,
             void* y, int64_t ldy_bytes, int M, int K, int N, void* stream);
 
+/* The same with the down projection's K split over `down_k_splits` slices (0 = the library chooses, 2 = the
+ * reference's do_splitK, tests/amx-mlp.cpp:768 and :560-593); workspace as for mmx_gemm_splitk.  M <= 32 (decode
+ * kernels) and workspace = NULL run without slices. */
+int mmx_mlp_splitk(const void* x, int64_t ldx_bytes, const void* w_gate_up, const void* w_down, void* h,
+                   int64_t ldh_bytes, void* y, int64_t ldy_bytes, int M, int K, int N, int down_k_splits,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- introspection / tuning (no reference counterpart) --------------------------------------- */
-/* Force the MFMA tile shape ("256x256", "256x192", "128x256", "128x192", "128x128", "128x64", "" = automatic). */
+/* Force the MFMA tile shape ("256x256", "256x192", "128x256", "128x192", "128x128", "128x64", "" = automatic)
+ * for the calling thread's later calls. */
 int mmx_set_tile(const char* shape);
 /* Name of the kernel variant the last mmx_gemm call of this thread launched. */
 const char* mmx_last_kernel(void);
@@ -156,13 +188,14 @@ const char* mmx_last_kernel(void);
  * kernel for M <= 4 splits every 32-column panel over two workgroups — -1 (default) where that fills the
  * CUs better, 0 never, 1 always while x takes at most 46 KiB of LDS (the two forms add the partial sums in
  * different orders). */
-int mmx_set_option(const char* name, int value);  /* process-wide, like mmx_set_tile: set them before the threads start */
+int mmx_set_option(const char* name, int value);  /* like mmx_set_tile: affects the calling thread's later calls only */
 /* HIP-event timing of `iters` back-to-back launches of the given gemm on `stream`, launch i
  * using the packed weights Bpacked_rot[i % n_rot] (rotate over several copies so that a
  * bandwidth-bound shape is not served from cache); returns the average milliseconds per launch
- * in *ms_out.  Other arguments as for mmx_gemm.  Blocks until the last launch has finished. */
+ * in *ms_out.  Other arguments as for mmx_gemm_splitk.  Blocks until the last launch has finished. */
 int mmx_time_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* const* Bpacked_rot, int n_rot,
-                  int M, int K, int N, int n0, int n1, const mmx_epilogue* ep, void* stream, int iters, float* ms_out);
+                  int M, int K, int N, int n0, int n1, const mmx_epilogue* ep, int k_splits, void* workspace,
+                  size_t workspace_bytes, void* stream, int iters, float* ms_out);
 
 /* What an issue-bound loop of independent 32x32 MFMAs (dtype MMX_BF16 or MMX_I8) reaches on this device
  * right now, with all-zero operands (random_operands = 0) or with random ones (bf16: N(0,1) x N(0,0.02);

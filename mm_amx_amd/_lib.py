@@ -16,8 +16,12 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.environ.get("MMX_LIB_PATH") or os.path.join(_HERE, "libmm_amx_amd.so")
 
 EXPORTS = ["mmx_last_error", "mmx_init", "mmx_packed_b_bytes", "mmx_repack_b", "mmx_repack_gate_up",
-           "mmx_quantize_weights", "mmx_quantize_pack_int4", "mmx_dequant_packed", "mmx_gemm", "mmx_matvec", "mmx_mlp", "mmx_set_tile",
+           "mmx_quantize_weights", "mmx_quantize_pack_int4", "mmx_dequant_packed", "mmx_gemm", "mmx_gemm_splitk",
+           "mmx_gemm_workspace_bytes", "mmx_matvec", "mmx_mlp", "mmx_mlp_splitk", "mmx_set_tile",
            "mmx_set_option", "mmx_last_kernel", "mmx_time_gemm", "mmx_probe_mfma"]
+
+# a workspace of this size serves every shape when the library chooses the K split itself (include/mm_amx_amd.h)
+WORKSPACE_BYTES = (64 << 20) + (16 << 10)
 
 
 class MmxError(RuntimeError):
@@ -60,14 +64,20 @@ def lib():
         l.mmx_dequant_packed.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
         l.mmx_gemm.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
                                C.c_int, C.POINTER(_Epilogue), C.c_void_p]
+        l.mmx_gemm_splitk.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
+                                      C.c_int, C.POINTER(_Epilogue), C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]
+        l.mmx_gemm_workspace_bytes.restype = C.c_size_t
+        l.mmx_gemm_workspace_bytes.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_uint32, C.c_int]
+        l.mmx_mlp_splitk.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p,
+                                     C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]
         l.mmx_matvec.argtypes = [C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
         l.mmx_mlp.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p,
                               C.c_int64, C.c_int, C.c_int, C.c_int, C.c_void_p]
         l.mmx_set_tile.argtypes = [C.c_char_p]
         l.mmx_set_option.argtypes = [C.c_char_p, C.c_int]
         l.mmx_time_gemm.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int64, C.POINTER(C.c_void_p), C.c_int, C.c_int,
-                                    C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(_Epilogue), C.c_void_p, C.c_int,
-                                    C.POINTER(C.c_float)]
+                                    C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(_Epilogue), C.c_int, C.c_void_p, C.c_size_t,
+                                    C.c_void_p, C.c_int, C.POINTER(C.c_float)]
         l.mmx_probe_mfma.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.POINTER(C.c_float),
                                      C.POINTER(C.c_float)]
         _lib = l
@@ -196,30 +206,113 @@ def dequant_packed(packed_i8, K, N):
     return out
 
 
-def gemm(A, Bpacked, N, ep, b_dtype=None, n0=0, n1=None):
-    """C[:, n0:n1] = PP(A · B[:, n0:n1]); A [M,K] bf16/int8, Bpacked from repack_b of the full [K,N]."""
+_workspaces = {}
+
+
+def workspace(device=None, nbytes=WORKSPACE_BYTES):
+    """The K-split workspace of the current stream on `device` (zeroed once, when it is created).  Calls
+    on one stream are ordered, so one workspace per stream is enough; returns None while the stream is
+    being captured into a graph and has no workspace yet (an allocation there would be captured too)."""
+    dev_index = torch.cuda.current_device() if device is None else (device.index or 0)
+    key = (dev_index, torch.cuda.current_stream(dev_index).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        if torch.cuda.is_current_stream_capturing():
+            return None
+        ws = torch.zeros(nbytes, dtype=torch.uint8, device=f"cuda:{dev_index}")
+        torch.cuda.current_stream(dev_index).synchronize()
+        _workspaces[key] = ws
+    return ws
+
+
+def _is_2d(t, what):
+    if not isinstance(t, torch.Tensor) or t.dim() != 2:
+        raise MmxError(f"{what} must be a 2-D tensor")
+
+
+def _check_gemm_args(A, Bpacked, N, ep, b_dt, n0, n1):
+    """Host-side checks of everything the kernels take on trust: a wrong size here would be an out-of-bounds
+    access on the GPU."""
+    _is_2d(A, "A")
+    M, K = A.shape
+    a_dt = dtype_code(A)
+    if a_dt not in (BF16, I8):
+        raise MmxError("A must be bf16 or int8")
+    if not isinstance(N, int) or N <= 0 or not (0 <= n0 < n1 <= N):
+        raise MmxError(f"column range [{n0}, {n1}) outside [0, {N})")
+    if not isinstance(Bpacked, torch.Tensor) or Bpacked.dtype != torch.uint8 or not Bpacked.is_contiguous():
+        raise MmxError("Bpacked must be a contiguous uint8 tensor (from repack_b)")
+    need = _packed_bytes_host(b_dt, K, N)
+    if Bpacked.numel() < need:
+        raise MmxError(f"Bpacked holds {Bpacked.numel()} bytes, a packed [{K}, {N}] matrix takes {need}")
+    Cout = ep.C
+    _is_2d(Cout, "C")
+    ncols = n1 // 2 if ep.steps & PP_SILU_GATE else n1
+    if Cout.shape[0] < M or Cout.shape[1] < ncols:
+        raise MmxError(f"C is {tuple(Cout.shape)}, the result needs at least [{M}, {ncols}]")
+    for v, name in ((ep.bias, "bias"), (ep.deq_oc, "deq_scale_per_oc"), (ep.q_oc, "q_scale_per_oc")):
+        if v is not None and v.numel() < n1:
+            raise MmxError(f"{name} holds {v.numel()} values, columns up to {n1} are computed")
+    return M, K, a_dt
+
+
+def _packed_bytes_host(dtype, K, N):
+    """mmx_packed_b_bytes restated on the host (so that arguments can be checked before the library is loaded)."""
+    if K <= 0 or N <= 0:
+        return 0
+    if dtype == I4:
+        return ((N + 31) // 32) * ((K + 255) // 256 * 4) * 1024
+    es = {BF16: 2, I8: 1}.get(dtype, 0)
+    return ((N + 31) // 32) * 32 * ((K * es + 127) // 128 * 128)
+
+
+def _split_args(A, k_splits, ws):
+    """(k_splits, workspace pointer, bytes): without an explicit workspace the stream's own one is used."""
+    if k_splits == 1:
+        return 1, None, 0
+    if ws is None:
+        ws = workspace(A.device)
+    if ws is None:
+        if k_splits > 1:
+            raise MmxError("a K split needs a workspace, and none can be allocated while the stream is being captured")
+        return 1, None, 0
+    if ws.dtype != torch.uint8 or not ws.is_cuda or not ws.is_contiguous():
+        raise MmxError("the workspace must be a contiguous uint8 tensor on the GPU")
+    return k_splits, ws.data_ptr(), ws.numel()
+
+
+def gemm(A, Bpacked, N, ep, b_dtype=None, n0=0, n1=None, k_splits=0, ws=None):
+    """C[:, n0:n1] = PP(A · B[:, n0:n1]); A [M,K] bf16/int8, Bpacked from repack_b of the full [K,N].
+    k_splits: 0 = the library decides whether to split K over several workgroups per tile, 1 = never,
+    2..4 = exactly that many slices; ws = the workspace for the partial sums (default: the stream's own)."""
+    n1 = N if n1 is None else n1
+    b_dt = (dtype_code(A) if isinstance(A, torch.Tensor) else None) if b_dtype is None else b_dtype
+    M, K, a_dt = _check_gemm_args(A, Bpacked, N, ep, b_dt, n0, n1)
     _dev(A, "A"), _dev(Bpacked, "Bpacked")
-    M, K = A.shape
-    a_dt = dtype_code(A)
-    b_dt = a_dt if b_dtype is None else b_dtype
-    n1 = N if n1 is None else n1
     s = ep.struct()
-    _check(lib().mmx_gemm(a_dt, b_dt, A.data_ptr(), _row_stride_bytes(A), Bpacked.data_ptr(), M, K, N, n0, n1,
-                          C.byref(s), _stream()))
+    ks, wsp, wsb = _split_args(A, k_splits, ws)
+    _check(lib().mmx_gemm_splitk(a_dt, b_dt, A.data_ptr(), _row_stride_bytes(A), Bpacked.data_ptr(), M, K, N, n0, n1,
+                                 C.byref(s), ks, wsp, wsb, _stream()))
 
 
-def time_gemm(A, Bpacked_list, N, ep, iters, b_dtype=None, n0=0, n1=None):
+def gemm_workspace_bytes(a_dtype, b_dtype, M, K, N, steps=PP_NONE, k_splits=0, n0=0, n1=None):
+    return lib().mmx_gemm_workspace_bytes(a_dtype, b_dtype, M, K, N, n0, N if n1 is None else n1, int(steps), k_splits)
+
+
+def time_gemm(A, Bpacked_list, N, ep, iters, b_dtype=None, n0=0, n1=None, k_splits=0, ws=None):
     """Average ms per launch over `iters` back-to-back launches, rotating over the weight copies."""
-    _dev(A, "A")
-    M, K = A.shape
-    a_dt = dtype_code(A)
-    b_dt = a_dt if b_dtype is None else b_dtype
     n1 = N if n1 is None else n1
+    b_dt = (dtype_code(A) if isinstance(A, torch.Tensor) else None) if b_dtype is None else b_dtype
+    for Bp in Bpacked_list:
+        M, K, a_dt = _check_gemm_args(A, Bp, N, ep, b_dt, n0, n1)
+        _dev(Bp, "Bpacked")
+    _dev(A, "A")
     s = ep.struct()
     arr = (C.c_void_p * len(Bpacked_list))(*[b.data_ptr() for b in Bpacked_list])
     ms = C.c_float(0)
+    ks, wsp, wsb = _split_args(A, k_splits, ws)
     _check(lib().mmx_time_gemm(a_dt, b_dt, A.data_ptr(), _row_stride_bytes(A), arr, len(Bpacked_list), M, K, N, n0,
-                               n1, C.byref(s), _stream(), iters, C.byref(ms)))
+                               n1, C.byref(s), ks, wsp, wsb, _stream(), iters, C.byref(ms)))
     return ms.value
 
 
@@ -233,24 +326,52 @@ def probe_mfma(dtype, random_operands, iters=20000):
 
 
 def matvec(A, b, out=None):
-    _dev(A, "A"), _dev(b, "b")
+    """c[M] = A[M,K] · b[K]; bf16 (c fp32) or int8 (c int32)."""
+    _is_2d(A, "A")
     M, K = A.shape
     dt = dtype_code(A)
+    if dt not in (BF16, I8):
+        raise MmxError("A must be bf16 or int8")
+    if not isinstance(b, torch.Tensor) or b.dtype != A.dtype or b.numel() != K or not b.is_contiguous():
+        raise MmxError(f"b must be a contiguous {A.dtype} vector of K = {K} elements")
+    want = torch.float32 if dt == BF16 else torch.int32
+    if out is not None and (out.dtype != want or out.numel() < M or not out.is_contiguous()):
+        raise MmxError(f"out must be a contiguous {want} vector of at least M = {M} elements")
+    _dev(A, "A"), _dev(b, "b")
     if out is None:
-        out = torch.empty(M, dtype=torch.float32 if dt == BF16 else torch.int32, device=A.device)
+        out = torch.empty(M, dtype=want, device=A.device)
+    _dev(out, "out")
     _check(lib().mmx_matvec(dt, A.data_ptr(), _row_stride_bytes(A), b.data_ptr(), out.data_ptr(), M, K, _stream()))
     return out
 
 
-def mlp(x, w_gate_up, w_down, N, h=None, y=None):
-    _dev(x, "x")
+def mlp(x, w_gate_up, w_down, N, h=None, y=None, down_k_splits=0, ws=None):
+    """h = bf16(silu(x·Wg) * (x·Wu)), y = bf16(h·Wd): x [M,K] bf16, w_gate_up from repack_gate_up, w_down from
+    repack_b(transpose=True) of the [K,N] down_proj weight.  down_k_splits: K slices of the down projection
+    (0 = the library chooses, 1 = none, 2 = the reference's two-way split)."""
+    _is_2d(x, "x")
     M, K = x.shape
+    if x.dtype != torch.bfloat16:
+        raise MmxError("x must be bf16")
+    if not isinstance(N, int) or N <= 0 or N % 32:
+        raise MmxError("N must be a positive multiple of 32")
+    for t, name, need in ((w_gate_up, "w_gate_up", _packed_bytes_host(BF16, K, 2 * N)), (w_down, "w_down", _packed_bytes_host(BF16, N, K))):
+        if not isinstance(t, torch.Tensor) or t.dtype != torch.uint8 or not t.is_contiguous() or t.numel() < need:
+            raise MmxError(f"{name} must be a contiguous uint8 tensor of at least {need} bytes (packed weights)")
+    for t, name, cols in ((h, "h", N), (y, "y", K)):
+        if t is not None:
+            _is_2d(t, name)
+            if t.dtype != torch.bfloat16 or t.shape[0] < M or t.shape[1] < cols:
+                raise MmxError(f"{name} must be bf16 of at least [{M}, {cols}]")
+    _dev(x, "x"), _dev(w_gate_up, "w_gate_up"), _dev(w_down, "w_down")
     if h is None:
         h = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
     if y is None:
         y = torch.empty((M, K), dtype=torch.bfloat16, device=x.device)
-    _check(lib().mmx_mlp(x.data_ptr(), _row_stride_bytes(x), w_gate_up.data_ptr(), w_down.data_ptr(), h.data_ptr(),
-                         _row_stride_bytes(h), y.data_ptr(), _row_stride_bytes(y), M, K, N, _stream()))
+    _dev(h, "h"), _dev(y, "y")
+    ks, wsp, wsb = _split_args(x, down_k_splits, ws) if M > 32 else (1, None, 0)
+    _check(lib().mmx_mlp_splitk(x.data_ptr(), _row_stride_bytes(x), w_gate_up.data_ptr(), w_down.data_ptr(), h.data_ptr(),
+                                _row_stride_bytes(h), y.data_ptr(), _row_stride_bytes(y), M, K, N, ks, wsp, wsb, _stream()))
     return h, y
 
 

@@ -3,13 +3,16 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "common.hpp"
 
 namespace mmx {
 
 static thread_local char g_err[512] = "";
 static thread_local char g_kernel[128] = "";
-static int g_cus = 0;
+static std::atomic<int> g_cus{0};
+static std::mutex g_attr_mutex;
 
 int set_error(int code, const char* fmt, ...) {
     va_list ap;
@@ -29,12 +32,31 @@ void note_kernel(const char* name) {
     g_kernel[sizeof g_kernel - 1] = 0;
 }
 
-int num_cus() { return g_cus > 0 ? g_cus : 256; }
+int num_cus() {
+    const int c = g_cus.load(std::memory_order_relaxed);
+    return c > 0 ? c : 256;
+}
+
+int ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done_on_device) {
+    int dev = 0;
+    int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
+    if (rc) return rc;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done_on_device.load(std::memory_order_acquire) & bit) return MMX_OK;
+    std::lock_guard<std::mutex> lock(g_attr_mutex);
+    if (done_on_device.load(std::memory_order_relaxed) & bit) return MMX_OK;
+    rc = check_hip(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes),
+                   "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+    if (!rc) done_on_device.fetch_or(bit, std::memory_order_release);
+    return rc;
+}
+
 
 int launch_gemm_tiles_bf16(const void* A, int64_t lda, const void* Bp, int M, int K, int N, int n0, int n1,
-                           const Epilogue& ep, hipStream_t st);
+                           const Epilogue& ep, const SplitRequest& rq, hipStream_t st);
 int launch_gemm_tiles_i8(const void* A, int64_t lda, const void* Bp, int M, int K, int N, int n0, int n1,
-                         const Epilogue& ep, hipStream_t st);
+                         const Epilogue& ep, const SplitRequest& rq, hipStream_t st);
+size_t plan_workspace_bytes(int elesz, int M, int K, int Ncols, uint32_t steps, int k_splits);
 bool skinny_i8_eligible(const void* x, int64_t ldx, int M, int K);
 int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
                   const Epilogue& ep, hipStream_t st);
@@ -51,9 +73,10 @@ int launch_matvec(bool i8, const void* A, int64_t lda, const void* b, void* c, i
 struct TileCfg {
     int bm, bn;
 };
-static TileCfg g_forced = {0, 0};
-static int g_load_mode = 2;
-static int g_decode_halves = -1;
+// tuning knobs: per thread, like the error string, so that one thread's choice never changes another's dispatch
+static thread_local TileCfg g_forced = {0, 0};
+static thread_local int g_load_mode = 2;
+static thread_local int g_decode_halves = -1;
 TileCfg forced_tile() { return g_forced; }
 int load_mode() { return g_load_mode; }
 int decode_halves() { return g_decode_halves; }
@@ -69,7 +92,7 @@ static int out_size(int dtype) {
     }
 }
 
-static int make_epilogue(const mmx_epilogue* in, int a_dtype, int b_dtype, int n0, Epilogue* out) {
+static int make_epilogue(const mmx_epilogue* in, int a_dtype, int b_dtype, int M, int n0, int n1, Epilogue* out) {
     if (!in) return set_error(MMX_E_INVALID, "epilogue descriptor is NULL");
     if (!in->C) return set_error(MMX_E_INVALID, "epilogue: output pointer C is NULL");
     const int sz = out_size(in->out_dtype);
@@ -90,6 +113,11 @@ static int make_epilogue(const mmx_epilogue* in, int a_dtype, int b_dtype, int n
         return set_error(MMX_E_INVALID, "epilogue: int32 output is the raw accumulator of an int8 GEMM (steps must be 0)");
     if (in->ldc_bytes % sz) return set_error(MMX_E_INVALID, "epilogue: ldc_bytes %lld is not a multiple of the element size", (long long)in->ldc_bytes);
     if (reinterpret_cast<uintptr_t>(in->C) % sz) return set_error(MMX_E_INVALID, "epilogue: C is not aligned to its element size");
+    // C points at column 0 of the full row: a row must hold the columns up to n1 (half of them with SILU_GATE),
+    // or rows would overlap (a single row has no stride to speak of)
+    const int64_t row_bytes = (int64_t)((in->steps & MMX_PP_SILU_GATE) ? n1 / 2 : n1) * sz;
+    if (M > 1 && in->ldc_bytes < row_bytes)
+        return set_error(MMX_E_INVALID, "epilogue: ldc_bytes %lld smaller than the %lld bytes of a row of C", (long long)in->ldc_bytes, (long long)row_bytes);
     out->steps = in->steps;
     out->out_dtype = in->out_dtype;
     out->C = static_cast<char*>(in->C);
@@ -104,7 +132,7 @@ static int make_epilogue(const mmx_epilogue* in, int a_dtype, int b_dtype, int n
 }
 
 static int gemm_dispatch(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* Bpacked, int M, int K,
-                         int N, int n0, int n1, const mmx_epilogue* ep_in, hipStream_t st) {
+                         int N, int n0, int n1, const mmx_epilogue* ep_in, const SplitRequest& rq, hipStream_t st) {
     if (!A || !Bpacked) return set_error(MMX_E_INVALID, "mmx_gemm: NULL operand");
     if (M <= 0 || K <= 0 || N <= 0) return set_error(MMX_E_INVALID, "mmx_gemm: M, K, N must be positive (got %d, %d, %d)", M, K, N);
     const bool bf = a_dtype == MMX_BF16 && b_dtype == MMX_BF16;
@@ -120,16 +148,21 @@ static int gemm_dispatch(int a_dtype, int b_dtype, const void* A, int64_t lda_by
     if (lda_bytes % esa || reinterpret_cast<uintptr_t>(A) % esa) return set_error(MMX_E_INVALID, "mmx_gemm: A is not aligned to its element size");
     if (reinterpret_cast<uintptr_t>(Bpacked) & 15) return set_error(MMX_E_INVALID, "mmx_gemm: packed weights must be 16-byte aligned");
     Epilogue ep;
-    int rc = make_epilogue(ep_in, a_dtype, b_dtype, n0, &ep);
+    int rc = make_epilogue(ep_in, a_dtype, b_dtype, M, n0, n1, &ep);
     if (rc) return rc;
+    if (rq.k_splits < 0) return set_error(MMX_E_INVALID, "mmx_gemm: k_splits = %d", rq.k_splits);
+    if (rq.ws && (reinterpret_cast<uintptr_t>(rq.ws) & 255)) return set_error(MMX_E_INVALID, "mmx_gemm: the workspace must be 256-byte aligned");
+    // the decode kernels walk the whole of K in one workgroup per panel: they take no explicit K split
+    const bool decode = (M <= 32 && !i8) || (i8 && skinny_i8_eligible(A, lda_bytes, M, K) && forced_tile().bm == 0);
+    if (decode && rq.k_splits > 1) return set_error(MMX_E_UNSUPPORTED, "mmx_gemm: the decode kernels (M <= 32) take no K split");
     if ((ep.steps & MMX_PP_SILU_GATE) && ((n1 - n0) % 64)) return set_error(MMX_E_INVALID, "mmx_gemm: SILU_GATE needs (n1 - n0) %% 64 == 0");
     if (M <= 32 && !i8) return launch_skinny(w4 ? 2 : (w8 ? 1 : 0), A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st);
     if (i8 && skinny_i8_eligible(A, lda_bytes, M, K) && forced_tile().bm == 0)
         return launch_skinny(3, A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st);
     if (w4) return set_error(MMX_E_UNSUPPORTED, "mmx_gemm: bf16 x int4-weight is a decode path (M <= 32)");
     if (w8) return set_error(MMX_E_UNSUPPORTED, "mmx_gemm: bf16 x int8-weight with M > 32: convert the weights with mmx_dequant_packed and call the bf16 GEMM");
-    return i8 ? launch_gemm_tiles_i8(A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st)
-              : launch_gemm_tiles_bf16(A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st);
+    return i8 ? launch_gemm_tiles_i8(A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, rq, st)
+              : launch_gemm_tiles_bf16(A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, rq, st);
 }
 
 }  // namespace mmx
@@ -193,6 +226,9 @@ int mmx_quantize_weights(const void* W, int64_t ldw_bytes, int rows, int cols, v
     if (!W || !Wq || !scales_out || !absmax_scratch) return set_error(MMX_E_INVALID, "mmx_quantize_weights: NULL pointer");
     if (rows <= 0 || cols <= 0 || ldw_bytes < (int64_t)cols * 2 || ldq_bytes < cols)
         return set_error(MMX_E_INVALID, "mmx_quantize_weights: bad shape or stride");
+    if ((ldw_bytes & 1) || (reinterpret_cast<uintptr_t>(W) & 1) || (reinterpret_cast<uintptr_t>(scales_out) & 3) ||
+        (reinterpret_cast<uintptr_t>(absmax_scratch) & 3))
+        return set_error(MMX_E_INVALID, "mmx_quantize_weights: W, scales_out or absmax_scratch is not aligned to its element size");
     return launch_quantize(W, ldw_bytes, rows, cols, Wq, ldq_bytes, scales_out, absmax_scratch, static_cast<hipStream_t>(stream));
 }
 
@@ -216,7 +252,21 @@ int mmx_dequant_packed(const void* packed_i8, int K, int N, void* packed_bf16, v
 
 int mmx_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* Bpacked, int M, int K, int N, int n0,
              int n1, const mmx_epilogue* ep, void* stream) {
-    return gemm_dispatch(a_dtype, b_dtype, A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, static_cast<hipStream_t>(stream));
+    const SplitRequest none = {1, nullptr, 0};
+    return gemm_dispatch(a_dtype, b_dtype, A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, none, static_cast<hipStream_t>(stream));
+}
+
+int mmx_gemm_splitk(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* Bpacked, int M, int K, int N, int n0,
+                    int n1, const mmx_epilogue* ep, int k_splits, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!workspace && k_splits > 1) return set_error(MMX_E_INVALID, "mmx_gemm_splitk: %d K slices need a workspace", k_splits);
+    const SplitRequest rq = {workspace ? k_splits : 1, static_cast<char*>(workspace), workspace_bytes};
+    return gemm_dispatch(a_dtype, b_dtype, A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, rq, static_cast<hipStream_t>(stream));
+}
+
+size_t mmx_gemm_workspace_bytes(int a_dtype, int b_dtype, int M, int K, int N, int n0, int n1, uint32_t steps, int k_splits) {
+    const bool bf = a_dtype == MMX_BF16 && b_dtype == MMX_BF16, i8 = a_dtype == MMX_I8 && b_dtype == MMX_I8;
+    if ((!bf && !i8) || M <= 32 || K <= 0 || N <= 0 || n0 < 0 || n1 > N || n0 >= n1 || k_splits < 0) return 0;
+    return plan_workspace_bytes(bf ? 2 : 1, M, K, n1 - n0, steps, k_splits);
 }
 
 int mmx_matvec(int dtype, const void* A, int64_t lda_bytes, const void* b, void* c, int M, int K, void* stream) {
@@ -224,11 +274,18 @@ int mmx_matvec(int dtype, const void* A, int64_t lda_bytes, const void* b, void*
     if (!es) return set_error(MMX_E_INVALID, "mmx_matvec: dtype %d is neither bf16 nor int8", dtype);
     if (!A || !b || !c || M <= 0 || K <= 0) return set_error(MMX_E_INVALID, "mmx_matvec: bad argument");
     if (lda_bytes < (int64_t)K * es) return set_error(MMX_E_INVALID, "mmx_matvec: lda_bytes smaller than a row of A");
+    if (lda_bytes % es || (reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(b)) % es || reinterpret_cast<uintptr_t>(c) % 4)
+        return set_error(MMX_E_INVALID, "mmx_matvec: A, b or c is not aligned to its element size");
     return launch_matvec(dtype == MMX_I8, A, lda_bytes, b, c, M, K, static_cast<hipStream_t>(stream));
 }
 
 int mmx_mlp(const void* x, int64_t ldx_bytes, const void* w_gate_up, const void* w_down, void* h, int64_t ldh_bytes, void* y,
             int64_t ldy_bytes, int M, int K, int N, void* stream) {
+    return mmx_mlp_splitk(x, ldx_bytes, w_gate_up, w_down, h, ldh_bytes, y, ldy_bytes, M, K, N, 1, nullptr, 0, stream);
+}
+
+int mmx_mlp_splitk(const void* x, int64_t ldx_bytes, const void* w_gate_up, const void* w_down, void* h, int64_t ldh_bytes, void* y,
+                   int64_t ldy_bytes, int M, int K, int N, int down_k_splits, void* workspace, size_t workspace_bytes, void* stream) {
     if (!x || !w_gate_up || !w_down || !h || !y) return set_error(MMX_E_INVALID, "mmx_mlp: NULL pointer");
     if (N % 32) return set_error(MMX_E_INVALID, "mmx_mlp: N = %d must be a multiple of 32", N);
     mmx_epilogue e1;
@@ -245,7 +302,11 @@ int mmx_mlp(const void* x, int64_t ldx_bytes, const void* w_gate_up, const void*
     e2.out_dtype = MMX_BF16;
     e2.C = y;
     e2.ldc_bytes = ldy_bytes;
-    return mmx_gemm(MMX_BF16, MMX_BF16, h, ldh_bytes, w_down, M, N, K, 0, K, &e2, stream);
+    // AMX_MLP::MLP::setup builds `down` with do_splitK (tests/amx-mlp.cpp:768): two halves of its K blocks, summed
+    // and rounded to bf16 by the half that finishes last (:648-682).  The decode kernels (M <= 32) sum K inside one
+    // workgroup and take no slices.
+    if (M <= 32 || !workspace) return mmx_gemm(MMX_BF16, MMX_BF16, h, ldh_bytes, w_down, M, N, K, 0, K, &e2, stream);
+    return mmx_gemm_splitk(MMX_BF16, MMX_BF16, h, ldh_bytes, w_down, M, N, K, 0, K, &e2, down_k_splits, workspace, workspace_bytes, stream);
 }
 
 int mmx_set_tile(const char* shape) {
@@ -279,8 +340,10 @@ int mmx_probe_mfma(int dtype, int random_operands, int iters, void* scratch, voi
 }
 
 int mmx_time_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* const* Bpacked_rot, int n_rot, int M,
-                  int K, int N, int n0, int n1, const mmx_epilogue* ep, void* stream, int iters, float* ms_out) {
+                  int K, int N, int n0, int n1, const mmx_epilogue* ep, int k_splits, void* workspace, size_t workspace_bytes,
+                  void* stream, int iters, float* ms_out) {
     if (!Bpacked_rot || n_rot <= 0 || iters <= 0 || !ms_out) return set_error(MMX_E_INVALID, "mmx_time_gemm: bad argument");
+    const SplitRequest rq = {workspace ? k_splits : 1, static_cast<char*>(workspace), workspace_bytes};
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipEvent_t e0, e1;
     int rc = check_hip(hipEventCreate(&e0), "hipEventCreate");
@@ -289,7 +352,7 @@ int mmx_time_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, co
     if (rc) { (void)hipEventDestroy(e0); return rc; }
     rc = check_hip(hipEventRecord(e0, st), "hipEventRecord");
     for (int i = 0; i < iters && !rc; i++)
-        rc = gemm_dispatch(a_dtype, b_dtype, A, lda_bytes, Bpacked_rot[i % n_rot], M, K, N, n0, n1, ep, st);
+        rc = gemm_dispatch(a_dtype, b_dtype, A, lda_bytes, Bpacked_rot[i % n_rot], M, K, N, n0, n1, ep, rq, st);
     if (!rc) rc = check_hip(hipEventRecord(e1, st), "hipEventRecord");
     if (!rc) rc = check_hip(hipEventSynchronize(e1), "hipEventSynchronize");
     float ms = 0.0f;

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/mm_amx_amd.h"
 
 namespace mmx {
@@ -22,6 +24,9 @@ int set_error(int code, const char* fmt, ...);
 int check_hip(hipError_t e, const char* what);
 void note_kernel(const char* name);
 int num_cus();
+// Raises a kernel's dynamic LDS limit to `bytes` on the current device, once per device; `done_on_device`
+// (one per kernel, a bit per device) records where that has happened.  Safe to call from any thread.
+int ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done_on_device);
 
 struct Epilogue {
     uint32_t steps;
@@ -34,6 +39,13 @@ struct Epilogue {
     float q;
     const float* q_oc;
     int c_vec_ok;  // C and ldc are 16-byte aligned
+};
+
+// A caller's request for a split of K over several workgroups per tile, and the memory for its partial sums.
+struct SplitRequest {
+    int k_splits;     // 0: choose; 1: none; 2 and up: exactly this many slices
+    char* ws;         // workspace (NULL: no split possible)
+    size_t ws_bytes;
 };
 
 // ---- element-wise epilogue arithmetic -----------------------------------------------------

@@ -1,21 +1,26 @@
-// int8 x int8 -> int32 MFMA tile GEMM instantiations (v_mfma_i32_32x32x32_i8).
+// i8 x i8 MFMA tile GEMM (v_mfma_i32_32x32x32_i8): launch geometry and dispatch on the output type.
 #include "gemm_tile.hpp"
 
 namespace mmx {
 
+int launch_tiles_i8_out_f32(const GemmArgs& g, TileCfg t, int mode, int grid, hipStream_t st);
+int launch_tiles_i8_out_bf16(const GemmArgs& g, TileCfg t, int mode, int grid, hipStream_t st);
+int launch_tiles_i8_out_i8(const GemmArgs& g, TileCfg t, int mode, int grid, hipStream_t st);
+int launch_tiles_i8_out_i32(const GemmArgs& g, TileCfg t, int mode, int grid, hipStream_t st);
+
 int launch_gemm_tiles_i8(const void* A, int64_t lda, const void* Bp, int M, int K, int N, int n0, int n1,
-                         const Epilogue& ep, hipStream_t st) {
+                           const Epilogue& ep, const SplitRequest& rq, hipStream_t st) {
     GemmArgs g;
     TileCfg t;
     int mode;
-    const int grid = prepare_gemm(g, t, mode, 1, A, lda, Bp, M, K, N, n0, n1, ep);
+    const int grid = prepare_gemm(g, t, mode, 1, A, lda, Bp, M, K, N, n0, n1, ep, rq);
     if (grid < 0) return grid;
     switch (ep.out_dtype) {
-    case MMX_F32: return launch_tiles<int8_t, float>(g, t, mode, grid, st);
-    case MMX_BF16: return launch_tiles<int8_t, uint16_t>(g, t, mode, grid, st);
-    case MMX_I8: return launch_tiles<int8_t, int8_t>(g, t, mode, grid, st);
-    case MMX_I32: return launch_tiles<int8_t, int32_t>(g, t, mode, grid, st);
-    default: return set_error(MMX_E_INVALID, "int8 GEMM: output dtype %d not supported", ep.out_dtype);
+    case MMX_F32: return launch_tiles_i8_out_f32(g, t, mode, grid, st);
+    case MMX_BF16: return launch_tiles_i8_out_bf16(g, t, mode, grid, st);
+    case MMX_I8: return launch_tiles_i8_out_i8(g, t, mode, grid, st);
+    case MMX_I32: return launch_tiles_i8_out_i32(g, t, mode, grid, st);
+    default: return set_error(MMX_E_INVALID, "i8 GEMM: output dtype %d not supported", ep.out_dtype);
     }
 }
 

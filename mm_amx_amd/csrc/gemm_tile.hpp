@@ -25,6 +25,7 @@
 //           multiple of 128) and for A rows that are not 16-byte aligned.  Rows past M and
 //           elements past K are read as zero, never touched in memory.
 #pragma once
+#include <atomic>
 #include <type_traits>
 
 #include "common.hpp"
@@ -84,8 +85,12 @@ struct GemmArgs {
     int nk;       // k-iterations of 128 bytes
     int npanels;  // 32-column panels in Bp
     int n0, n1;
-    int tiles_m, total_tiles, tiles_per_xcd;
+    int tiles_m, total_tiles, tiles_per_xcd;  // total_tiles and tiles_per_xcd count (tile, K slice) units
     int a_vec_ok;  // A and lda 16-byte aligned
+    int ksplit;    // K slices per tile (1: every workgroup walks the whole of K)
+    int kq;        // k-iterations per slice
+    char* ws_part;     // partial accumulators of the K slices: [tile][slice][BM*BN] 4-byte words
+    uint32_t* ws_cnt;  // one arrival counter per tile, zero between launches
     Epilogue ep;
 };
 
@@ -112,22 +117,41 @@ __device__ __forceinline__ u32x4 load_a_chunk_masked(const char* rowptr, int kby
     return u32x4{w[0], w[1], w[2], w[3]};
 }
 
-// LDS ring of the hand-scheduled pipeline: R half-stages of (BM + BN) rows x 64 bytes.
+// LDS ring of the hand-scheduled pipeline: RA stages of A (BM rows x 128 bytes) and R half-stages of B (BN columns
+// x 64 bytes).  The ring is as deep as 156 KiB of LDS allow (R <= 2 RA - 2, see the pipeline): the loads of R - 1
+// half-stages are in flight while one is multiplied, and a small tile multiplies a half-stage in far less time
+// than a load takes (128x64: 128 cycles of MFMA issue against 1000+ cycles of L2 latency - with three half-stages
+// in flight that tile was bound by latency, 350 cycles per half-stage).  The large tiles get 3 or 4 as before:
+// their half-stages are long enough.
 template <int BM, int BN>
 struct Ring {
     static constexpr int A_ST = BM * 128;  // A: one stage = 128 bytes of K per row (whole cache lines)
     static constexpr int BH = BN * 64;     // B: one half-stage = 64 bytes of K per column (two fragments per panel)
-    static constexpr int RA = 3;           // A stages in LDS
-    static constexpr int R = (RA * A_ST + 4 * BH <= 156 * 1024) ? 4 : 3;  // B half-stages in LDS (R <= 2 RA - 2)
-    static constexpr int B0 = RA * A_ST;   // the B ring follows the A ring
+    static constexpr int NL = BM / 64 + BN / 64;  // HBM->LDS loads per thread per half-stage
+    static constexpr int stages_for(int r) { return (r + 3) / 2; }
+    static constexpr bool fits(int r) {
+        return stages_for(r) * A_ST + r * BH <= 156 * 1024 && (r - 2) * NL + (NL + 1) / 2 <= 63;  // LDS; vmcnt is a 6-bit counter
+    }
+    static constexpr int depth() {
+        int r = 3;
+        for (int c = 4; c <= 12; c++)
+            if (fits(c)) r = c;
+        return r;
+    }
+    static constexpr int R = depth();          // B half-stages in LDS
+    static constexpr int RA = stages_for(R);   // A stages in LDS
+    static constexpr int B0 = RA * A_ST;       // the B ring follows the A ring
     static constexpr int BYTES = B0 + R * BH;
 };
 
-template <typename TIn, int BM, int BN, int MODE, typename TOut>
+// SMAX: the largest number of K slices per tile this instantiation can combine (1: no K split; the
+// code of the split is then absent and the kernel is the plain one).
+template <typename TIn, int BM, int BN, int MODE, typename TOut, int SMAX>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_kernel(const GemmArgs g) {
     using MF = Mfma<TIn>;
     using frag = typename MF::frag;
     using accv = typename MF::accv;
+    using acc_t = typename std::conditional<std::is_same<TIn, int8_t>::value, int, float>::type;
     // the four waves form a 2x2 grid over the tile, or 4x1 when the tile is only 64 columns wide
     constexpr int WGN = BN >= 128 ? 2 : 1, WGM = 4 / WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -147,7 +171,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // contiguous run of tiles (m fastest): tiles that share a B panel run on one L2.
     const int L = (blockIdx.x & 7) * g.tiles_per_xcd + (blockIdx.x >> 3);
     if (L >= g.total_tiles) return;
-    const int tn = L / g.tiles_m, tm = L % g.tiles_m;
+    // K split: the slices of a tile are neighbours in L, so they run on one XCD and meet in its L2
+    int tile = L, slice = 0, kt0 = 0, nk = g.nk;
+    if constexpr (SMAX > 1) {
+        tile = L / g.ksplit;
+        slice = L - tile * g.ksplit;
+        kt0 = slice * g.kq;
+        nk = g.nk - kt0 < g.kq ? g.nk - kt0 : g.kq;
+    }
+    const char* const a_base = g.A + (int64_t)kt0 * 128;
+    const int tn = tile / g.tiles_m, tm = tile % g.tiles_m;
     const int m0 = tm * BM;
     const int ntile0 = g.n0 + tn * BN;
     const int panel0 = ntile0 >> 5;
@@ -269,10 +302,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             panel = panel < g.npanels ? panel : g.npanels - 1;
             boff[it] = (uint32_t)(panel - panel0) * (uint32_t)g.panel_stride + (uint32_t)((c & 127) * 16);
         }
-        const char* const b_base = g.Bp + (int64_t)panel0 * g.panel_stride;
+        const char* const b_base = g.Bp + (int64_t)panel0 * g.panel_stride + (int64_t)kt0 * 4096;
         const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(
             (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)(smem + wave * 1024));
-        const int last_hs = 2 * g.nk - 1, last_st = g.nk - 1;
+        const int last_hs = 2 * nk - 1, last_st = nk - 1;
 
         using std::integral_constant;
         typedef integral_constant<int, 0> c0;
@@ -316,7 +349,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             } else if constexpr (PART == 2) {
                 int st = (w + 1) >> 1;
                 st = st < last_st ? st : last_st;
-                n.srcA = g.A + (int64_t)st * 128;
+                n.srcA = a_base + (int64_t)st * 128;
                 asm volatile("" : "+s"(n.srcA));
             } else {
                 // A operand of k-step s (0..3 within the stage): position (2 s + g32) ^ ((row >> 1) & 7) of the row
@@ -380,7 +413,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         {
             KParams kp;
             kp.m0A = lds_wave;
-            kp.srcA = g.A;
+            kp.srcA = a_base;
             static_for<0, A_IT2>([&](auto it_c) { dma(integral_constant<int, B_IT2 + decltype(it_c)::value>{}, c0{}, kp); });
             static_for<0, R>([&](auto w_c) {
                 constexpr int W = decltype(w_c)::value;
@@ -391,7 +424,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 kp.m0B = lds_wave + B0 + W * BH;
                 kp.m0A = lds_wave + (((W + 1) >> 1) % RA) * A_ST + HALF * (BM / 2) * 128;
                 kp.srcB = b_base + (int64_t)hs * 2048;
-                kp.srcA = g.A + (int64_t)st * 128;
+                kp.srcA = a_base + (int64_t)st * 128;
                 static_for<0, (W < R - 1 ? NL : H)>([&](auto q_c) { dma(q_c, integral_constant<int, HALF>{}, kp); });
             });
         }
@@ -442,7 +475,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         }
         asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // the re-fetched slots past the end must land before the wave ends
     } else {
-    fetch(0);
+    fetch(kt0);
     commit(0);
     __syncthreads();
     read_frags(0, 0, fa[0], fb[0]);
@@ -457,12 +490,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     __builtin_amdgcn_sched_group_barrier(0x008, MI * NJ - (MI + NJ), 0);   \
     __builtin_amdgcn_sched_barrier(0)
 
-    for (int kt = 0; kt < g.nk; kt++) {
+    for (int kt = 0; kt < nk; kt++) {
         const int stage = kt & 1;
         // the last iteration re-fetches its own stage into the idle buffer: harmless, and it keeps
         // the loop body free of branches so that the schedule below is one straight block
-        const int kt_next = (kt + 1 < g.nk) ? kt + 1 : kt;
-        fetch(kt_next);
+        const int kt_next = (kt + 1 < nk) ? kt + 1 : kt;
+        fetch(kt0 + kt_next);
         __builtin_amdgcn_sched_barrier(0);
         read_frags(stage, 1, fa[1], fb[1]);
         mma(fa[0], fb[0]);
@@ -490,6 +523,95 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // MFMAs retire (a 32x32 MFMA needs up to 18 wait states before its result may be read)
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
+    // ---- K split: park the partial sums, the last slice to arrive combines them ---------------------------
+    // Every slice writes its accumulators to its own part of the workspace (each lane 16 bytes per store,
+    // in the order it holds them, so the reader's lanes find their own elements again) and counts itself
+    // in.  The slice that finds all others counted adds the partial sums in slice order 0, 1, 2, ... - its
+    // own from registers - so the result does not depend on which slice came last, and goes on to the
+    // post-op.  The counter wraps to zero with the last arrival (atomicInc), ready for the next launch.
+    // Nobody waits for anybody.
+    // The partial sums cross from one workgroup to another, possibly on another XCD with its own L2:
+    // they are written and read at device scope (sc1: written through to, and read from, the level all
+    // XCDs share), the writer waits until its stores have been acknowledged before it counts itself in,
+    // and the counter is a device-scope atomic.  A device-scope fence would do the same for ordinary
+    // stores, but it writes back and invalidates the whole L2 - 25 us on a kernel of 15.
+    bool combine = false;
+    constexpr int AUX_SC1 = 16;  // cache policy operand of the buffer instructions: device scope
+    constexpr int TILE_BYTES = BM * BN * 4;
+    __amdgpu_buffer_rsrc_t parts;                                             // this tile's partial sums, all slices
+    const int part_lane = wave * (MI * NJ * 4096) + lane * 16;                // this lane's place in a slice's tile
+    if constexpr (SMAX > 1) {
+        if (g.ksplit > 1) {
+            parts = __builtin_amdgcn_make_buffer_rsrc(g.ws_part + (int64_t)tile * g.ksplit * TILE_BYTES, 0, g.ksplit * TILE_BYTES, 0x00020000);
+            const int mine = slice * TILE_BYTES + part_lane;
+            static_for<0, MI * NJ>([&](auto bc) __attribute__((always_inline)) {
+                constexpr int b = decltype(bc)::value;
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    u32x4 w;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const acc_t a = acc_read(acc[b / NJ][b % NJ][4 * q + e]);
+                        w[e] = __builtin_bit_cast(uint32_t, a);
+                    }
+                    __builtin_amdgcn_raw_buffer_store_b128(w, parts, mine + (b * 4 + q) * 1024, 0, AUX_SC1);
+                }
+            });
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // every store of this wave has been acknowledged
+            __syncthreads();
+            if (tid == 0) *reinterpret_cast<volatile uint32_t*>(smem) = atomicInc(g.ws_cnt + tile, (uint32_t)g.ksplit - 1u);
+            __syncthreads();
+            if (*reinterpret_cast<volatile uint32_t*>(smem) != (uint32_t)g.ksplit - 1u) return;
+            asm volatile("" ::: "memory");
+            combine = true;
+        }
+    }
+    // the other slices' sums of block b (held by this lane), requested one block ahead of their use
+    acc_t pf[2][SMAX][16];
+    auto part_load = [&](auto bc, acc_t (&dst)[SMAX][16]) __attribute__((always_inline)) {
+        constexpr int b = decltype(bc)::value;
+        static_for<0, SMAX>([&](auto sc) __attribute__((always_inline)) {
+            constexpr int sl = decltype(sc)::value;
+            if (sl < g.ksplit && sl != slice) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(parts, sl * TILE_BYTES + part_lane + (b * 4 + q) * 1024, 0, AUX_SC1);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const uint32_t bits = w[e];  // (a bit_cast straight from the vector element reads element 0 with this compiler)
+                        dst[sl][4 * q + e] = __builtin_bit_cast(acc_t, bits);
+                    }
+                }
+            }
+        });
+    };
+    // block (i, j) of the finished sum: the accumulators, or slice 0 + slice 1 + ... in that order
+    auto block_values = [&](auto ic, auto jc, auto step_c, acc_t (&vals)[16]) __attribute__((always_inline)) {
+        constexpr int i = decltype(ic)::value, j = decltype(jc)::value, step = decltype(step_c)::value;
+        if constexpr (SMAX > 1) {
+            if (combine) {
+                static_for<0, SMAX>([&](auto sc) __attribute__((always_inline)) {
+                    constexpr int sl = decltype(sc)::value;
+                    if (sl < g.ksplit) {
+                        acc_t x[16];
+                        if (sl == slice) {
+#pragma unroll
+                            for (int v = 0; v < 16; v++) x[v] = acc_read(acc[i][j][v]);
+                        } else {
+#pragma unroll
+                            for (int v = 0; v < 16; v++) x[v] = pf[step & 1][sl][v];
+                        }
+#pragma unroll
+                        for (int v = 0; v < 16; v++) vals[v] = sl == 0 ? x[v] : vals[v] + x[v];
+                    }
+                });
+                return;
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; v++) vals[v] = acc_read(acc[i][j][v]);
+    };
+
     // ---- epilogue: accumulators -> post-op -> global memory, block by block ---------------------------
     // The weights are the first MFMA operand, so a lane holds ONE output row of a 32x32 block
     // (m = lane % 32) and four runs of four consecutive columns (n = 8q + 4(lane / 32) + 0..3, q = 0..3).
@@ -515,9 +637,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             }
         }
     };
-    // stores the 16 values r[] (or raw int32 accumulators) of one block: row grow, output columns
+    // stores the 16 values r[] (or the raw int32 sums) of one block: row grow, output columns
     // ocol + 8(v/4) + 4 g32 + v%4
-    auto store_block = [&](const float (&r)[16], const accv& raw, int grow, int ocol) {
+    auto store_block = [&](const float (&r)[16], const acc_t (&raw)[16], int grow, int ocol) {
         constexpr int SZ = sizeof(TOut);
         constexpr int DW = SZ;  // dwords per run of four elements
         uint32_t w[4][DW];
@@ -567,7 +689,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         }
     };
 
-    if (silu_gate) {
+    if (silu_gate) {  // (never combined with a K split: the host refuses it)
         if constexpr (NJ % 2 == 0) {
             const uint32_t seg_of_lane = kRcp14Seg[lane];
             static_for<0, NJ / 2>([&](auto jc) __attribute__((always_inline)) {
@@ -575,18 +697,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 static_for<0, MI>([&](auto ic) __attribute__((always_inline)) {
                     constexpr int i = decltype(ic)::value;
                     float gt[16], up[16], r[16];
+                    acc_t raw[16];
 #pragma unroll
                     for (int v = 0; v < 16; v++) {
-                        gt[v] = MF::to_f32(acc_read(acc[i][j][v]));
+                        raw[v] = acc_read(acc[i][j][v]);
+                        gt[v] = MF::to_f32(raw[v]);
                         up[v] = MF::to_f32(acc_read(acc[i][j + 1][v]));
                     }
                     silu_mul_x16(gt, up, r, seg_of_lane);
-                    store_block(r, acc[i][j], m0 + wm * WM + 32 * i + l32, ((wave_col0 + 32 * j) >> 1));
+                    store_block(r, raw, m0 + wm * WM + 32 * i + l32, ((wave_col0 + 32 * j) >> 1));
                     __builtin_amdgcn_sched_barrier(0);
                 });
             });
         }
     } else {
+        // blocks are finished in the order step = j * MI + i; block b = i * NJ + j of the workspace
+        if constexpr (SMAX > 1) {
+            if (combine) part_load(std::integral_constant<int, 0>{}, pf[0]);
+        }
         static_for<0, NJ>([&](auto jc) __attribute__((always_inline)) {
             constexpr int j = decltype(jc)::value;
             const int bcol = wave_col0 + 32 * j;
@@ -596,9 +724,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             if ((ep.steps & MMX_PP_QUANT) && ep.q_oc) load_per_oc(ep.q_oc, bcol, q_v);
             static_for<0, MI>([&](auto ic) __attribute__((always_inline)) {
                 constexpr int i = decltype(ic)::value;
+                constexpr int step = j * MI + i;
+                if constexpr (SMAX > 1 && step + 1 < MI * NJ) {
+                    constexpr int ni = (step + 1) % MI, nj = (step + 1) / MI;
+                    if (combine) part_load(std::integral_constant<int, ni * NJ + nj>{}, pf[(step + 1) & 1]);
+                }
+                acc_t raw[16];
+                block_values(ic, jc, std::integral_constant<int, step>{}, raw);
                 float r[16];
 #pragma unroll
-                for (int v = 0; v < 16; v++) r[v] = MF::to_f32(acc_read(acc[i][j][v]));
+                for (int v = 0; v < 16; v++) r[v] = MF::to_f32(raw[v]);
                 if (ep.steps & MMX_PP_DEQUANT) {
                     if (ep.deq_oc) {
 #pragma unroll
@@ -622,7 +757,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                         for (int v = 0; v < 16; v++) r[v] = r[v] * ep.q;
                     }
                 }
-                store_block(r, acc[i][j], m0 + wm * WM + 32 * i + l32, bcol);
+                store_block(r, raw, m0 + wm * WM + 32 * i + l32, bcol);
                 __builtin_amdgcn_sched_barrier(0);
             });
         });
@@ -636,25 +771,63 @@ struct TileCfg {
 };
 TileCfg forced_tile();
 int load_mode();
+int ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done_on_device);
 
-// Pick the tile that minimises (tiles per CU, rounded up) x (work per tile) / (per-tile efficiency).
-// Workgroups that share a CU share its matrix pipe, so what counts is how many tiles the busiest CU
-// has to finish.  The efficiency factors are measured on the 1024 x 4096 x 11008 FC: larger tiles
-// re-use each LDS fragment for more MFMAs and load fewer bytes per flop.
-static inline TileCfg choose_tile(int M, int Ncols, bool need_pairs) {
-    const TileCfg f = forced_tile();
-    if (f.bm) return f;
+// Where the partial sums of a K split live: the first WS_COUNTER_BYTES hold one arrival counter per tile
+// (zero between launches), the partial tiles follow.
+constexpr int WS_MAX_TILES = 4096;
+constexpr size_t WS_COUNTER_BYTES = (size_t)WS_MAX_TILES * 4;
+constexpr int KSPLIT_MAX = 4;  // slices a kernel instantiation can combine (its SMAX)
+
+// K slices are whole blocks of 512 bytes of K per row (256 bf16: the K block of AMX_MLP::Linear,
+// tests/amx-mlp.cpp:548-566, whose two-way split S = 2 reproduces): slice s covers k-iterations
+// [s * kq, min((s + 1) * kq, nk)).
+static inline int slice_kiters(int nk, int S) { return 4 * (((nk + 3) / 4 + S - 1) / S); }
+
+struct Plan {
+    TileCfg t;
+    int S;
+};
+
+// Pick the tile shape and the number of K slices that minimise a model of the launch's duration, in
+// shader cycles of the busiest CU: rounds of resident workgroups x (prologue + main loop + epilogue
+// [+ parking and combining partial sums]).  The main loop takes the longer of MFMA issue (BM*BN/32 cycles
+// per k-iteration of 128 bytes, at the measured issue efficiency of the shape) and of pulling its
+// (BM + BN) * 128 bytes per k-iteration through the CU's L2 -> L1 path (about 48 bytes per cycle).
+// A K split is considered where the slices of all tiles are resident at once.
+static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, int mode, const SplitRequest& rq) {
     static const struct { int bm, bn; float eff; } cand[] = {
-        {256, 256, 1.00f}, {256, 192, 0.97f}, {128, 256, 0.90f}, {128, 192, 0.86f}, {128, 128, 0.80f}, {128, 64, 0.48f}};
+        {256, 256, 0.92f}, {256, 192, 0.90f}, {128, 256, 0.86f}, {128, 192, 0.84f}, {128, 128, 0.80f}, {128, 64, 0.70f}};
+    const TileCfg f = forced_tile();
     const int cus = num_cus();
+    const float l1_bytes_per_clk = 48.0f, ws_bytes_per_clk = 40.0f;
     float best = 1e30f;
-    TileCfg pick = {128, 128};
+    Plan pick = {{128, 128}, 1};
     for (const auto& c : cand) {
+        if (f.bm && (f.bm != c.bm || f.bn != c.bn)) continue;
         if (need_pairs && (c.bn % 128) != 0) continue;
+        if (mode == 3 && !(c.bm == 128 && c.bn == 128)) continue;   // the masked path exists for one tile shape
+        if (mode != 2 && c.bn == 64) continue;                      // the 64-wide tile exists for the ring pipeline only
         const int tiles = ((M + c.bm - 1) / c.bm) * ((Ncols + c.bn - 1) / c.bn);
-        const int per_cu = (tiles + cus - 1) / cus;
-        const float t = (float)per_cu * (float)(c.bm * c.bn) / c.eff;
-        if (t < best) { best = t; pick = {c.bm, c.bn}; }
+        for (int S = 1; S <= KSPLIT_MAX; S++) {
+            if (rq.k_splits > 0 && S != rq.k_splits) continue;
+            if (S > 1) {
+                if (need_pairs || c.bn == 64 || !rq.ws || tiles > WS_MAX_TILES) break;
+                const int kq = slice_kiters(nk, S);
+                if ((S - 1) * kq >= nk) continue;  // an empty last slice
+                if (WS_COUNTER_BYTES + (size_t)tiles * S * c.bm * c.bn * 4 > rq.ws_bytes) continue;
+                if (rq.k_splits == 0 && (tiles * S > cus || kq < 8)) continue;
+            }
+            const int kit = S > 1 ? slice_kiters(nk, S) : nk;
+            const float mfma = (float)(c.bm * c.bn / 32) / c.eff, bytes = (float)((c.bm + c.bn) * 128) / l1_bytes_per_clk;
+            const float loop = (float)kit * (mfma > bytes ? mfma : bytes);
+            const float epi = (float)(c.bm * c.bn / 256) * 100.0f;  // between a plain store (45) and a GELU (170): the plan must
+                                                                   // not depend on the post-op, or a GEMM and its fused form would sum differently
+            const float split = S > 1 ? 3000.0f + (float)(c.bm * c.bn * 4) * (float)S / ws_bytes_per_clk : 0.0f;
+            const int per_cu = (tiles * S + cus - 1) / cus;
+            const float t = (float)per_cu * (3700.0f + loop + epi + split);
+            if (t < best) { best = t; pick = {{c.bm, c.bn}, S}; }
+        }
     }
     return pick;
 }
@@ -666,48 +839,45 @@ template <> constexpr const char* type_tag<int8_t>() { return "i8"; }
 template <> constexpr const char* type_tag<int32_t>() { return "i32"; }
 template <> constexpr const char* type_tag<float>() { return "f32"; }
 
-template <typename TIn, int BM, int BN, int MODE, typename TOut>
+template <typename TIn, int BM, int BN, int MODE, typename TOut, int SMAX>
 static int launch_cfg(const GemmArgs& g, int grid, hipStream_t st) {
     constexpr int lds = MODE == 2 ? Ring<BM, BN>::BYTES : 2 * (BM + BN) * 128;
-    auto kern = gemm_kernel<TIn, BM, BN, MODE, TOut>;
-    static bool attr_done = false;  // one flag and one name per instantiation
-    static char name[64];
-    if (!name[0]) {
-        static const char* const loads[] = {"regs", "", "ring", "masked"};
-        snprintf(name, sizeof name, "gemm_%s_%dx%d_%s_out_%s", type_tag<TIn>(), BM, BN, loads[MODE], type_tag<TOut>());
-    }
-    if (!attr_done) {
-        int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds),
-                           "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
-        if (rc) return rc;
-        attr_done = true;
-    }
+    auto kern = gemm_kernel<TIn, BM, BN, MODE, TOut, SMAX>;
+    static std::atomic<uint64_t> attr_done{0};  // one per instantiation: the devices whose LDS limit has been raised
+    int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, attr_done);
+    if (rc) return rc;
+    static const char* const loads[] = {"regs", "", "ring", "masked"};
+    char name[96];
+    snprintf(name, sizeof name, "gemm_%s_%dx%d_%s_out_%s%s", type_tag<TIn>(), BM, BN, loads[MODE], type_tag<TOut>(),
+             g.ksplit == 2 ? "_ksplit2" : g.ksplit == 3 ? "_ksplit3" : g.ksplit == 4 ? "_ksplit4" : "");
     note_kernel(name);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, g);
     return check_hip(hipGetLastError(), name);
 }
 
-#define MMX_LAUNCH(TIn, BM, BN, MODE, TOut) \
-    launch_cfg<TIn, BM, BN, MODE, TOut>(g, grid, st)
-#define MMX_LAUNCH_MODES(TIn, BM, BN, TOut) \
-    (mode == 2 ? MMX_LAUNCH(TIn, BM, BN, 2, TOut) : MMX_LAUNCH(TIn, BM, BN, 0, TOut))
+// The K split exists for the ring pipeline (MODE 2) and tiles at least 128 columns wide.
+#define MMX_LAUNCH(TIn, BM, BN, MODE, TOut, SMAX) \
+    launch_cfg<TIn, BM, BN, MODE, TOut, SMAX>(g, grid, st)
+#define MMX_LAUNCH_MODES(TIn, BM, BN, TOut)                                                  \
+    (g.ksplit > 1 ? MMX_LAUNCH(TIn, BM, BN, 2, TOut, KSPLIT_MAX)                              \
+                  : (mode == 2 ? MMX_LAUNCH(TIn, BM, BN, 2, TOut, 1) : MMX_LAUNCH(TIn, BM, BN, 0, TOut, 1)))
 
 template <typename TIn, typename TOut>
 static int launch_tiles(const GemmArgs& g, TileCfg t, int mode, int grid, hipStream_t st) {
-    if (mode == 3) return MMX_LAUNCH(TIn, 128, 128, 3, TOut);  // the masked path exists for one tile shape
+    if (g.ksplit > 1 && mode != 2) return set_error(MMX_E_UNSUPPORTED, "the K split needs the ring pipeline (aligned A, K a multiple of 128 bytes)");
+    if (mode == 3) return MMX_LAUNCH(TIn, 128, 128, 3, TOut, 1);  // the masked path exists for one tile shape
     if (t.bm == 256 && t.bn == 256) return MMX_LAUNCH_MODES(TIn, 256, 256, TOut);
     if (t.bm == 256 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 256, 192, TOut);
     if (t.bm == 128 && t.bn == 256) return MMX_LAUNCH_MODES(TIn, 128, 256, TOut);
     if (t.bm == 128 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 128, 192, TOut);
     if (t.bm == 128 && t.bn == 128) return MMX_LAUNCH_MODES(TIn, 128, 128, TOut);
-    if (t.bm == 128 && t.bn == 64 && mode == 2) return MMX_LAUNCH(TIn, 128, 64, 2, TOut);  // ring pipeline only
+    if (t.bm == 128 && t.bn == 64 && mode == 2 && g.ksplit == 1) return MMX_LAUNCH(TIn, 128, 64, 2, TOut, 1);  // ring pipeline only
     return set_error(MMX_E_UNSUPPORTED, "no MFMA tile kernel for %dx%d", t.bm, t.bn);
 }
 
 // Fills the launch geometry; returns the grid size (or a negative error code).
 static inline int prepare_gemm(GemmArgs& g, TileCfg& t, int& mode, int elesz, const void* A, int64_t lda, const void* Bp,
-                               int M, int K, int N, int n0, int n1, const Epilogue& ep) {
+                               int M, int K, int N, int n0, int n1, const Epilogue& ep, const SplitRequest& rq) {
     g.A = static_cast<const char*>(A);
     g.lda = lda;
     g.Bp = static_cast<const char*>(Bp);
@@ -726,14 +896,28 @@ static inline int prepare_gemm(GemmArgs& g, TileCfg& t, int& mode, int elesz, co
     mode = fast_ok ? load_mode() : 3;
     // mode 2 addresses A through 32-bit per-thread offsets
     if (mode == 2 && ((int64_t)M * lda >= ((int64_t)1 << 32) - 4096 || g.panel_stride >= ((int64_t)1 << 28))) mode = 0;
-    t = choose_tile(M, n1 - n0, pairs);
-    if (mode == 3) t = {128, 128};
-    if (mode != 2 && t.bn == 64) t = {128, 128};  // the 64-wide tile exists for the ring pipeline only
+    SplitRequest use = rq;
+    if (mode != 2 || pairs) {
+        if (rq.k_splits > 1)
+            return set_error(MMX_E_UNSUPPORTED, "a K split needs 16-byte aligned rows of A, K a multiple of 128 bytes and no SILU_GATE");
+        use.k_splits = 1;
+    }
+    if (use.k_splits > KSPLIT_MAX) return set_error(MMX_E_INVALID, "at most %d K slices", KSPLIT_MAX);
+    if (use.k_splits > 1 && !use.ws) return set_error(MMX_E_INVALID, "a K split needs a workspace");
+    const Plan plan = choose_plan(M, n1 - n0, g.nk, pairs, mode, use);
+    if (use.k_splits > 1 && plan.S != use.k_splits)
+        return set_error(MMX_E_INVALID, "%d K slices do not fit: K too short, the workspace too small, or more than %d tiles",
+                         use.k_splits, WS_MAX_TILES);
+    t = plan.t;
     if (pairs && (t.bn % 128) != 0)
         return set_error(MMX_E_INVALID, "SILU_GATE needs a tile width that is a multiple of 128");
+    g.ksplit = plan.S;
+    g.kq = plan.S > 1 ? slice_kiters(g.nk, plan.S) : g.nk;
+    g.ws_cnt = reinterpret_cast<uint32_t*>(use.ws);
+    g.ws_part = use.ws ? use.ws + WS_COUNTER_BYTES : nullptr;
     g.tiles_m = (M + t.bm - 1) / t.bm;
     const int tiles_n = (n1 - n0 + t.bn - 1) / t.bn;
-    g.total_tiles = g.tiles_m * tiles_n;
+    g.total_tiles = g.tiles_m * tiles_n * g.ksplit;
     g.tiles_per_xcd = (g.total_tiles + 7) / 8;
     return g.tiles_per_xcd * 8;
 }

@@ -947,20 +947,15 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
     const int zero_off = (M * K * 2 + 1023) & ~1023;
     const int xbytes = zero_off + K * 2;  // x, a gap up to the next KiB, one row of zeros
     if (kpad == K && s.x_vec_ok && !w8 && !pairs && M >= 2 && M <= 4 && xbytes > 46 * 1024 && xbytes <= 128 * 1024 &&
-        decode_halves() != 0 && panels <= 256 && (int64_t)s.nfrag * 512 >= 128 * 1024) {
+        decode_halves() != 0 && panels <= num_cus() && (int64_t)s.nfrag * 512 >= 128 * 1024) {
         // A few rows of a long x (the MLP's down projection at M = 2-4: 66-110 KiB with the zero row) and at
         // most one half-panel per CU: the half-panel form with one workgroup per CU still has all of x in LDS.
         typedef void (*HalfKernel)(const SkinnyArgs, int);
-        static bool attr_done = false;
-        if (!attr_done) {
-            const HalfKernel kernels[2] = {skinny_half_kernel<false, 1, true, 16>, skinny_half_kernel<false, 1, false, 16>};
-            for (HalfKernel k : kernels) {
-                const int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                             128 * 1024),
-                                         "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
-                if (rc) return rc;
-            }
-            attr_done = true;
+        static std::atomic<uint64_t> attr_done[2];
+        const HalfKernel kernels[2] = {skinny_half_kernel<false, 1, true, 16>, skinny_half_kernel<false, 1, false, 16>};
+        for (int i = 0; i < 2; i++) {
+            const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernels[i]), 128 * 1024, attr_done[i]);
+            if (rc) return rc;
         }
         note_kernel("skinny_half_bf16");
         if (((s.nfrag >> 1) + 3) / 4 <= 16)
@@ -975,17 +970,12 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
     const bool bigx = !pairs && xbytes > 46 * 1024 && xbytes <= 80 * 1024;
     if (bigx) {
         typedef void (*StreamKernel)(const SkinnyArgs, int);
-        static bool attr_done = false;
-        if (!attr_done) {
-            const StreamKernel kernels[4] = {skinny_stream_kernel<0, 1, true>, skinny_stream_kernel<0, 1, false>,
-                                             skinny_stream_kernel<1, 1, true>, skinny_stream_kernel<1, 1, false>};
-            for (StreamKernel k : kernels) {
-                const int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                             80 * 1024),
-                                         "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
-                if (rc) return rc;
-            }
-            attr_done = true;
+        static std::atomic<uint64_t> attr_done[4];
+        const StreamKernel kernels[4] = {skinny_stream_kernel<0, 1, true>, skinny_stream_kernel<0, 1, false>,
+                                         skinny_stream_kernel<1, 1, true>, skinny_stream_kernel<1, 1, false>};
+        for (int i = 0; i < 4; i++) {
+            const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernels[i]), 80 * 1024, attr_done[i]);
+            if (rc) return rc;
         }
     }
     if (kpad == K && (xbytes <= 46 * 1024 || bigx) && s.x_vec_ok && !(pairs && w8)) {
@@ -1002,7 +992,7 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         const int wg_per_cu = (160 * 1024 / lds_wg) < 4 ? (160 * 1024 / lds_wg) : 4;
         const int64_t unit_bytes = (int64_t)s.nfrag * 512 * (pairs ? 2 : 1);
         const int force = decode_halves();  // -1: by the rule above, 0: never, 1: for every M <= 4 (tests pin the path with it)
-        const bool halves = M <= 4 && !bigx && force != 0 && (force == 1 || (2 * units <= 2 * 256 * wg_per_cu && unit_bytes >= 128 * 1024));
+        const bool halves = M <= 4 && !bigx && force != 0 && (force == 1 || (2 * units <= 2 * num_cus() * wg_per_cu && unit_bytes >= 128 * 1024));
         const int per_wave_h = ((s.nfrag >> 1) + 3) / 4;
 #define MMX_STREAM(W8, NP, GRID)                                                                                     \
     do {                                                                                                             \

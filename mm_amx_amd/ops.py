@@ -194,6 +194,10 @@ class MLP:
         self.down = L.repack_b(w_down, transpose=True)
 
     def run(self, x, y=None):
+        if self.gate_up is None:
+            raise L.MmxError("run: setup has not been called")
+        if x.dim() != 2 or x.shape[1] != self.m_K:
+            raise L.MmxError(f"run: x must be [M, {self.m_K}]")
         M = x.shape[0]
         if self.actUp is None or self.actUp.shape[0] < M:  # setM (tests/amx-mlp.cpp:771-776)
             self.actUp = torch.empty((M, self.m_N), dtype=torch.bfloat16, device=x.device)

@@ -64,3 +64,147 @@ def test_package_fails_loudly_without_the_library(monkeypatch):
     monkeypatch.setattr(L, "_LIB_PATH", "/nonexistent/libmm_amx_amd.so")
     with pytest.raises(L.MmxError, match="no CPU or PyTorch fallback"):
         L.lib()
+
+
+# ---- the Python binding checks shapes and dtypes on the host, before any pointer crosses the boundary ----------
+def _cpu_case():
+    import torch
+    import mm_amx_amd._lib as L
+    A = torch.zeros((64, 128), dtype=torch.bfloat16)
+    packed = torch.zeros(L._packed_bytes_host(L.BF16, 128, 96), dtype=torch.uint8)
+    C_out = torch.zeros((64, 96), dtype=torch.float32)
+    return torch, L, A, packed, C_out
+
+
+def test_host_restatement_of_the_packed_size(lib):
+    import mm_amx_amd._lib as L
+    lib.mmx_packed_b_bytes.restype = C.c_size_t
+    for dt in (L.BF16, L.I8, L.I4):
+        for K, N in ((64, 32), (65, 33), (4096, 11008), (300, 45), (1, 1)):
+            assert L._packed_bytes_host(dt, K, N) == lib.mmx_packed_b_bytes(dt, K, N)
+
+
+def test_gemm_rejects_wrong_sizes_before_any_launch():
+    torch, L, A, packed, C_out = _cpu_case()
+
+    class Ep:  # the fields gemm() reads, without the GPU-residency check of L.Epilogue
+        def __init__(self, Cx, steps=0, bias=None, deq=None, q=None):
+            self.C, self.steps, self.bias, self.deq_oc, self.q_oc = Cx, steps, bias, deq, q
+
+    with pytest.raises(L.MmxError, match="C is"):
+        L.gemm(A, packed, 96, Ep(C_out[:32]))            # too few rows
+    with pytest.raises(L.MmxError, match="C is"):
+        L.gemm(A, packed, 96, Ep(C_out[:, :64]))         # too few columns
+    with pytest.raises(L.MmxError, match="Bpacked holds"):
+        L.gemm(A, packed[:-1], 96, Ep(C_out))
+    with pytest.raises(L.MmxError, match="uint8"):
+        L.gemm(A, packed.view(torch.int8), 96, Ep(C_out))
+    with pytest.raises(L.MmxError, match="bias holds"):
+        L.gemm(A, packed, 96, Ep(C_out, L.PP_BIAS, bias=torch.zeros(95)))
+    with pytest.raises(L.MmxError, match="deq_scale_per_oc holds"):
+        L.gemm(A, packed, 96, Ep(C_out, L.PP_DEQUANT, deq=torch.zeros(10)))
+    with pytest.raises(L.MmxError, match="column range"):
+        L.gemm(A, packed, 96, Ep(C_out), n0=0, n1=128)
+    with pytest.raises(L.MmxError, match="2-D"):
+        L.gemm(A[0], packed, 96, Ep(C_out))
+    with pytest.raises(L.MmxError, match="not part of this path"):
+        L.gemm(A.to(torch.float16), packed, 96, Ep(C_out))
+    # SILU_GATE halves the columns of C
+    with pytest.raises(L.MmxError, match="C is"):
+        L.gemm(A, torch.zeros(L._packed_bytes_host(L.BF16, 128, 128), dtype=torch.uint8), 128, Ep(C_out[:, :63], L.PP_SILU_GATE))
+    # everything in order: the call gets as far as asking for GPU tensors, and no further
+    with pytest.raises(L.MmxError, match="on the GPU"):
+        L.gemm(A, packed, 96, Ep(C_out))
+
+
+def test_matvec_and_mlp_reject_wrong_sizes_before_any_launch():
+    torch, L, A, packed, C_out = _cpu_case()
+    with pytest.raises(L.MmxError, match="b must be"):
+        L.matvec(A, torch.zeros(127, dtype=torch.bfloat16))
+    with pytest.raises(L.MmxError, match="b must be"):
+        L.matvec(A, torch.zeros(128, dtype=torch.float32))
+    with pytest.raises(L.MmxError, match="b must be"):
+        L.matvec(A, torch.zeros(256, dtype=torch.bfloat16)[::2])
+    with pytest.raises(L.MmxError, match="out must be"):
+        L.matvec(A, torch.zeros(128, dtype=torch.bfloat16), torch.zeros(63, dtype=torch.float32))
+    with pytest.raises(L.MmxError, match="out must be"):
+        L.matvec(A, torch.zeros(128, dtype=torch.bfloat16), torch.zeros(64, dtype=torch.int32))
+    with pytest.raises(L.MmxError, match="on the GPU"):
+        L.matvec(A, torch.zeros(128, dtype=torch.bfloat16))
+    K, N = 128, 96
+    gu = torch.zeros(L._packed_bytes_host(L.BF16, K, 2 * N), dtype=torch.uint8)
+    dn = torch.zeros(L._packed_bytes_host(L.BF16, N, K), dtype=torch.uint8)
+    with pytest.raises(L.MmxError, match="x must be bf16"):
+        L.mlp(A.float(), gu, dn, N)
+    with pytest.raises(L.MmxError, match="w_gate_up"):
+        L.mlp(A, gu[:-1], dn, N)
+    with pytest.raises(L.MmxError, match="w_down"):
+        L.mlp(A, gu, dn[:100], N)
+    with pytest.raises(L.MmxError, match="h must be"):
+        L.mlp(A, gu, dn, N, h=torch.zeros((64, N - 1), dtype=torch.bfloat16))
+    with pytest.raises(L.MmxError, match="y must be"):
+        L.mlp(A, gu, dn, N, y=torch.zeros((64, K), dtype=torch.float32))
+    with pytest.raises(L.MmxError, match="multiple of 32"):
+        L.mlp(A, gu, dn, 90)
+    with pytest.raises(L.MmxError, match="on the GPU"):
+        L.mlp(A, gu, dn, N)
+    from mm_amx_amd import ops
+    m = ops.MLP()
+    with pytest.raises(L.MmxError, match="setup has not"):
+        m.run(A)
+    m.m_K, m.m_N, m.gate_up, m.down = K, N, gu, dn
+    with pytest.raises(L.MmxError, match=r"x must be \[M, 128\]"):
+        m.run(torch.zeros((4, 64), dtype=torch.bfloat16))
+
+
+def test_abi_rejects_overlapping_rows_of_c_and_misaligned_operands(lib):
+    lib.mmx_last_error.restype = C.c_char_p
+
+    class Ep(C.Structure):
+        _fields_ = [("steps", C.c_uint32), ("out_dtype", C.c_int32), ("C", C.c_void_p), ("ldc_bytes", C.c_int64),
+                    ("bias", C.c_void_p), ("deq_scale", C.c_float), ("deq_scale_per_oc", C.c_void_p),
+                    ("q_scale", C.c_float), ("q_scale_per_oc", C.c_void_p)]
+    gemm = lib.mmx_gemm
+    gemm.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+                     C.POINTER(Ep), C.c_void_p]
+    fake = 0x10000  # never dereferenced: validation fails first
+    ep = Ep(0, 0, fake, 4 * 63, None, 1.0, None, 0.0, None)   # fp32 rows of 63 < 64 columns
+    assert gemm(1, 1, fake, 256, fake, 64, 128, 64, 0, 64, C.byref(ep), None) == -1
+    assert b"ldc_bytes" in lib.mmx_last_error()
+    ep = Ep(0, 0, fake, -256, None, 1.0, None, 0.0, None)
+    assert gemm(1, 1, fake, 256, fake, 64, 128, 64, 0, 64, C.byref(ep), None) == -1
+    mv = lib.mmx_matvec
+    mv.argtypes = [C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
+    assert mv(1, fake + 1, 256, fake, fake, 4, 128, None) == -1 and b"aligned" in lib.mmx_last_error()
+    assert mv(1, fake, 255, fake, fake, 4, 100, None) == -1
+    qw = lib.mmx_quantize_weights
+    qw.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
+    assert qw(fake + 1, 256, 4, 128, fake, 128, fake, fake, None) == -1 and b"aligned" in lib.mmx_last_error()
+    # K split requests that can be refused without a device
+    sk = lib.mmx_gemm_splitk
+    sk.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+                   C.POINTER(Ep), C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]
+    ep = Ep(0, 0, fake, 4 * 64, None, 1.0, None, 0.0, None)
+    assert sk(1, 1, fake, 256, fake, 64, 128, 64, 0, 64, C.byref(ep), 2, None, 0, None) == -1 and b"workspace" in lib.mmx_last_error()
+    assert sk(1, 1, fake, 256, fake, 64, 128, 64, 0, 64, C.byref(ep), -1, fake, 1 << 20, None) == -1
+    assert sk(1, 1, fake, 256, fake, 64, 128, 64, 0, 64, C.byref(ep), 2, fake + 16, 1 << 20, None) == -1 and b"256-byte" in lib.mmx_last_error()
+    assert sk(1, 1, fake, 256, fake, 8, 128, 64, 0, 64, C.byref(ep), 2, fake, 1 << 20, None) == -2 and b"decode" in lib.mmx_last_error()
+
+
+def test_tuning_knobs_are_per_thread(lib):
+    """mmx_set_tile / mmx_set_option change the calling thread's dispatch only; a first call from two threads at once
+    must not race on anything."""
+    import threading
+    lib.mmx_last_error.restype = C.c_char_p
+    seen = {}
+
+    def worker(name, shape, ok):
+        rc = lib.mmx_set_tile(shape)
+        err = lib.mmx_last_error()
+        seen[name] = (rc, err)
+
+    t1 = threading.Thread(target=worker, args=("good", b"256x192", True))
+    t2 = threading.Thread(target=worker, args=("bad", b"17x3", False))
+    t1.start(), t2.start(), t1.join(), t2.join()
+    assert seen["good"][0] == 0 and seen["bad"][0] == -1 and b"17x3" in seen["bad"][1]
+    assert b"17x3" not in lib.mmx_last_error()  # this thread's error string is its own

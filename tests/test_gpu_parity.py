@@ -122,7 +122,7 @@ def test_bf16_256_cube(po):
     assert err < 1e-5
 
 
-@pytest.mark.parametrize("M", [128, 1024])
+@pytest.mark.parametrize("M", [128, 512, 1024, 2048])
 def test_ffn_up_bias_gelu_full_size(po, M):
     """The headline FC at its real shape: K=4096, N=11008, BIAS_GELU -> bf16."""
     w = wl.ffn_up_bias_gelu(M=M)
@@ -446,6 +446,7 @@ def _mlp_case(po, M, K, N, seed):
     m = mx.MLP()
     m.setup(dev_bf16(w["w_gate"]), dev_bf16(w["w_up"]), dev_bf16(w["w_down"]))
     y = m.run(dev_bf16(w["x"]))
+    k_down = mx.last_kernel()
     h = host_bits(m.actUp[:M])
     # stage 1: h from the same x
     e1, f1 = check_float_parity(bf16_to_f32(h), bf16_to_f32(h_ref), f"mlp h M={M}")
@@ -480,8 +481,10 @@ def _mlp_case(po, M, K, N, seed):
     _, y_e2e = po.mlp(w["x"], w["w_gate"], w["w_up"], w["w_down"], split_k=True)
     yf, rf = bf16_to_f32(host_bits(y)).astype(np.float64), bf16_to_f32(y_e2e).astype(np.float64)
     e3 = np.linalg.norm(yf - rf) / np.linalg.norm(rf)
-    print(f"mlp M={M}: h rel={e1:.2e} ({f1 * 100:.3f}% <=1ulp)  y|h rel={e2:.2e} ({f2 * 100:.3f}%)  end-to-end rel={e3:.2e}")
+    print(f"mlp M={M}: h rel={e1:.2e} ({f1 * 100:.3f}% <=1ulp)  y|h rel={e2:.2e} ({f2 * 100:.3f}%)  end-to-end rel={e3:.2e}  "
+          f"kernels={k_fused}, {k_down}")
     assert e3 < 3e-3
+    return k_fused, k_down
 
 
 @pytest.mark.parametrize("M", [32, 64])
@@ -518,9 +521,12 @@ def test_mlp_small(po, M):
     _mlp_case(po, M, 512, 768, seed=20 + M)
 
 
-@pytest.mark.parametrize("M", [1, 256])
+@pytest.mark.parametrize("M", [1, 256, 2048])
 def test_mlp_llama7b_shape(po, M):
-    _mlp_case(po, M, 4096, 11008, seed=30 + M)
+    """AMX_MLP's own test shape (tests/amx-mlp.cpp:845-849, M=256) and the two benchmark points M=1 and M=2048."""
+    kernels = _mlp_case(po, M, 4096, 11008, seed=30 + M)
+    if M == 2048:  # the tile kernels the benchmark times at this M
+        assert "256x256" in kernels[0] and "128x256" in kernels[1], kernels
 
 
 # ---- torch-ext call shape -------------------------------------------------------------------------------
@@ -865,3 +871,143 @@ def test_int8_decode_form(po, shape):
     mx.gemm(odd[:, :K], packed, N, mx.Epilogue(C2, mx.PP_NONE))
     assert "skinny" not in mx.last_kernel() or M == 1
     assert np.array_equal(host_bits(C2), acc_ref)
+
+
+# ---- K split over several workgroups per tile (the split-K of AMX_MLP::Linear, tests/amx-mlp.cpp:560-593, 648-704) ----
+@pytest.fixture()
+def ws():
+    w = torch.zeros((64 << 20) + (16 << 10), dtype=torch.uint8, device="cuda")
+    yield w
+    torch.cuda.synchronize()
+    assert not w[:16 << 10].any().item(), "the arrival counters must be left at zero"
+
+
+@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x192", "128x128"])
+@pytest.mark.parametrize("S", [2, 3, 4])
+def test_ksplit_int8_bit_exact(po, ws, tile, S):
+    """int32 partial sums add exactly in any order: raw sums and requantised outputs equal the oracle's bits."""
+    M, K, N = 520, 4096 - 512 * (S == 3), 704   # 8 blocks of 512 bytes of K per row (7 for three slices: 3 + 3 + 1)
+    rng = np.random.default_rng(130 + S)
+    A = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    deq = (np.float32(0.02) * rng.uniform(1e-3, 1e-2, N).astype(np.float32)).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    steps = po.PP_DEQUANT | po.PP_BIAS | po.PP_QUANT
+    acc_ref = po.gemm_i8(A, B)
+    ref = po.pp(acc_ref, steps, po.I8, bias=bias, deq_per_oc=deq, q=20.0)
+    Ad, packed = dev(A), mx.repack_b(dev(B))
+    mx.set_tile(tile)
+    try:
+        for rep in range(2):  # twice: the second launch finds the counters as the first one left them
+            acc = torch.full((M, N), -3, dtype=torch.int32, device="cuda")
+            mx.gemm(Ad, packed, N, mx.Epilogue(acc, mx.PP_NONE), k_splits=S, ws=ws)
+            assert tile in mx.last_kernel() and f"ksplit{S}" in mx.last_kernel(), mx.last_kernel()
+            assert np.array_equal(host_bits(acc), acc_ref)
+            out = torch.zeros((M, N), dtype=torch.int8, device="cuda")
+            mx.gemm(Ad, packed, N, mx.Epilogue(out, steps, bias=dev(bias), deq_scale_per_oc=dev(deq), q_scale=20.0),
+                    k_splits=S, ws=ws)
+            assert np.array_equal(host_bits(out), ref)
+    finally:
+        mx.set_tile("")
+
+
+@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x192", "128x128"])
+@pytest.mark.parametrize("S", [2, 3, 4])
+def test_ksplit_bf16_fixed_order(po, ws, tile, S):
+    """fp32 partial sums are added in slice order whatever slice arrives last: repeated launches give the same
+    bits, the fused post-op equals the oracle's on those accumulators, and the accumulators are the oracle's
+    slice sums added in that order, within the bar of the unsplit kernel."""
+    M, K, N = 600, 2048, 832
+    rng = np.random.default_rng(140 + S)
+    A, B = rand_bf16(rng, (M, K), 1.0), rand_bf16(rng, (K, N), 0.05)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    # the slices are whole blocks of 256 of K: ceil(blocks / S) blocks each
+    blocks = K // 256
+    q = -(-blocks // S) * 256
+    acc_ref = None
+    for s0 in range(0, K, q):
+        part = po.gemm_bf16(np.ascontiguousarray(A[:, s0:s0 + q]), np.ascontiguousarray(B[s0:s0 + q]))
+        acc_ref = part if acc_ref is None else (acc_ref + part).astype(np.float32)
+    Ad, packed = dev_bf16(A), mx.repack_b(dev_bf16(B))
+    mx.set_tile(tile)
+    try:
+        accs = []
+        for rep in range(3):
+            acc = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+            mx.gemm(Ad, packed, N, mx.Epilogue(acc, mx.PP_NONE), k_splits=S, ws=ws)
+            assert tile in mx.last_kernel() and f"ksplit{S}" in mx.last_kernel(), mx.last_kernel()
+            accs.append(host_bits(acc))
+        assert np.array_equal(accs[0], accs[1]) and np.array_equal(accs[0], accs[2])
+        check_float_parity(accs[0], acc_ref, f"ksplit{S} accumulators {tile}")
+        C = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+        mx.gemm(Ad, packed, N, mx.Epilogue(C, mx.PP_BIAS | mx.PP_GELU, bias=dev(bias)), k_splits=S, ws=ws)
+        assert np.array_equal(host_bits(C), po.pp(accs[0], po.PP_BIAS | po.PP_GELU, po.BF16, bias=bias))
+    finally:
+        mx.set_tile("")
+
+
+def test_ksplit_two_way_is_the_reference_partition(po, ws):
+    """Linear::run with do_splitK (tests/amx-mlp.cpp:648-682): y = bf16(p0 + p1), p0 over the first
+    ceil(blocks/2) K blocks of 256, p1 over the rest.  K = 11008 = 43 blocks -> 22 + 21."""
+    M, K, N = 96, 11008, 256
+    rng = np.random.default_rng(150)
+    h, Wd = rand_bf16(rng, (M, K), 0.3), rand_bf16(rng, (N, K), 0.02)   # w_down in torch layout [out, in]
+    ref = po.mlp_down(h, Wd, split_k=True)
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    mx.gemm(dev_bf16(h), mx.repack_b(dev_bf16(Wd), transpose=True), N, mx.Epilogue(y, mx.PP_NONE), k_splits=2, ws=ws)
+    assert "ksplit2" in mx.last_kernel()
+    check_float_parity(bf16_to_f32(host_bits(y)), bf16_to_f32(ref), "two-way split-K down projection")
+
+
+def test_ksplit_full_size_configs(po, ws):
+    """The shapes the split is there for, at full size, with the library's own choice of slices."""
+    w = wl.int8_fc()
+    steps = po.PP_DEQUANT | po.PP_BIAS | po.PP_QUANT
+    acc_ref = po.gemm_i8(w["A"], w["B"])
+    out_ref = po.pp(acc_ref, steps, po.I8, bias=w["bias"], deq_per_oc=w["deq"], q=float(w["q"]))
+    Ad, packed = dev(w["A"]), mx.repack_b(dev(w["B"]))
+    acc = torch.zeros((w["M"], w["N"]), dtype=torch.int32, device="cuda")
+    mx.gemm(Ad, packed, w["N"], mx.Epilogue(acc, mx.PP_NONE), ws=ws)
+    k_acc = mx.last_kernel()
+    out = torch.zeros((w["M"], w["N"]), dtype=torch.int8, device="cuda")
+    mx.gemm(Ad, packed, w["N"], mx.Epilogue(out, steps, bias=dev(w["bias"]), deq_scale_per_oc=dev(w["deq"]), q_scale=float(w["q"])), ws=ws)
+    print(f"int8 fc 512x4096x4096: {k_acc} / {mx.last_kernel()}")
+    assert np.array_equal(host_bits(acc), acc_ref) and np.array_equal(host_bits(out), out_ref)
+
+
+def test_ksplit_requests_that_cannot_be_met(ws):
+    A = torch.zeros((64, 1024), dtype=torch.bfloat16, device="cuda")
+    packed = mx.repack_b(torch.zeros((1024, 256), dtype=torch.bfloat16, device="cuda"))
+    C = torch.zeros((64, 256), dtype=torch.float32, device="cuda")
+    with pytest.raises(mx.MmxError, match="at most 4"):
+        mx.gemm(A, packed, 256, mx.Epilogue(C), k_splits=5, ws=ws)
+    with pytest.raises(mx.MmxError, match="do not fit"):
+        mx.gemm(A, packed, 256, mx.Epilogue(C), k_splits=2, ws=ws[:32 << 10])
+    with pytest.raises(mx.MmxError, match="decode kernels"):
+        mx.gemm(A[:8], packed, 256, mx.Epilogue(C), k_splits=2, ws=ws)
+    with pytest.raises(mx.MmxError, match="K split needs"):
+        mx.gemm(A[:, :1000], mx.repack_b(torch.zeros((1000, 256), dtype=torch.bfloat16, device="cuda")), 256, mx.Epilogue(C), k_splits=2, ws=ws)
+    gu = mx.repack_gate_up(torch.zeros((128, 1024), dtype=torch.bfloat16, device="cuda"), torch.zeros((128, 1024), dtype=torch.bfloat16, device="cuda"))
+    h = torch.zeros((64, 128), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(mx.MmxError, match="K split needs"):
+        mx.gemm(A, gu, 256, mx.Epilogue(h, mx.PP_SILU_GATE), k_splits=2, ws=ws)
+    assert mx.gemm_workspace_bytes(mx.BF16, mx.BF16, 64, 1024, 256, k_splits=2) > 16 << 10
+    assert mx.gemm_workspace_bytes(mx.BF16, mx.BF16, 64, 1024, 256, k_splits=1) == 0
+
+
+@pytest.mark.parametrize("M", [64, 300])
+def test_mlp_down_projection_split(po, ws, M):
+    """mmx_mlp_splitk with the reference's two-way split of the down projection: same h, y within the bar of the
+    oracle's split form, and the same bits on every run."""
+    K, N = 512, 2816
+    w = wl.llama_mlp(M=M, K=K, N=N, seed=160 + M)
+    gu = mx.repack_gate_up(dev_bf16(w["w_gate"]), dev_bf16(w["w_up"]))
+    dn = mx.repack_b(dev_bf16(w["w_down"]), transpose=True)
+    ys = []
+    for rep in range(2):
+        h, y = mx.mlp(dev_bf16(w["x"]), gu, dn, N, down_k_splits=2, ws=ws)
+        assert "ksplit2" in mx.last_kernel(), mx.last_kernel()
+        ys.append(host_bits(y))
+    assert np.array_equal(ys[0], ys[1])
+    y_ref = po.mlp_down(host_bits(h), w["w_down"], split_k=True)
+    check_float_parity(bf16_to_f32(ys[0]), bf16_to_f32(y_ref), f"mlp down split M={M}")
