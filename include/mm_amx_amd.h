@@ -156,6 +156,18 @@ int mmx_gemm_splitk(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, 
 size_t mmx_gemm_workspace_bytes(int a_dtype, int b_dtype, int M, int K, int N, int n0, int n1, uint32_t steps,
                                 int k_splits);
 
+/* mmx_gemm_splitk for callers that cannot allocate device memory (code under HIP graph capture, serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  The workspace is a 64 MiB + 16 KiB array
+ * built into the library, one copy per GPU, held until the process ends; the call allocates and frees nothing.
+ * Same arguments, results and errors as mmx_gemm_splitk with a workspace of that size (so k_splits = 0 always
+ * fits; an explicit k_splits whose partial tiles need more returns MMX_E_INVALID and says how much).  mmx_init()
+ * must have been called for the current device.  The array is shared by every call on that GPU and keeps the last
+ * call's partial sums; its arrival counters are zero when the library is loaded and every completed call leaves
+ * them zero.  Calls that overlap in time on one GPU (two streams, two threads) race on it: use mmx_gemm_splitk
+ * with a workspace per stream there. */
+int mmx_gemm_splitk_static(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* Bpacked, int M,
+                           int K, int N, int n0, int n1, const mmx_epilogue* ep, int k_splits, void* stream);
+
 /* ---- c[M] = A[M, K] · b[K]: amx_kernel::MatmulVector::operator() (include/kernels_amx.hpp:959)
  * and amx_kernel::GemAvB::operator() (:1534).  dtype MMX_BF16 (c fp32) or MMX_I8 (c int32). */
 int mmx_matvec(int dtype, const void* A, int64_t lda_bytes, const void* b, void* c, int M, int K, void* stream);

@@ -17,7 +17,7 @@ _LIB_PATH = os.environ.get("MMX_LIB_PATH") or os.path.join(_HERE, "libmm_amx_amd
 
 EXPORTS = ["mmx_last_error", "mmx_init", "mmx_packed_b_bytes", "mmx_repack_b", "mmx_repack_gate_up",
            "mmx_quantize_weights", "mmx_quantize_pack_int4", "mmx_dequant_packed", "mmx_gemm", "mmx_gemm_splitk",
-           "mmx_gemm_workspace_bytes", "mmx_matvec", "mmx_mlp", "mmx_mlp_splitk", "mmx_set_tile",
+           "mmx_gemm_splitk_static", "mmx_gemm_workspace_bytes", "mmx_matvec", "mmx_mlp", "mmx_mlp_splitk", "mmx_set_tile",
            "mmx_set_option", "mmx_last_kernel", "mmx_time_gemm", "mmx_probe_mfma"]
 
 # a workspace of this size serves every shape when the library chooses the K split itself (include/mm_amx_amd.h)
@@ -66,6 +66,8 @@ def lib():
                                C.c_int, C.POINTER(_Epilogue), C.c_void_p]
         l.mmx_gemm_splitk.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
                                       C.c_int, C.POINTER(_Epilogue), C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]
+        l.mmx_gemm_splitk_static.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_int, C.c_int, C.c_int,
+                                             C.c_int, C.c_int, C.POINTER(_Epilogue), C.c_int, C.c_void_p]
         l.mmx_gemm_workspace_bytes.restype = C.c_size_t
         l.mmx_gemm_workspace_bytes.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_uint32, C.c_int]
         l.mmx_mlp_splitk.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p,
@@ -293,6 +295,17 @@ def gemm(A, Bpacked, N, ep, b_dtype=None, n0=0, n1=None, k_splits=0, ws=None):
     ks, wsp, wsb = _split_args(A, k_splits, ws)
     _check(lib().mmx_gemm_splitk(a_dt, b_dt, A.data_ptr(), _row_stride_bytes(A), Bpacked.data_ptr(), M, K, N, n0, n1,
                                  C.byref(s), ks, wsp, wsb, _stream()))
+
+
+def gemm_static(A, Bpacked, N, ep, b_dtype=None, n0=0, n1=None, k_splits=0):
+    """gemm() on the workspace built into the library (mmx_gemm_splitk_static): allocates nothing."""
+    n1 = N if n1 is None else n1
+    b_dt = (dtype_code(A) if isinstance(A, torch.Tensor) else None) if b_dtype is None else b_dtype
+    M, K, a_dt = _check_gemm_args(A, Bpacked, N, ep, b_dt, n0, n1)
+    _dev(A, "A"), _dev(Bpacked, "Bpacked")
+    s = ep.struct()
+    _check(lib().mmx_gemm_splitk_static(a_dt, b_dt, A.data_ptr(), _row_stride_bytes(A), Bpacked.data_ptr(), M, K, N, n0, n1,
+                                        C.byref(s), k_splits, _stream()))
 
 
 def gemm_workspace_bytes(a_dtype, b_dtype, M, K, N, steps=PP_NONE, k_splits=0, n0=0, n1=None):

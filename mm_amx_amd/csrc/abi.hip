@@ -14,6 +14,15 @@ static thread_local char g_kernel[128] = "";
 static std::atomic<int> g_cus{0};
 static std::mutex g_attr_mutex;
 
+// The K-split workspace of callers that cannot allocate (mmx_gemm_splitk_static): arrival counters and partial
+// tiles as in a caller's workspace, held by every GPU the library runs on until the process ends.  All zero when
+// the code object is loaded; every completed call leaves the counters zero.  `static_ws` is the host-side stand-in
+// of the array: its device address is taken once per device in mmx_init and only that address is ever used.
+constexpr size_t STATIC_WS_BYTES = ((size_t)64 << 20) + ((size_t)16 << 10);
+static __device__ __align__(256) unsigned char static_ws[STATIC_WS_BYTES];
+constexpr int MAX_DEVICES = 64;
+static std::atomic<char*> g_static_ws[MAX_DEVICES];
+
 int set_error(int code, const char* fmt, ...) {
     va_list ap;
     va_start(ap, fmt);
@@ -187,6 +196,12 @@ int mmx_init(int device) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return set_error(MMX_E_DEVICE, "mmx_init: device %d is %s, this library holds gfx950 code only", device, prop.gcnArchName);
     g_cus = prop.multiProcessorCount;
+    if (device < MAX_DEVICES && !g_static_ws[device].load(std::memory_order_acquire)) {
+        void* p = nullptr;  // this device's copy of the array (each GPU has its own, at its own address)
+        rc = check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(static_ws)), "hipGetSymbolAddress(static workspace)");
+        if (rc) return rc;
+        g_static_ws[device].store(static_cast<char*>(p), std::memory_order_release);
+    }
     return MMX_OK;
 }
 
@@ -260,6 +275,23 @@ int mmx_gemm_splitk(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, 
                     int n1, const mmx_epilogue* ep, int k_splits, void* workspace, size_t workspace_bytes, void* stream) {
     if (!workspace && k_splits > 1) return set_error(MMX_E_INVALID, "mmx_gemm_splitk: %d K slices need a workspace", k_splits);
     const SplitRequest rq = {workspace ? k_splits : 1, static_cast<char*>(workspace), workspace_bytes};
+    return gemm_dispatch(a_dtype, b_dtype, A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, rq, static_cast<hipStream_t>(stream));
+}
+
+int mmx_gemm_splitk_static(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* Bpacked, int M, int K, int N,
+                           int n0, int n1, const mmx_epilogue* ep, int k_splits, void* stream) {
+    int dev = 0;
+    int rc = check_hip(hipGetDevice(&dev), "hipGetDevice");
+    if (rc) return rc;
+    char* ws = dev < MAX_DEVICES ? g_static_ws[dev].load(std::memory_order_acquire) : nullptr;
+    if (!ws) return set_error(MMX_E_INVALID, "mmx_gemm_splitk_static: call mmx_init(%d) first (it takes the address of this device's workspace)", dev);
+    if (k_splits > 1 && M > 32) {
+        const size_t need = mmx_gemm_workspace_bytes(a_dtype, b_dtype, M, K, N, n0, n1, ep ? ep->steps : 0, k_splits);
+        if (need > STATIC_WS_BYTES)
+            return set_error(MMX_E_INVALID, "mmx_gemm_splitk_static: %d K slices of this shape need %zu bytes of workspace, the built-in one holds %zu",
+                             k_splits, need, STATIC_WS_BYTES);
+    }
+    const SplitRequest rq = {k_splits, ws, STATIC_WS_BYTES};
     return gemm_dispatch(a_dtype, b_dtype, A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, rq, static_cast<hipStream_t>(stream));
 }
 
