@@ -118,14 +118,15 @@ int mmx_quantize_weights(const void* W, int64_t ldw_bytes, int rows, int cols, v
 int mmx_quantize_pack_int4(const void* W, int64_t ldw_bytes, int K, int N, int transpose, void* packed,
                            float* deq_scales_out, void* stream);
 
-/* int8 packed weights -> bf16 packed weights (exact), the on-the-fly dequant of
- * include/kernels_amx.hpp:490-506 done once for the large-M weight-compressed path. */
+/* int8 packed weights -> bf16 packed weights (exact): the conversion of include/kernels_amx.hpp:490-506 as a
+ * one-off, for callers that want a bf16 copy of compressed weights (mmx_gemm itself converts on the fly). */
 int mmx_dequant_packed(const void* packed_i8, int K, int N, void* packed_bf16, void* stream);
 
 /* ---- C[:, n0:n1] = PP( A · B[:, n0:n1] ): amx_kernel::Matmul<TA,TB,TC>::operator()
  * (include/kernels_amx.hpp:1169-1314; int8-weight specialisation :1319-1516) -----------------
- * a_dtype/b_dtype: (BF16,BF16), (I8,I8), or (BF16,I8) = bf16 activations on int8-compressed
- * weights, dequantised in registers (M <= 32 only; larger M goes through mmx_dequant_packed).
+ * a_dtype/b_dtype: (BF16,BF16), (I8,I8), (BF16,I8) = bf16 activations on int8-compressed weights, converted to
+ * bf16 in registers on their way to the MFMA (exact; any M: :1381-1441 for small M, :1447-1497 for large M;
+ * tiles of 128 or 256 columns), or (BF16,I4) = int4-compressed weights (M <= 32 only).
  * A is [M, K] row-major with row stride lda_bytes; Bpacked comes from mmx_repack_b for the
  * FULL [K, N]; n0 % 32 == 0, 0 <= n0 < n1 <= N.  M <= 32 takes the bandwidth-bound decode
  * kernel (the M<=16 paths of the reference and weight_compression/fc16m.cpp:451-502), larger

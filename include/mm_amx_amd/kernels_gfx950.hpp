@@ -16,7 +16,9 @@
 
 #include <cstdint>
 #include <cstring>
+#include <map>
 #include <memory>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 #include <type_traits>
@@ -280,6 +282,32 @@ inline PackedB<T> repackB_1x2(const tensor2D<T>& Bi, bool transpose = false, hip
     return p;
 }
 
+// ---- workspace of the K split -------------------------------------------------------------------------
+// AMX_MLP::Linear keeps the partial results of its two K halves in per-thread buffers (work.C,
+// tests/amx-mlp.cpp:648-682); here the partial tiles of mmx_gemm_splitk live in one zero-initialised device
+// buffer per (device, stream): calls on one stream are ordered, so they can share it, calls on different
+// streams must not.  64 MiB + 16 KiB serves every shape when the library chooses the number of slices.
+struct Workspace {
+    void* data = nullptr;
+    size_t bytes = 0;
+};
+inline Workspace workspace_for(hipStream_t stream) {
+    static std::mutex mu;
+    static std::map<std::pair<int, hipStream_t>, std::shared_ptr<void>> all;
+    constexpr size_t kBytes = (size_t(64) << 20) + (size_t(16) << 10);
+    int dev = 0;
+    check_hip(hipGetDevice(&dev), "workspace_for: hipGetDevice");
+    std::lock_guard<std::mutex> lock(mu);
+    std::shared_ptr<void>& slot = all[std::make_pair(dev, stream)];
+    if (!slot) {
+        void* p = nullptr;
+        check_hip(hipMalloc(&p, kBytes), "workspace_for: hipMalloc");
+        check_hip(hipMemset(p, 0, kBytes), "workspace_for: hipMemset");  // the arrival counters start at zero
+        slot = std::shared_ptr<void>(p, [](void* q) { (void)hipFree(q); });
+    }
+    return Workspace{slot.get(), kBytes};
+}
+
 // ---- Matmul<TA,TB,TC> (include/kernels_amx.hpp:1045-1315) ---------------------------------------
 // C = PP(A · B[:, n0:n1]).  With constB the packed weights are made at the first call and kept
 // (1188-1192); otherwise B is repacked on every call.  One object is used by one thread at a time,
@@ -289,6 +317,9 @@ struct Matmul {
     PackedB<TB> internalB;
     bool constB;
     bool transposeB;
+    // K slices per output tile, the split-K of AMX_MLP::Linear (tests/amx-mlp.cpp:560-593, 648-682):
+    // 0 = the library chooses, 1 = never, 2 = the reference's two halves, up to 4
+    int k_splits = 0;
 
     static_assert(std::is_same<TA, TB>::value, "Matmul<TA,TB>: TA == TB except for the <bfloat16,int8_t,float> form");
     constexpr static bool is_i8_mode = std::is_same<TA, int8_t>::value;
@@ -310,20 +341,21 @@ struct Matmul {
         require(ppkernel.out_rows() >= M && ppkernel.out_cols() >= n1, "Matmul: C is smaller than M x n1");
         if (!constB || !internalB) internalB = repackB_1x2(matB, transposeB, stream);
         const mmx_epilogue e = ppkernel.descriptor();
-        check(mmx_gemm(dtype_of<TA>::value, dtype_of<TB>::value, matA.data, matA.stride, internalB.data, M, K, N, n0, n1, &e,
-                       stream),
+        const Workspace ws = (k_splits == 1 || M <= 32) ? Workspace() : workspace_for(stream);
+        check(mmx_gemm_splitk(dtype_of<TA>::value, dtype_of<TB>::value, matA.data, matA.stride, internalB.data, M, K, N, n0, n1,
+                              &e, ws.data ? k_splits : 1, ws.data, ws.bytes, stream),
               "Matmul");
     }
 };
 
 // Matmul<bfloat16, int8_t, float> (include/kernels_amx.hpp:1319-1516): takes the bf16 weights,
 // compresses them to int8 per tensor at the first call (1363-1377) and sets the post-op's dequant
-// scale (1379).  M <= 32 streams the int8 weights; larger M multiplies by the exactly converted
-// bf16 copy of the packed int8 weights, made once.
+// scale (1379).  The packed int8 weights are the only copy: M <= 32 streams them through the decode kernels,
+// larger M converts the int8 fragments to bf16 between LDS and the MFMA operand (the reference's on-the-fly
+// dequantisation, 1447-1497).
 template <>
 struct Matmul<bfloat16, int8_t, float> {
     PackedB<int8_t> internalBI8;
-    PackedB<bfloat16> weiBuff;
     bool constB;
     bool transposeB;
     constexpr static int kStep = 32;
@@ -344,6 +376,7 @@ struct Matmul<bfloat16, int8_t, float> {
         const int N = matB.dims[transposeB ? 0 : 1];
         require(K == matB.dims[transposeB ? 1 : 0], "Matmul: K of A and B differ");
         require(K >= kStep, "Matmul: K must be at least kStep");
+        require(ppkernel.out_rows() >= M && ppkernel.out_cols() >= n1, "Matmul: C is smaller than M x n1");
         if (!constB || !internalBI8) {
             tensor2D<int8_t> Wq(matB.dims[0], matB.dims[1]);
             device_vector<float> scales(2);
@@ -356,21 +389,11 @@ struct Matmul<bfloat16, int8_t, float> {
             const std::vector<float> s = scales.to_host();
             quant_scale_B = s[0];
             dequant_scale_B = s[1];
-            weiBuff = PackedB<bfloat16>();
         }
         ppkernel.set_deq_scale(dequant_scale_B);
         const mmx_epilogue e = ppkernel.descriptor();
-        if (M <= 32) {
-            check(mmx_gemm(MMX_BF16, MMX_I8, matA.data, matA.stride, internalBI8.data, M, K, N, n0, n1, &e, stream),
-                  "Matmul<bf16,int8>");
-        } else {
-            if (!weiBuff) {
-                weiBuff = alloc_packed<bfloat16>(K, N);
-                check(mmx_dequant_packed(internalBI8.data, K, N, weiBuff.data, stream), "Matmul<bf16,int8>: dequant");
-            }
-            check(mmx_gemm(MMX_BF16, MMX_BF16, matA.data, matA.stride, weiBuff.data, M, K, N, n0, n1, &e, stream),
-                  "Matmul<bf16,int8>");
-        }
+        check(mmx_gemm(MMX_BF16, MMX_I8, matA.data, matA.stride, internalBI8.data, M, K, N, n0, n1, &e, stream),
+              "Matmul<bf16,int8>");
     }
 };
 
@@ -398,6 +421,7 @@ struct MatmulW4 {
         const int N = matB.dims[transposeB ? 0 : 1];
         require(K == matB.dims[transposeB ? 1 : 0], "MatmulW4: K of A and B differ");
         require(M <= 32, "MatmulW4: int4 weights are a decode path (M <= 32)");
+        require(ppkernel.out_rows() >= M && ppkernel.out_cols() >= n1, "MatmulW4: C is smaller than M x n1");
         if (!constB || !internalB4.data) {
             // (freeing the previous buffers waits for the launches that still read them)
             internalB4 = device_vector<uint8_t>(mmx_packed_b_bytes(MMX_I4, K, N));
@@ -472,6 +496,9 @@ struct MLP {
     int m_N = 0, m_K = 0, m_M = 0;
     PackedB<bfloat16> gate_up, down;
     tensor2D<bfloat16> actUp;
+    // K slices of the down projection: the reference builds `down` with do_splitK = true (two halves,
+    // tests/amx-mlp.cpp:768); 0 = the library chooses, 1 = never, 2 = the reference's partition
+    int down_k_splits = 0;
 
     void setup(const tensor2D<bfloat16>& w_gate, const tensor2D<bfloat16>& w_up, const tensor2D<bfloat16>& w_down,
                hipStream_t stream = nullptr) {
@@ -496,8 +523,9 @@ struct MLP {
         const int M = x.dims[0];
         require(x.dims[1] == m_K && y.dims[0] == M && y.dims[1] == m_K, "run: x and y must be [M, K]");
         setM(M);
-        check(mmx_mlp(x.data, x.stride, gate_up.data, down.data, actUp.data, actUp.stride, y.data, y.stride, M, m_K, m_N,
-                      stream),
+        const Workspace ws = (down_k_splits == 1 || M <= 32) ? Workspace() : workspace_for(stream);
+        check(mmx_mlp_splitk(x.data, x.stride, gate_up.data, down.data, actUp.data, actUp.stride, y.data, y.stride, M, m_K, m_N,
+                             ws.data ? down_k_splits : 1, ws.data, ws.bytes, stream),
               "MLP::run");
     }
 };

@@ -270,7 +270,7 @@ def _packed_bytes_host(dtype, K, N):
 
 def _split_args(A, k_splits, ws):
     """(k_splits, workspace pointer, bytes): without an explicit workspace the stream's own one is used."""
-    if k_splits == 1:
+    if k_splits == 1 and ws is None:
         return 1, None, 0
     if ws is None:
         ws = workspace(A.device)

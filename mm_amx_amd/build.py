@@ -14,7 +14,8 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmm_amx_amd.so")
 # the MFMA tile GEMM is instantiated per (input type, output type) pair in a file of its own, so that the
 # pairs compile side by side
-SOURCES = ["abi.hip", "gemm_bf16.hip", "gemm_i8.hip",
+SOURCES = ["abi.hip", "gemm_bf16.hip", "gemm_i8.hip", "gemm_w8.hip",
+           "gemm_w8_out_bf16.hip", "gemm_w8_out_f32.hip", "gemm_w8_out_i8.hip",
            "gemm_bf16_out_bf16.hip", "gemm_bf16_out_f32.hip", "gemm_bf16_out_i8.hip",
            "gemm_i8_out_i8.hip", "gemm_i8_out_i32.hip", "gemm_i8_out_f32.hip", "gemm_i8_out_bf16.hip",
            "skinny.hip", "repack.hip", "probe.hip"]

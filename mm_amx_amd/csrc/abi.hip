@@ -65,7 +65,9 @@ int launch_gemm_tiles_bf16(const void* A, int64_t lda, const void* Bp, int M, in
                            const Epilogue& ep, const SplitRequest& rq, hipStream_t st);
 int launch_gemm_tiles_i8(const void* A, int64_t lda, const void* Bp, int M, int K, int N, int n0, int n1,
                          const Epilogue& ep, const SplitRequest& rq, hipStream_t st);
-size_t plan_workspace_bytes(int elesz, int M, int K, int Ncols, uint32_t steps, int k_splits);
+int launch_gemm_tiles_w8(const void* A, int64_t lda, const void* Bp, int M, int K, int N, int n0, int n1,
+                         const Epilogue& ep, const SplitRequest& rq, hipStream_t st);
+size_t plan_workspace_bytes(int elesz, bool w8, int M, int K, int Ncols, uint32_t steps, int k_splits);
 bool skinny_i8_eligible(const void* x, int64_t ldx, int M, int K);
 int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
                   const Epilogue& ep, hipStream_t st);
@@ -169,7 +171,7 @@ static int gemm_dispatch(int a_dtype, int b_dtype, const void* A, int64_t lda_by
     if (i8 && skinny_i8_eligible(A, lda_bytes, M, K) && forced_tile().bm == 0)
         return launch_skinny(3, A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st);
     if (w4) return set_error(MMX_E_UNSUPPORTED, "mmx_gemm: bf16 x int4-weight is a decode path (M <= 32)");
-    if (w8) return set_error(MMX_E_UNSUPPORTED, "mmx_gemm: bf16 x int8-weight with M > 32: convert the weights with mmx_dequant_packed and call the bf16 GEMM");
+    if (w8) return launch_gemm_tiles_w8(A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, rq, st);
     return i8 ? launch_gemm_tiles_i8(A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, rq, st)
               : launch_gemm_tiles_bf16(A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, rq, st);
 }
@@ -297,8 +299,9 @@ int mmx_gemm_splitk_static(int a_dtype, int b_dtype, const void* A, int64_t lda_
 
 size_t mmx_gemm_workspace_bytes(int a_dtype, int b_dtype, int M, int K, int N, int n0, int n1, uint32_t steps, int k_splits) {
     const bool bf = a_dtype == MMX_BF16 && b_dtype == MMX_BF16, i8 = a_dtype == MMX_I8 && b_dtype == MMX_I8;
-    if ((!bf && !i8) || M <= 32 || K <= 0 || N <= 0 || n0 < 0 || n1 > N || n0 >= n1 || k_splits < 0) return 0;
-    return plan_workspace_bytes(bf ? 2 : 1, M, K, n1 - n0, steps, k_splits);
+    const bool w8 = a_dtype == MMX_BF16 && b_dtype == MMX_I8;
+    if ((!bf && !i8 && !w8) || M <= 32 || K <= 0 || N <= 0 || n0 < 0 || n1 > N || n0 >= n1 || k_splits < 0) return 0;
+    return plan_workspace_bytes(i8 ? 1 : 2, w8, M, K, n1 - n0, steps, k_splits);
 }
 
 int mmx_matvec(int dtype, const void* A, int64_t lda_bytes, const void* b, void* c, int M, int K, void* stream) {

@@ -23,12 +23,12 @@ int launch_gemm_tiles_bf16(const void* A, int64_t lda, const void* Bp, int M, in
 }
 
 // Bytes of workspace the plan for this shape would use (0: no K split), assuming operands the ring pipeline takes.
-size_t plan_workspace_bytes(int elesz, int M, int K, int Ncols, uint32_t steps, int k_splits) {
+size_t plan_workspace_bytes(int elesz, bool w8, int M, int K, int Ncols, uint32_t steps, int k_splits) {
     const int64_t kbytes = (int64_t)K * elesz;
     if (kbytes % 128) return 0;
     const SplitRequest rq = {k_splits, reinterpret_cast<char*>(256), ~(size_t)0};
     if (steps & MMX_PP_SILU_GATE) return 0;
-    const Plan p = choose_plan(M, Ncols, (int)(kbytes / 128), false, 2, rq);
+    const Plan p = choose_plan(M, Ncols, (int)(kbytes / 128), false, w8, 2, rq);
     if (p.S <= 1) return 0;
     const size_t tiles = (size_t)((M + p.t.bm - 1) / p.t.bm) * ((Ncols + p.t.bn - 1) / p.t.bn);
     return WS_COUNTER_BYTES + tiles * p.S * p.t.bm * p.t.bn * 4;

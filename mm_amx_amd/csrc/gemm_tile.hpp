@@ -59,6 +59,22 @@ template <>
 struct Mfma<__bf16> {
     using frag = bf16x8;
     using accv = f32x16;
+    static constexpr bool W8 = false;
+    static __device__ __forceinline__ accv run(frag a, frag b, accv c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float to_f32(float v) { return v; }
+};
+// bf16 activations on int8-compressed weights, converted (exactly) on their way from LDS to the MFMA operand:
+// the on-the-fly dequantisation of amx_kernel::Matmul<bf16,int8,float> (include/kernels_amx.hpp:1447-1497).
+// A packed int8 fragment holds 32 of k per column, 16 consecutive k per lane: it feeds two bf16 MFMAs (the
+// lane's first and second eight k), and the A operand is read from the matching places of its row.
+struct w8_t {};
+template <>
+struct Mfma<w8_t> {
+    using frag = bf16x8;
+    using accv = f32x16;
+    static constexpr bool W8 = true;
     static __device__ __forceinline__ accv run(frag a, frag b, accv c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
@@ -68,6 +84,7 @@ template <>
 struct Mfma<int8_t> {
     using frag = i32x4;
     using accv = i32x16;
+    static constexpr bool W8 = false;
     static __device__ __forceinline__ accv run(frag a, frag b, accv c) {
         return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
     }
@@ -123,11 +140,12 @@ __device__ __forceinline__ u32x4 load_a_chunk_masked(const char* rowptr, int kby
 // than a load takes (128x64: 128 cycles of MFMA issue against 1000+ cycles of L2 latency - with three half-stages
 // in flight that tile was bound by latency, 350 cycles per half-stage).  The large tiles get 3 or 4 as before:
 // their half-stages are long enough.
-template <int BM, int BN>
+template <int BM, int BN, bool W8 = false>
 struct Ring {
     static constexpr int A_ST = BM * 128;  // A: one stage = 128 bytes of K per row (whole cache lines)
-    static constexpr int BH = BN * 64;     // B: one half-stage = 64 bytes of K per column (two fragments per panel)
-    static constexpr int NL = BM / 64 + BN / 64;  // HBM->LDS loads per thread per half-stage
+    static constexpr int BH = BN * (W8 ? 32 : 64);  // B: one half-stage = 64 bytes of K per column (two fragments per panel;
+                                                    // one fragment of 32 bytes per column for int8 weights under bf16 A)
+    static constexpr int NL = BM / 64 + BH / 4096;  // HBM->LDS loads per thread per half-stage
     static constexpr int stages_for(int r) { return (r + 3) / 2; }
     static constexpr bool fits(int r) {
         return stages_for(r) * A_ST + r * BH <= 156 * 1024 && (r - 2) * NL + (NL + 1) / 2 <= 63;  // LDS; vmcnt is a 6-bit counter
@@ -146,18 +164,35 @@ struct Ring {
 
 // SMAX: the largest number of K slices per tile this instantiation can combine (1: no K split; the
 // code of the split is then absent and the kernel is the plain one).
+// Development aid, compiled in with -DMMX_STAMPS only: workgroup L records the shader clock at a few points of
+// its life in the 64 bytes at ws_part + 96 MiB + 64 L (the caller provides that much workspace).
+#ifdef MMX_STAMPS
+#define MMX_STAMP(i)                                                                                                   \
+    do {                                                                                                               \
+        if (threadIdx.x == 0 && g.ws_part) {                                                                           \
+            uint64_t* st_ = reinterpret_cast<uint64_t*>(g.ws_part + ((size_t)96 << 20)) + 8 * (size_t)L;              \
+            st_[i] = (i) == 0 || (i) == 7 ? __builtin_amdgcn_s_memrealtime() : __builtin_readcyclecounter();          \
+        }                                                                                                              \
+    } while (0)
+#else
+#define MMX_STAMP(i) do {} while (0)
+#endif
+
 template <typename TIn, int BM, int BN, int MODE, typename TOut, int SMAX>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_kernel(const GemmArgs g) {
     using MF = Mfma<TIn>;
     using frag = typename MF::frag;
     using accv = typename MF::accv;
     using acc_t = typename std::conditional<std::is_same<TIn, int8_t>::value, int, float>::type;
+    constexpr bool W8 = MF::W8;
+    // per panel and k-iteration the packed weights hold 4 KiB (four fragments; two of 32 k each for int8 under bf16 A)
+    constexpr int BP_IT = W8 ? 2048 : 4096;
     // the four waves form a 2x2 grid over the tile, or 4x1 when the tile is only 64 columns wide
     constexpr int WGN = BN >= 128 ? 2 : 1, WGM = 4 / WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int MI = WM / 32, NJ = WN / 32;
-    constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
-    constexpr int A_IT = BM / 32, B_IT = BN / 32;  // 16-byte chunks per thread per stage
+    constexpr int A_BYTES = BM * 128, B_BYTES = BN / 32 * BP_IT, STAGE = A_BYTES + B_BYTES;
+    constexpr int A_IT = BM / 32, B_IT = BN * (BP_IT / 32) / 4096;  // 16-byte chunks per thread per stage
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -181,6 +216,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
     const char* const a_base = g.A + (int64_t)kt0 * 128;
     const int tn = tile / g.tiles_m, tm = tile % g.tiles_m;
+    MMX_STAMP(0);
+    MMX_STAMP(1);
     const int m0 = tm * BM;
     const int ntile0 = g.n0 + tn * BN;
     const int panel0 = ntile0 >> 5;
@@ -218,9 +255,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             // 256 chunks = one panel's 4 KiB of this k-iteration.  A tile may reach past the last
             // panel of the packed weights: re-read the last panel instead (those columns are never
             // stored), which keeps the loop free of branches.
-            int panel = panel0 + it;
+            const int c = it * 256 + tid;
+            int panel = panel0 + c / (BP_IT / 16);
             panel = panel < g.npanels ? panel : g.npanels - 1;
-            const char* src = g.Bp + (int64_t)panel * g.panel_stride + (int64_t)kt * 4096 + tid * 16;
+            const char* src = g.Bp + (int64_t)panel * g.panel_stride + (int64_t)kt * BP_IT + (c % (BP_IT / 16)) * 16;
             rb[it] = *reinterpret_cast<const u32x4*>(src);
         }
     };
@@ -238,12 +276,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     frag fa[2][MI], fb[2][NJ];
     auto read_frags = [&](int stage, int s, frag (&a)[MI], frag (&b)[NJ]) {
         const char* sA = smem + stage * STAGE + (wm * WM + l32) * 128;
-        const char* sB = smem + stage * STAGE + A_BYTES + (wn * NJ * 4) * 1024 + lane * 16;
-        const int slot = (2 * s + g32) ^ (l32 & 7);
+        const char* sB = smem + stage * STAGE + A_BYTES + (wn * NJ) * BP_IT + lane * 16;
+        // k-step s of the stage: the lane's eight k are 16 s + 8 g32 + 0..7, or, under an int8 fragment f = s / 2
+        // (whose lane holds 16 consecutive k), 32 f + 16 g32 + 8 (s % 2) + 0..7
+        const int chunk = W8 ? 4 * (s >> 1) + 2 * g32 + (s & 1) : 2 * s + g32;
+        const int slot = chunk ^ (l32 & 7);
 #pragma unroll
         for (int i = 0; i < MI; i++) a[i] = *reinterpret_cast<const frag*>(sA + i * 32 * 128 + slot * 16);
 #pragma unroll
-        for (int j = 0; j < NJ; j++) b[j] = *reinterpret_cast<const frag*>(sB + (j * 4 + s) * 1024);
+        for (int j = 0; j < NJ; j++) {
+            if constexpr (W8) {
+                const u32x4 raw = *reinterpret_cast<const u32x4*>(sB + (j * 2 + (s >> 1)) * 1024);
+                b[j] = (s & 1) ? s8x8_to_bf16(raw[2], raw[3]) : s8x8_to_bf16(raw[0], raw[1]);
+            } else {
+                b[j] = *reinterpret_cast<const frag*>(sB + (j * 4 + s) * 1024);
+            }
+        }
     };
     auto mma = [&](const frag (&a)[MI], const frag (&b)[NJ]) {
 #pragma unroll
@@ -271,9 +319,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         // While half-stage h is multiplied the windows h+1 .. h+R-1 are in flight.  One workgroup
         // barrier per half-stage; it waits only for window h+1 (s_waitcnt vmcnt(N), the younger loads
         // stay outstanding; loads return in order).
-        using RG = Ring<BM, BN>;
+        using RG = Ring<BM, BN, W8>;
         constexpr int R = RG::R, RA = RG::RA, BH = RG::BH, A_ST = RG::A_ST, B0 = RG::B0;
-        constexpr int A_IT2 = BM / 64, B_IT2 = BN / 64;   // 16-byte chunks per thread per window
+        constexpr int BP_HS = BP_IT / 2;                  // bytes per panel and half-stage
+        static_assert(BH % 4096 == 0, "a half-stage of B must be whole 4 KiB loads of the workgroup");
+        constexpr int A_IT2 = BM / 64, B_IT2 = BH / 4096; // 16-byte chunks per thread per window
         constexpr int MN = MI * NJ;                       // MFMAs per k-step
         constexpr int NL = A_IT2 + B_IT2;                 // HBM->LDS loads per thread per window
         constexpr int H = (NL + 1) / 2;                   // issued in two groups, one load per MFMA slot
@@ -298,11 +348,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
         for (int it = 0; it < B_IT2; it++) {
             const int c = it * 256 + tid;
-            int panel = panel0 + (c >> 7);  // 128 chunks = one panel's two fragments of this half-stage
+            int panel = panel0 + c / (BP_HS / 16);  // 128 chunks = one panel's two fragments of this half-stage (64 = one int8 fragment)
             panel = panel < g.npanels ? panel : g.npanels - 1;
-            boff[it] = (uint32_t)(panel - panel0) * (uint32_t)g.panel_stride + (uint32_t)((c & 127) * 16);
+            boff[it] = (uint32_t)(panel - panel0) * (uint32_t)g.panel_stride + (uint32_t)((c % (BP_HS / 16)) * 16);
         }
-        const char* const b_base = g.Bp + (int64_t)panel0 * g.panel_stride + (int64_t)kt0 * 4096;
+        const char* const b_base = g.Bp + (int64_t)panel0 * g.panel_stride + (int64_t)kt0 * BP_IT;
         const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(
             (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)(smem + wave * 1024));
         const int last_hs = 2 * nk - 1, last_st = nk - 1;
@@ -313,8 +363,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         typedef integral_constant<int, H> cH;
         typedef integral_constant<int, NL> cNL;
 
-        const int a_x0 = (wm * WM + l32) * 128 + ((g32 ^ ((l32 >> 1) & 7)) * 16);
-        const int b_frag_off = B0 + wn * NJ * 2 * 1024 + lane * 16;
+        // A operand of k-step s = 2 PAR + KS of a stage: chunk 2 s + g32 of the row; under int8 fragments (16
+        // consecutive k per lane) chunk 4 PAR + 2 g32 + KS.  Chunks sit at position chunk ^ ((row >> 1) & 7).
+        constexpr int KS1 = W8 ? 1 : 2;  // chunk distance from k-step 0 to k-step 1 of a half-stage
+        const int a_x0 = (wm * WM + l32) * 128 + (((W8 ? 2 * g32 : g32) ^ ((l32 >> 1) & 7)) * 16);
+        const int b_frag_off = B0 + wn * NJ * BP_HS + lane * 16;
+        u32x4 braw[W8 ? NJ : 1];  // int8 fragments as read from LDS: each feeds both k-steps of its half-stage
 
         // Everything a k-step needs besides its operands: where its LDS reads come from and where its
         // loads go.  A wave issues in order and an MFMA slot is 32 cycles = about six instructions, so
@@ -344,7 +398,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 asm volatile("" : "+s"(n.m0B), "+s"(n.m0A));
             } else if constexpr (PART == 1) {
                 const int hs = w < last_hs ? w : last_hs;
-                n.srcB = b_base + (int64_t)hs * 2048;
+                n.srcB = b_base + (int64_t)hs * BP_HS;
                 asm volatile("" : "+s"(n.srcB));
             } else if constexpr (PART == 2) {
                 int st = (w + 1) >> 1;
@@ -354,8 +408,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             } else {
                 // A operand of k-step s (0..3 within the stage): position (2 s + g32) ^ ((row >> 1) & 7) of the row
                 if constexpr (KS == 0) {  // reads k-step 1 of this half-stage
-                    n.rdA = as * A_ST + (a_x0 ^ ((4 * PAR + 2) * 16));
-                    n.rdB = bs * BH + b_frag_off + 1024;
+                    n.rdA = as * A_ST + (a_x0 ^ ((4 * PAR + KS1) * 16));
+                    n.rdB = bs * BH + b_frag_off + 1024;  // (unused with int8 fragments: the second half is in registers)
                 } else {                  // reads k-step 0 of the next half-stage
                     const int nbs = bs + 1 < R ? bs + 1 : 0;
                     n.rdA = PAR == 0 ? as * A_ST + (a_x0 ^ (4 * 16)) : nas * A_ST + a_x0;
@@ -384,9 +438,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
         // one k-step: MFMAs on (ca, cb); meanwhile fill (na, nb) for the next k-step, issue loads [Q0, Q1)
         // and let `prep(part)` work out the parameters of the next k-step in the last slots
+        // ks_c: which k-step of its half-stage this is (the fragments it fetches are those of the other one)
         auto kstep = [&](const frag (&ca)[MI], const frag (&cb)[NJ], frag (&na)[MI], frag (&nb)[NJ], const KParams& kp,
-                         auto q0_c, auto q1_c, auto half_c, auto&& prep) {
-            constexpr int Q0 = decltype(q0_c)::value, Q1 = decltype(q1_c)::value;
+                         auto q0_c, auto q1_c, auto half_c, auto ks_c, auto&& prep) {
+            constexpr int Q0 = decltype(q0_c)::value, Q1 = decltype(q1_c)::value, KS = decltype(ks_c)::value;
             const char* sA = smem + kp.rdA;
             const char* sB = smem + kp.rdB;
             static_for<0, MN>([&](auto t_c) {
@@ -394,8 +449,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 acc[t / NJ][t % NJ] = MF::run(cb[t % NJ], ca[t / NJ], acc[t / NJ][t % NJ]);
                 static_for<t * RPS, (t + 1) * RPS>([&](auto rd_c) {
                     constexpr int rd = decltype(rd_c)::value;
-                    if constexpr (rd < NJ) nb[rd] = *reinterpret_cast<const frag*>(sB + rd * 2 * 1024);
-                    else if constexpr (rd < NJ + MI) na[rd - NJ] = *reinterpret_cast<const frag*>(sA + (rd - NJ) * 32 * 128);
+                    if constexpr (rd < NJ) {
+                        if constexpr (!W8) {
+                            nb[rd] = *reinterpret_cast<const frag*>(sB + rd * BP_HS);
+                        } else if constexpr (KS == 1) {  // next: k-step 0 of the next half-stage - fetch its fragment, use the first half
+                            braw[rd] = *reinterpret_cast<const u32x4*>(sB + rd * BP_HS);
+                            nb[rd] = s8x8_to_bf16(braw[rd][0], braw[rd][1]);
+                        } else {                         // next: k-step 1 of this half-stage - the second half of what is here
+                            nb[rd] = s8x8_to_bf16(braw[rd][2], braw[rd][3]);
+                        }
+                    } else if constexpr (rd < NJ + MI) na[rd - NJ] = *reinterpret_cast<const frag*>(sA + (rd - NJ) * 32 * 128);
                 });
                 if constexpr (Q0 + t < Q1) dma(integral_constant<int, Q0 + t>{}, half_c, kp);
                 // four parts of the next k-step's parameters in the last four slots (all in the last one
@@ -423,7 +486,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 st = st < last_st ? st : last_st;
                 kp.m0B = lds_wave + B0 + W * BH;
                 kp.m0A = lds_wave + (((W + 1) >> 1) % RA) * A_ST + HALF * (BM / 2) * 128;
-                kp.srcB = b_base + (int64_t)hs * 2048;
+                kp.srcB = b_base + (int64_t)hs * BP_HS;
                 kp.srcA = a_base + (int64_t)st * 128;
                 static_for<0, (W < R - 1 ? NL : H)>([&](auto q_c) { dma(q_c, integral_constant<int, HALF>{}, kp); });
             });
@@ -432,13 +495,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         static_for<0, 4>([&](auto part_c) { prepare(part_c, kpa, c0{}, c0{}, 0, 0, RA > 1 ? 1 : 0, 0); });
         asm volatile("s_waitcnt vmcnt(%0)" : : "n"((R - 2) * NL + H) : "memory");  // window 0 and all before it have landed
         __syncthreads();
+        MMX_STAMP(2);
         {
             const char* sA = smem + a_x0;
             const char* sB = smem + b_frag_off;
 #pragma unroll
             for (int i = 0; i < MI; i++) fa[0][i] = *reinterpret_cast<const frag*>(sA + i * 32 * 128);
 #pragma unroll
-            for (int j = 0; j < NJ; j++) fb[0][j] = *reinterpret_cast<const frag*>(sB + j * 2 * 1024);
+            for (int j = 0; j < NJ; j++) {
+                if constexpr (W8) {
+                    braw[j] = *reinterpret_cast<const u32x4*>(sB + j * BP_HS);
+                    fb[0][j] = s8x8_to_bf16(braw[j][0], braw[j][1]);
+                } else {
+                    fb[0][j] = *reinterpret_cast<const frag*>(sB + j * BP_HS);
+                }
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
 
@@ -447,7 +518,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         auto half_stage = [&](auto par_c, int h, int as, int nas, int bs) {
             constexpr int PAR = decltype(par_c)::value;
             // k-step 0: read k-step 1 of this half-stage; second group of the loads of window h+R-1
-            kstep(fa[0], fb[0], fa[1], fb[1], kpa, cH{}, cNL{}, integral_constant<int, (PAR + R) & 1>{},
+            kstep(fa[0], fb[0], fa[1], fb[1], kpa, cH{}, cNL{}, integral_constant<int, (PAR + R) & 1>{}, c0{},
                   [&](auto part_c) { prepare(part_c, kpb, par_c, c1{}, h, as, nas, bs); });
             // every wave now holds all of half-stage h in registers; window h+1 must have landed, the
             // (R-2) younger ones may still be in flight
@@ -461,7 +532,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 as_n = nas;
                 nas_n = nas + 1 < RA ? nas + 1 : 0;
             }
-            kstep(fa[1], fb[1], fa[0], fb[0], kpb, c0{}, cH{}, integral_constant<int, (PAR + R + 1) & 1>{},
+            kstep(fa[1], fb[1], fa[0], fb[0], kpb, c0{}, cH{}, integral_constant<int, (PAR + R + 1) & 1>{}, c1{},
                   [&](auto part_c) { prepare(part_c, kpa, integral_constant<int, 1 - PAR>{}, c0{}, h + 1, as_n, nas_n, nbs); });
         };
         int as = 0, bs = 0;
@@ -522,6 +593,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // the explicit accumulator reads below are invisible to the compiler's hazard checks: let the last
     // MFMAs retire (a 32x32 MFMA needs up to 18 wait states before its result may be read)
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    MMX_STAMP(3);
 
     // ---- K split: park the partial sums, the last slice to arrive combines them ---------------------------
     // Every slice writes its accumulators to its own part of the workspace (each lane 16 bytes per store,
@@ -561,8 +633,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             __syncthreads();
             if (tid == 0) *reinterpret_cast<volatile uint32_t*>(smem) = atomicInc(g.ws_cnt + tile, (uint32_t)g.ksplit - 1u);
             __syncthreads();
-            if (*reinterpret_cast<volatile uint32_t*>(smem) != (uint32_t)g.ksplit - 1u) return;
+            if (*reinterpret_cast<volatile uint32_t*>(smem) != (uint32_t)g.ksplit - 1u) {
+                MMX_STAMP(6);
+                return;
+            }
             asm volatile("" ::: "memory");
+            MMX_STAMP(4);
             combine = true;
         }
     }
@@ -762,6 +838,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             });
         });
     }
+    MMX_STAMP(5);
+    MMX_STAMP(7);
 }
 
 // ---- host side ---------------------------------------------------------------------------------
@@ -795,7 +873,7 @@ struct Plan {
 // per k-iteration of 128 bytes, at the measured issue efficiency of the shape) and of pulling its
 // (BM + BN) * 128 bytes per k-iteration through the CU's L2 -> L1 path (about 48 bytes per cycle).
 // A K split is considered where the slices of all tiles are resident at once.
-static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, int mode, const SplitRequest& rq) {
+static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, bool wide_only, int mode, const SplitRequest& rq) {
     static const struct { int bm, bn; float eff; } cand[] = {
         {256, 256, 0.92f}, {256, 192, 0.90f}, {128, 256, 0.86f}, {128, 192, 0.84f}, {128, 128, 0.80f}, {128, 64, 0.70f}};
     const TileCfg f = forced_tile();
@@ -805,7 +883,7 @@ static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, int mo
     Plan pick = {{128, 128}, 1};
     for (const auto& c : cand) {
         if (f.bm && (f.bm != c.bm || f.bn != c.bn)) continue;
-        if (need_pairs && (c.bn % 128) != 0) continue;
+        if ((need_pairs || wide_only) && (c.bn % 128) != 0) continue;   // (int8 weights under bf16 A: 128 columns per load)
         if (mode == 3 && !(c.bm == 128 && c.bn == 128)) continue;   // the masked path exists for one tile shape
         if (mode != 2 && c.bn == 64) continue;                      // the 64-wide tile exists for the ring pipeline only
         const int tiles = ((M + c.bm - 1) / c.bm) * ((Ncols + c.bn - 1) / c.bn);
@@ -834,6 +912,7 @@ static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, int mo
 
 template <typename T> constexpr const char* type_tag();
 template <> constexpr const char* type_tag<__bf16>() { return "bf16"; }
+template <> constexpr const char* type_tag<w8_t>() { return "w8"; }
 template <> constexpr const char* type_tag<uint16_t>() { return "bf16"; }
 template <> constexpr const char* type_tag<int8_t>() { return "i8"; }
 template <> constexpr const char* type_tag<int32_t>() { return "i32"; }
@@ -841,7 +920,8 @@ template <> constexpr const char* type_tag<float>() { return "f32"; }
 
 template <typename TIn, int BM, int BN, int MODE, typename TOut, int SMAX>
 static int launch_cfg(const GemmArgs& g, int grid, hipStream_t st) {
-    constexpr int lds = MODE == 2 ? Ring<BM, BN>::BYTES : 2 * (BM + BN) * 128;
+    constexpr bool W8 = Mfma<TIn>::W8;
+    constexpr int lds = MODE == 2 ? Ring<BM, BN, W8>::BYTES : 2 * (BM * 128 + BN * (W8 ? 64 : 128));
     auto kern = gemm_kernel<TIn, BM, BN, MODE, TOut, SMAX>;
     static std::atomic<uint64_t> attr_done{0};  // one per instantiation: the devices whose LDS limit has been raised
     int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, attr_done);
@@ -867,24 +947,27 @@ static int launch_tiles(const GemmArgs& g, TileCfg t, int mode, int grid, hipStr
     if (g.ksplit > 1 && mode != 2) return set_error(MMX_E_UNSUPPORTED, "the K split needs the ring pipeline (aligned A, K a multiple of 128 bytes)");
     if (mode == 3) return MMX_LAUNCH(TIn, 128, 128, 3, TOut, 1);  // the masked path exists for one tile shape
     if (t.bm == 256 && t.bn == 256) return MMX_LAUNCH_MODES(TIn, 256, 256, TOut);
-    if (t.bm == 256 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 256, 192, TOut);
     if (t.bm == 128 && t.bn == 256) return MMX_LAUNCH_MODES(TIn, 128, 256, TOut);
-    if (t.bm == 128 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 128, 192, TOut);
     if (t.bm == 128 && t.bn == 128) return MMX_LAUNCH_MODES(TIn, 128, 128, TOut);
-    if (t.bm == 128 && t.bn == 64 && mode == 2 && g.ksplit == 1) return MMX_LAUNCH(TIn, 128, 64, 2, TOut, 1);  // ring pipeline only
+    if constexpr (!Mfma<TIn>::W8) {  // (int8 weights under bf16 A come in tiles of 128 or 256 columns)
+        if (t.bm == 256 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 256, 192, TOut);
+        if (t.bm == 128 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 128, 192, TOut);
+        if (t.bm == 128 && t.bn == 64 && mode == 2 && g.ksplit == 1) return MMX_LAUNCH(TIn, 128, 64, 2, TOut, 1);  // ring pipeline only
+    }
     return set_error(MMX_E_UNSUPPORTED, "no MFMA tile kernel for %dx%d", t.bm, t.bn);
 }
 
 // Fills the launch geometry; returns the grid size (or a negative error code).
+// w8: bf16 A on int8-compressed packed weights (elesz = 2, the size of an element of A).
 static inline int prepare_gemm(GemmArgs& g, TileCfg& t, int& mode, int elesz, const void* A, int64_t lda, const void* Bp,
-                               int M, int K, int N, int n0, int n1, const Epilogue& ep, const SplitRequest& rq) {
+                               int M, int K, int N, int n0, int n1, const Epilogue& ep, const SplitRequest& rq, bool w8 = false) {
     g.A = static_cast<const char*>(A);
     g.lda = lda;
     g.Bp = static_cast<const char*>(Bp);
     g.M = M;
     g.kbytes = K * elesz;
     g.nk = (g.kbytes + 127) / 128;
-    g.panel_stride = (int64_t)g.nk * 4096;
+    g.panel_stride = w8 ? (int64_t)((K + 127) / 128) * 4096 : (int64_t)g.nk * 4096;  // int8 panels: K padded to 128
     g.npanels = (N + 31) / 32;
     g.n0 = n0;
     g.n1 = n1;
@@ -904,7 +987,7 @@ static inline int prepare_gemm(GemmArgs& g, TileCfg& t, int& mode, int elesz, co
     }
     if (use.k_splits > KSPLIT_MAX) return set_error(MMX_E_INVALID, "at most %d K slices", KSPLIT_MAX);
     if (use.k_splits > 1 && !use.ws) return set_error(MMX_E_INVALID, "a K split needs a workspace");
-    const Plan plan = choose_plan(M, n1 - n0, g.nk, pairs, mode, use);
+    const Plan plan = choose_plan(M, n1 - n0, g.nk, pairs, w8, mode, use);
     if (use.k_splits > 1 && plan.S != use.k_splits)
         return set_error(MMX_E_INVALID, "%d K slices do not fit: K too short, the workspace too small, or more than %d tiles",
                          use.k_splits, WS_MAX_TILES);

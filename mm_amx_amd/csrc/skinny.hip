@@ -53,27 +53,6 @@ __device__ __forceinline__ bf16x8 load_x8(const char* xrow, int k0, int K, bool 
     return v;
 }
 
-// 8 int8 (two dwords) -> 8 bf16, exact.  The SDWA form of v_cvt_f32_i32 picks and sign-extends the byte itself:
-// 12 instructions with the packing against 20 for bit-field extract + int-to-float.
-__device__ __forceinline__ bf16x8 s8x8_to_bf16(uint32_t lo, uint32_t hi) {
-    float f[8];
-#define MMX_CVT8(DST, SRC, BYTE) \
-    asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:" BYTE : "=v"(DST) : "v"(SRC))
-    MMX_CVT8(f[0], lo, "BYTE_0");
-    MMX_CVT8(f[1], lo, "BYTE_1");
-    MMX_CVT8(f[2], lo, "BYTE_2");
-    MMX_CVT8(f[3], lo, "BYTE_3");
-    MMX_CVT8(f[4], hi, "BYTE_0");
-    MMX_CVT8(f[5], hi, "BYTE_1");
-    MMX_CVT8(f[6], hi, "BYTE_2");
-    MMX_CVT8(f[7], hi, "BYTE_3");
-#undef MMX_CVT8
-    bf16x8 r;
-#pragma unroll
-    for (int e = 0; e < 8; e++) r[e] = (__bf16)f[e];
-    return r;
-}
-
 // 8 int4 (one dword, element e in bits 4e .. 4e+3, two's complement) -> 8 bf16 holding q / 16, exact.
 // v_cvt_off_f32_i4 maps the low nibble of its source to (signed nibble) / 16; its SDWA form picks the byte,
 // so the even nibbles come straight from the dword and the odd ones from the dword shifted by four:

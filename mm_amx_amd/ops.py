@@ -82,7 +82,6 @@ class Matmul:
     def __init__(self, constB=False, transposeB=False, weight_int8=False):
         self.constB, self.transposeB, self.weight_int8 = constB, transposeB, weight_int8
         self.internalB = None
-        self._bf16_from_i8 = None
         self.quant_scale_B = self.dequant_scale_B = None
 
     def __call__(self, matA, matB, n0=None, n1=None, ppkernel=None):
@@ -105,17 +104,12 @@ class Matmul:
                 q, dq = scales.tolist()
                 self.quant_scale_B, self.dequant_scale_B = q, dq
                 self.internalB = L.repack_b(Wq, self.transposeB)
-                self._bf16_from_i8 = None
             else:
                 self.internalB = L.repack_b(matB, self.transposeB)
         if self.weight_int8:
             ppkernel.set_deq_scale(self.dequant_scale_B)  # include/kernels_amx.hpp:1379
-            if M <= 32:
-                L.gemm(matA, self.internalB, N, ppkernel.descriptor(), b_dtype=L.I8, n0=n0, n1=n1)
-            else:
-                if self._bf16_from_i8 is None or not self.constB:
-                    self._bf16_from_i8 = L.dequant_packed(self.internalB, K, N)
-                L.gemm(matA, self._bf16_from_i8, N, ppkernel.descriptor(), n0=n0, n1=n1)
+            # the int8 fragments are converted between LDS and the MFMA operand at every M (:1447-1497); no bf16 copy
+            L.gemm(matA, self.internalB, N, ppkernel.descriptor(), b_dtype=L.I8, n0=n0, n1=n1)
         else:
             L.gemm(matA, self.internalB, N, ppkernel.descriptor(), n0=n0, n1=n1)
 

@@ -8,6 +8,7 @@
 #include <cstdlib>
 #include <functional>
 #include <random>
+#include <thread>
 #include <vector>
 
 #include "../../include/mm_amx_amd/kernels_gfx950.hpp"
@@ -170,6 +171,22 @@ static void test_matmul_i8_requant(int M, int K, int N) {
     EXPECT(gacc == racc, "int32 accumulators differ");
     EXPECT(got == ref, "requantised int8 output differs");
     EXPECT(gsplit == got, "column-range split differs from the whole-N call");
+    // K split over two workgroups per tile (tests/amx-mlp.cpp:560-593, 648-682): int32 partial sums add exactly
+    if (K >= 1024 && M > 32) {
+        tensor2D<int8_t> Ck(M, N);
+        Ck.zero();
+        Matmul<int8_t, int8_t> mk(true, false);
+        mk.k_splits = 2;
+        PP::BiasGeluStore<int8_t, S> ppk(Ck, bias.data);
+        ppk.set_deq_scale(2e-5f);
+        ppk.set_q_scale(q.data);
+        mk(A, B, ppk);
+        check_hip(hipDeviceSynchronize(), "sync");
+        EXPECT(std::string(mmx_last_kernel()).find("ksplit2") != std::string::npos, "kernel %s is not a two-way K split", mmx_last_kernel());
+        std::vector<int8_t> gk(got.size());
+        Ck.download(gk.data());
+        EXPECT(gk == ref, "two-way K split: requantised int8 output differs");
+    }
 }
 
 // ---- Matmul<bf16,int8,float>: weight compression inside the op (include/kernels_amx.hpp:1319-1516) ----
@@ -279,8 +296,8 @@ static void test_linear_nxn(int M, int K, int N) {
 }
 
 // ---- MLP, stage by stage (h from the same x; y from the same h) ----
-static void test_mlp(int M, int K, int N) {
-    std::printf("  MLP M=%d K=%d N=%d\n", M, K, N);
+static void test_mlp(int M, int K, int N, int down_k_splits = 0) {
+    std::printf("  MLP M=%d K=%d N=%d down_k_splits=%d\n", M, K, N, down_k_splits);
     auto hx = rand_bf16(static_cast<size_t>(M) * K, 1.0f);
     auto hg = rand_bf16(static_cast<size_t>(N) * K, 0.02f), hu = rand_bf16(static_cast<size_t>(N) * K, 0.02f);
     auto hd = rand_bf16(static_cast<size_t>(K) * N, 0.02f);
@@ -290,8 +307,11 @@ static void test_mlp(int M, int K, int N) {
     wu.upload(hu.data());
     wd.upload(hd.data());
     MLP mlp;
+    mlp.down_k_splits = down_k_splits;
     mlp.setup(wg, wu, wd);
     mlp.run(x, y);
+    if (down_k_splits > 1)
+        EXPECT(std::string(mmx_last_kernel()).find("ksplit") != std::string::npos, "down projection ran %s, not a K split", mmx_last_kernel());
     check_hip(hipDeviceSynchronize(), "sync");
     std::vector<bfloat16> gh(static_cast<size_t>(M) * N), gy(static_cast<size_t>(M) * K);
     tensor2D<bfloat16> hview(M, N, mlp.actUp.data, mlp.actUp.stride);
@@ -302,12 +322,57 @@ static void test_mlp(int M, int K, int N) {
     orc_mlp(bits(hx), bits(hg), bits(hu), bits(hd), bits(rh), bits(ry), M, K, N, 0, 0);
     const Err eh = compare(to_f32(gh), to_f32(rh));
     EXPECT(eh.fro <= 1e-3 && eh.within >= 0.999, "h: rel Frobenius %.3e, %.3f%% within 1 bf16 ulp", eh.fro, eh.within * 100);
-    orc_mlp_down(bits(gh), bits(hd), bits(ry_from_gh), M, K, N, 0, 0);
+    orc_mlp_down(bits(gh), bits(hd), bits(ry_from_gh), M, K, N, down_k_splits == 2 ? 1 : 0, 0);
     const Err ey = compare(to_f32(gy), to_f32(ry_from_gh));
     EXPECT(ey.fro <= 1e-3 && ey.within >= 0.999, "y from the GPU's h: rel Frobenius %.3e, %.3f%% within 1 bf16 ulp", ey.fro,
            ey.within * 100);
     const Err ee = compare(to_f32(gy), to_f32(ry));
     EXPECT(ee.fro <= 1e-3, "y end to end: rel Frobenius %.3e", ee.fro);
+}
+
+// ---- first calls from two threads at once: nothing in the library may race on its one-time set-up, and the tuning
+// knobs of one thread must not reach the other ----
+static void test_two_threads_first_call() {
+    std::printf("  first calls from two threads\n");
+    const int M = 300, K = 256, N = 512;
+    auto hA = rand_bf16(static_cast<size_t>(M) * K, 1.0f), hB = rand_bf16(static_cast<size_t>(K) * N, 0.05f);
+    std::vector<float> racc(static_cast<size_t>(M) * N);
+    orc_gemm_bf16(bits(hA), K, bits(hB), N, 0, racc.data(), N, M, K, N, 0);
+    std::vector<float> got[2];
+    std::string kernels[2], errors[2];
+    const char* tiles[2] = {"256x256", "128x256"};  // kernel variants no earlier test has launched with fp32 outputs
+    auto worker = [&](int t) {
+        try {
+            check_hip(hipSetDevice(0), "hipSetDevice");
+            check(mmx_set_tile(tiles[t]), "mmx_set_tile");
+            hipStream_t st;
+            check_hip(hipStreamCreate(&st), "hipStreamCreate");
+            tensor2D<bfloat16> A(M, K), B(K, N);
+            tensor2D<float> C(M, N);
+            A.upload(hA.data());
+            B.upload(hB.data());
+            Matmul<bfloat16, bfloat16> mm(true, false);
+            for (int rep = 0; rep < 3; rep++) mm(A, B, PP::BiasGeluStore<float, PP::NONE>(C), st);
+            kernels[t] = mmx_last_kernel();
+            check_hip(hipStreamSynchronize(st), "sync");
+            got[t].resize(racc.size());
+            C.download(got[t].data());
+            check_hip(hipStreamDestroy(st), "hipStreamDestroy");
+        } catch (const std::exception& e) {
+            errors[t] = e.what();
+        }
+    };
+    std::thread t0(worker, 0), t1(worker, 1);
+    t0.join();
+    t1.join();
+    for (int t = 0; t < 2; t++) {
+        EXPECT(errors[t].empty(), "thread %d: %s", t, errors[t].c_str());
+        EXPECT(kernels[t].find(tiles[t]) != std::string::npos, "thread %d ran %s, its own tile choice was %s", t, kernels[t].c_str(), tiles[t]);
+        if (!got[t].empty()) {
+            const Err e = compare(got[t], racc);
+            EXPECT(e.fro <= 1e-3 && e.within >= 0.999, "thread %d: rel Frobenius %.3e", t, e.fro);
+        }
+    }
 }
 
 // ---- preconditions raise where the reference asserts ----
@@ -345,7 +410,8 @@ int main() {
         test_matmul_i8_requant(256, 512, 320);
         test_matmul_i8_requant(77, 200, 95);
         test_matmul_weight_int8(2, 2560, 192);  // fc16m.cpp:749
-        test_matmul_weight_int8(160, 512, 256);
+        test_matmul_weight_int8(160, 512, 256);   // large M: int8 fragments converted between LDS and the MFMA operand
+        test_matmul_weight_int8(300, 200, 96);    // ... with a K tail (masked loads)
         test_matmul_weight_int4(1, 4096, 352);
         test_matmul_weight_int4(7, 300, 77);
         test_matvec(901, 80);  // main.cpp:884
@@ -354,6 +420,9 @@ int main() {
         test_linear_nxn(512, 128, 4096);  // torch-ext/test.py:37
         test_mlp(1, 512, 1024);
         test_mlp(96, 512, 1024);
+        test_mlp(96, 512, 1024, 2);  // the reference's do_splitK for the down projection (tests/amx-mlp.cpp:768)
+        test_matmul_i8_requant(160, 2048, 320);  // long enough K for the two-way K split
+        test_two_threads_first_call();
         test_errors();
     } catch (const std::exception& e) {
         std::printf("EXCEPTION: %s\n", e.what());

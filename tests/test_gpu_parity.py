@@ -379,7 +379,8 @@ def test_decode_half_panel_form_long_x(po, shape):
 
 @pytest.mark.parametrize("M", [4, 40])
 def test_weight_compressed_matmul(po, M):
-    """Matmul<bf16,int8,float>: bf16 weights compressed per tensor inside the op (include/kernels_amx.hpp:1363-1379)."""
+    """Matmul<bf16,int8,float> (include/kernels_amx.hpp:1319-1516): per-tensor int8 compression at first use, exact
+    int8 -> bf16 conversion on the fly, dequant scale in the post-op."""
     K, N = 512, 160
     rng = np.random.default_rng(15)
     A, W = rand_bf16(rng, (M, K), 1.0), rand_bf16(rng, (K, N), 0.02)
@@ -389,11 +390,67 @@ def test_weight_compressed_matmul(po, M):
     C = torch.zeros((M, N), dtype=torch.float32, device="cuda")
     mm = mx.Matmul(True, False, weight_int8=True)
     mm(dev_bf16(A), dev_bf16(W), ppkernel=mx.BiasGeluStore(C, mx.Steps.DEQUANT))
+    assert ("skinny" in mx.last_kernel()) == (M <= 32) and "w8" in mx.last_kernel(), mx.last_kernel()
     assert np.float32(mm.dequant_scale_B) == np.float32(dq) and np.float32(mm.quant_scale_B) == np.float32(q)
     check_float_parity(host_bits(C), ref, f"w8 matmul M={M}")
     # the compressed weights themselves are integer work: bit-exact
     Wq_gpu, _ = mx.quantize_weights(dev_bf16(W))
     assert np.array_equal(host_bits(Wq_gpu), Wq)
+
+
+def _w8_case(po, M, K, N, seed, steps=None, **gemm_kw):
+    """bf16 x int8-weight GEMM against the bf16 GEMM of the oracle on the (exactly representable) integers."""
+    rng = np.random.default_rng(seed)
+    A = rand_bf16(rng, (M, K), 1.0)
+    Wq = np.clip(np.rint(rng.standard_normal((K, N)) * 40.0), -127, 127).astype(np.int8)
+    scale = rng.uniform(1e-3, 5e-3, N).astype(np.float32)
+    _, acc_ref = po.gemv_w8(A, Wq, np.ones(N, np.float32), want_acc=True)
+    Ad, packed = dev_bf16(A), mx.repack_b(dev(Wq))
+    acc = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    mx.gemm(Ad, packed, N, mx.Epilogue(acc, mx.PP_NONE), b_dtype=mx.I8, **gemm_kw)
+    kernel = mx.last_kernel()
+    check_float_parity(host_bits(acc), acc_ref, f"w8 accumulators {M}x{K}x{N} {kernel}")
+    # per-channel dequant + bf16 store fused: the oracle's post-op on the GPU's accumulators, bit for bit
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    mx.gemm(Ad, packed, N, mx.Epilogue(y, mx.PP_DEQUANT, deq_scale_per_oc=dev(scale)), b_dtype=mx.I8, **gemm_kw)
+    assert mx.last_kernel() == kernel.replace("out_f32", "out_bf16")
+    assert np.array_equal(host_bits(y), po.pp(host_bits(acc), po.PP_DEQUANT, po.BF16, deq_per_oc=scale))
+    return kernel
+
+
+@pytest.mark.parametrize("tile", ["256x256", "128x256", "128x128"])
+@pytest.mark.parametrize("mode", [0, 2])
+def test_w8_gemm_every_kernel_variant(po, tile, mode):
+    """int8-compressed weights under bf16 activations at M > 32: the tile kernels convert the int8 fragments on
+    their way from LDS to the MFMA operand (include/kernels_amx.hpp:1447-1497); no bf16 copy of the weights."""
+    mx.set_tile(tile)
+    mx.set_option("load_mode", mode)
+    try:
+        kernel = _w8_case(po, 600, 512, 832, 170)
+        assert kernel.startswith("gemm_w8_") and tile in kernel and LOAD_NAMES[mode] in kernel, kernel
+    finally:
+        mx.set_tile("")
+        mx.set_option("load_mode", DEFAULT_LOAD_MODE)
+
+
+@pytest.mark.parametrize("shape", [(40, 512, 160), (33, 64, 32), (100, 320, 96), (735, 337, 271), (300, 1000, 200), (64, 4096, 352)])
+def test_w8_gemm_shapes(po, shape):
+    """K tails (masked loads), K = 64 mod 128 (the int8 panels are padded to 128), ragged M and N."""
+    M, K, N = shape
+    kernel = _w8_case(po, M, K, N, 171 + M)
+    assert kernel.startswith("gemm_w8_"), kernel
+
+
+@pytest.mark.parametrize("S", [2, 4])
+def test_w8_gemm_k_split(po, ws, S):
+    kernel = _w8_case(po, 200, 2048, 384, 172 + S, k_splits=S, ws=ws)
+    assert f"ksplit{S}" in kernel, kernel
+
+
+def test_w8_gemm_perf_log_shape(po):
+    """The shape the reference publishes its weight-compressed figure on (perf.log:36: M=896, K=2560, N=10240)."""
+    kernel = _w8_case(po, 896, 2560, 10240, 173)
+    print(f"w8 gemm 896x2560x10240: {kernel}")
 
 
 # ---- mat-vec ---------------------------------------------------------------------------------------------
