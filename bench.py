@@ -26,12 +26,48 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_INT8_TOPS = 5000.0     # MI355X dense int8 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
-# HBM-side bytes per launch of the headline kernel, from two counter runs of this script under
-# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (KiB per dispatch: 81969 and 27915), each scaled by
-# what the same counter reads for the 256 MiB device copy of --calibrate-copy (factors 2.000 and 1.000);
-# the summary is profiles/gemm_bf16_256x192_ffn_up_M1024_hbm_traffic.txt.  Counters cannot be read from
-# inside the process, so the figure is only reported when the kernel that ran is the one profiled.
-MEASURED_TRAFFIC_BYTES = {"gemm_bf16_256x192_ring_out_bf16": (81969 * 2.000 + 27915 * 1.000) * 1024}
+# HBM-side bytes per launch, from two counter runs of this script under `rocprofv3 --pmc FETCH_SIZE` and
+# `--pmc WRITE_SIZE` (KiB per dispatch), each scaled by what the same counter reads for the 256 MiB device copy of
+# --calibrate-copy (factors 2.000 and 1.000); the summaries are profiles/*_hbm_traffic.txt and
+# profiles/skinny_stream_w8_*.txt.  Counters cannot be read from inside the process, so a figure is only reported
+# when the kernel that ran is the one profiled AND its source is the one that was profiled (first 16 hex digits of
+# the SHA-256 of the kernel's source file): after a change of the kernel the figure reads null until it is re-measured.
+MEASURED_TRAFFIC = {
+    "gemm_bf16_256x192_ring_out_bf16": {"bytes": (81969 * 2.000 + 27915 * 1.000) * 1024, "source": "mm_amx_amd/csrc/gemm_tile.hpp",
+                                        "sha": "@GEMM_SHA@"},
+    "skinny_stream_w8": {"bytes": 22174 * 2.000 * 1024 + 22 * 1.000 * 1024, "source": "mm_amx_amd/csrc/skinny.hip", "sha": "@SKINNY_SHA@"},
+}
+
+
+def measured_traffic(kernel_name):
+    import hashlib
+    m = MEASURED_TRAFFIC.get(kernel_name)
+    if not m:
+        return None
+    with open(os.path.join(ROOT, m["source"]), "rb") as f:
+        sha = hashlib.sha256(f.read()).hexdigest()[:16]
+    return m["bytes"] if sha == m["sha"] else None
+
+
+def host_cores():
+    cores = os.cpu_count() or 1
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        pass
+    return min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+
+
+def time_cpu(fn, budget_s):
+    """(repetitions, seconds): fn() repeated until budget_s has passed (after one untimed call)."""
+    fn()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > budget_s:
+            return reps, el
 
 
 def main():
@@ -39,7 +75,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU time budget of the headline baseline (the others get a third each)")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 256 MiB device-to-device copy: a kernel of known traffic to scale profiler byte counters by")
@@ -93,6 +130,15 @@ def main():
     kernel_name = mx.last_kernel()
     value = flops / (ms_per_step * 1e-3) / 1e12
     achieved = flops / (kernel_ms * 1e-3) / 1e12
+    # the same launches once more with an event between every two of them: the median launch (not part of `value`)
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    evs[0].record()
+    for i in range(args.steps):
+        step()
+        evs[i + 1].record()
+    torch.cuda.synchronize()
+    per_launch = sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(args.steps))
+    kernel_median_ms = per_launch[len(per_launch) // 2]
 
     out = {
         "metric": "bf16 FC GEMM TFLOP/s (M=1024, K=4096, N=11008, fused BIAS+GELU, bf16 out)",
@@ -103,10 +149,10 @@ def main():
                    "inputs": "A~N(0,1) bf16, B~N(0,0.02) bf16 repacked once, bias~N(0,0.1) fp32, all resident in HBM"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(kernel_name),
+                     "traffic": measured_traffic(kernel_name),
                      "algorithmic_flop_per_launch": flops,
                      "algorithmic_bytes_per_launch": 2 * M * K + 2 * K * N + 4 * N + 2 * M * N,
-                     "kernel_avg_us": round(kernel_ms * 1e3, 2)},
+                     "kernel_avg_us": round(kernel_ms * 1e3, 2), "kernel_median_us": round(kernel_median_ms * 1e3, 2)},
     }
 
     if args.calibrate_copy:
@@ -118,30 +164,119 @@ def main():
         out["calibration_copy_bytes"] = {"read": 256 << 20, "written": 256 << 20}
         del src, dst
 
-    # ---- CPU baseline: the oracle (a port of the reference path) on this host's cores --------------
+    # ---- CPU baselines: the oracle (a port of the reference path) and torch-CPU (oneDNN) on this host's cores ----
+    # The reference itself cannot travel to this machine; what is timed is the CPU restatement of its arithmetic
+    # (oracle/, kind "port") and, as the "oneDNN path" of the reference's own comparisons (benchmark/mmbench/dnnl.cpp),
+    # torch's CPU matmul.  Every figure is over a bounded sample of the same workload; protocol as the reference's
+    # timeit (warm-up, then repeat for the budget, mean).
+    cpu_other = {}
     if not args.no_cpu:
         from oracle import pyoracle as po
-        cores = os.cpu_count() or 1
-        try:
-            cores = len(os.sched_getaffinity(0))
-        except AttributeError:
-            pass
-        cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
-        reps = 0
-        t0 = time.perf_counter()
-        while True:
+        cores = host_cores()
+        torch.set_num_threads(cores)
+        isa = po.isa()
+        amx = "has" if po.host_has_amx() else "has no"
+
+        def onednn_bf16(Abits, Bbits, budget):
+            At = torch.from_numpy(Abits.view(np.int16).copy()).view(torch.bfloat16)
+            Bt = torch.from_numpy(Bbits.view(np.int16).copy()).view(torch.bfloat16)
+            reps, el = time_cpu(lambda: torch.matmul(At, Bt), budget)
+            return reps, el
+
+        def gpu_note(fn):
+            try:
+                return fn()
+            except Exception as e:  # a CPU op torch does not have on this host: say so, do not invent a number
+                return {"value": None, "note": f"{type(e).__name__}: {e}"[:160]}
+
+        def run_ref():
             acc = po.gemm_bf16(w["A"], w["B"], nthreads=cores)
             po.pp(acc, po.PP_BIAS | po.PP_GELU, po.BF16, bias=w["bias"])
-            reps += 1
-            el = time.perf_counter() - t0
-            if el > 10.0:
-                break
+        reps, el = time_cpu(run_ref, args.cpu_seconds)
         out["cpu_baseline"] = {
             "value": round(flops * reps / el / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
             "sample": f"{reps} x the full workload (M=1024,K=4096,N=11008 + BIAS_GELU) in {el:.1f} s; portable "
-                      f"{po.isa()} restatement of the AMX summation order (the host "
-                      f"{'has' if po.host_has_amx() else 'has no'} AMX; the AMX intrinsics path is not used)",
+                      f"{isa} restatement of the AMX summation order (the host {amx} AMX; the AMX intrinsics path is not used)",
         }
+        r2, e2 = onednn_bf16(w["A"], w["B"], args.cpu_seconds / 3)
+        out["cpu_baseline"]["onednn"] = {"value": round(flops * r2 / e2 / 1e12, 4), "unit": "TFLOP/s", "cores": cores,
+                                         "sample": f"{r2} x torch.matmul (bf16, CPU, no post-op) of the same shape in {e2:.1f} s"}
+        b3 = args.cpu_seconds / 3
+
+        # config 1: bf16 256^3
+        w1c = wl.gemm_bf16_256()
+        reps, el = time_cpu(lambda: po.gemm_bf16(w1c["A"], w1c["B"], nthreads=cores), min(b3, 1.0))
+        r2, e2 = onednn_bf16(w1c["A"], w1c["B"], min(b3, 1.0))
+        cpu_other["bf16_gemm_256x256x256"] = {
+            "port": {"value": round(2.0 * 256 ** 3 * reps / el / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "sample": f"{reps} x in {el:.2f} s"},
+            "onednn": {"value": round(2.0 * 256 ** 3 * r2 / e2 / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "sample": f"{r2} x torch.matmul in {e2:.2f} s"}}
+
+        # config 3: int8 FC with requant
+        wic = wl.int8_fc()
+        opsi = 2.0 * wic["M"] * wic["K"] * wic["N"]
+
+        def run_i8():
+            acc = po.gemm_i8(wic["A"], wic["B"])
+            po.pp(acc, po.PP_DEQUANT | po.PP_BIAS | po.PP_QUANT, po.I8, bias=wic["bias"], deq_per_oc=wic["deq"], q=float(wic["q"]))
+        reps, el = time_cpu(run_i8, b3)
+
+        def onednn_i8():
+            Ai, Bi = torch.from_numpy(wic["A"]), torch.from_numpy(wic["B"])
+            r, e = time_cpu(lambda: torch._int_mm(Ai, Bi), b3)
+            return {"value": round(opsi * r / e / 1e12, 4), "unit": "TOP/s", "cores": cores, "sample": f"{r} x torch._int_mm (CPU, no post-op) in {e:.1f} s"}
+        cpu_other["int8_fc_requant_M512_K4096_N4096"] = {
+            "port": {"value": round(opsi * reps / el / 1e12, 4), "unit": "TOP/s", "cores": cores, "sample": f"{reps} x the full workload in {el:.1f} s"},
+            "onednn": gpu_note(onednn_i8)}
+
+        # config 4: decode GEMV over int8 weights, M=1, rotating over 8 weight copies (360 MB: nothing stays in a cache)
+        wgc = wl.decode_gemv_w8(M=1)
+        Wcopies = [wgc["W"].copy() for _ in range(8)]
+        turn = [0]
+
+        def run_gemv():
+            po.gemv_w8(wgc["x"], Wcopies[turn[0] % 8], wgc["scale"], nthreads=cores)
+            turn[0] += 1
+        reps, el = time_cpu(run_gemv, b3)
+        wbytes = float(wgc["K"]) * wgc["N"]
+
+        def onednn_gemv():
+            xt = torch.from_numpy(wgc["x"].view(np.int16).copy()).view(torch.bfloat16)
+            Wt = [torch.from_numpy(Wc).to(torch.bfloat16) for Wc in Wcopies]   # oneDNN has no mixed bf16 x int8 matmul: bf16 weights
+            t2 = [0]
+
+            def f():
+                torch.matmul(xt, Wt[t2[0] % 8])
+                t2[0] += 1
+            r, e = time_cpu(f, b3)
+            return {"value": round(2 * wbytes * r / e / 1e9, 2), "unit": "GB/s", "cores": cores,
+                    "sample": f"{r} x torch.matmul(x bf16 [1,4096], W bf16 [4096,11008]) over 8 rotated copies in {e:.1f} s (bf16 weights: 2 bytes each)"}
+        cpu_other["decode_gemv_int8w_K4096_N11008_M1"] = {
+            "port": {"value": round(wbytes * reps / el / 1e9, 2), "unit": "GB/s", "cores": cores,
+                     "sample": f"{reps} x the full GEMV over 8 rotated weight copies in {el:.1f} s (the restatement converts the weights to bf16 on every call)"},
+            "onednn": gpu_note(onednn_gemv)}
+        del Wcopies
+
+        # config 5: fused MLP at M=1 and M=2048
+        wmc = wl.llama_mlp(M=2048)
+        for Mm in (1, 2048):
+            xs = np.ascontiguousarray(wmc["x"][:Mm])
+            reps, el = time_cpu(lambda: po.mlp(xs, wmc["w_gate"], wmc["w_up"], wmc["w_down"], split_k=True), b3)
+            fl = 6.0 * Mm * wmc["K"] * wmc["N"]
+            ent = {"port": {"value": round(fl * reps / el / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "sample": f"{reps} x the full MLP in {el:.1f} s",
+                            "weight_GBps": round(6.0 * wmc["K"] * wmc["N"] * reps / el / 1e9, 1)}}
+
+            def onednn_mlp():
+                xt = torch.from_numpy(xs.view(np.int16).copy()).view(torch.bfloat16)
+                g, u, d = (torch.from_numpy(wmc[k].view(np.int16).copy()).view(torch.bfloat16) for k in ("w_gate", "w_up", "w_down"))
+                F = torch.nn.functional
+
+                def f():
+                    F.linear(F.silu(F.linear(xt, g)) * F.linear(xt, u), d)
+                r, e = time_cpu(f, b3)
+                return {"value": round(fl * r / e / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "sample": f"{r} x torch (three F.linear + silu, bf16, CPU) in {e:.1f} s"}
+            ent["onednn"] = gpu_note(onednn_mlp)
+            cpu_other[f"llama7b_mlp_fused_M{Mm}"] = ent
+        del wmc
 
     # ---- the other configurations of the path --------------------------------------------------------
     if not args.no_extra:
@@ -151,6 +286,11 @@ def main():
             # a new shape needs about a hundred launches before its time settles (fresh buffers, clocks)
             mx.time_gemm(Ain, packs, Nn, epi, max(100, iters // 2), **kw)
             return mx.time_gemm(Ain, packs, Nn, epi, iters, **kw)
+
+        def med_us(Ain, packs, Nn, epi, **kw):
+            # median of eleven means over as many launches as there are weight copies (at least ten)
+            n = max(10, len(packs))
+            return round(sorted(mx.time_gemm(Ain, packs, Nn, epi, n, **kw) for _ in range(11))[5] * 1e3, 2)
 
         # bf16 256^3, fp32 out, no post-op (launch-latency bound; reported, not a roofline case)
         w1 = wl.gemm_bf16_256()
@@ -167,8 +307,9 @@ def main():
             As = dev_bf16(ws["A"])
             Cs = torch.zeros((Ms, N), dtype=torch.bfloat16, device="cuda")
             ms = avg_ms(As, [Bp], N, mx.Epilogue(Cs, mx.PP_BIAS | mx.PP_GELU, bias=bias), 100)
-            sweep[str(Ms)] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * Ms * N * K / ms / 1e9, 1),
-                              "kernel": mx.last_kernel()}
+            sweep[str(Ms)] = {"us": round(ms * 1e3, 1), "median_us": med_us(As, [Bp], N, mx.Epilogue(Cs, mx.PP_BIAS | mx.PP_GELU, bias=bias)),
+                              "tflops": round(2.0 * Ms * N * K / ms / 1e9, 1),
+                              "frac_of_bf16_peak": round(2.0 * Ms * N * K / ms / 1e9 / PEAK_BF16_TFLOPS, 4), "kernel": mx.last_kernel()}
             del As, Cs
         extra["bf16_fc_bias_gelu_sweep_M"] = sweep
 
@@ -181,8 +322,8 @@ def main():
         ms = avg_ms(Ai, [Bi], wi["N"], epi, 100)
         ops = 2.0 * wi["M"] * wi["K"] * wi["N"]
         extra["int8_fc_requant_M512_K4096_N4096"] = {
-            "us": round(ms * 1e3, 2), "tops": round(ops / ms / 1e9, 1), "frac_of_int8_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4),
-            "kernel": mx.last_kernel()}
+            "us": round(ms * 1e3, 2), "median_us": med_us(Ai, [Bi], wi["N"], epi), "tops": round(ops / ms / 1e9, 1),
+            "frac_of_int8_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4), "kernel": mx.last_kernel()}
         del Ai, Bi, Ci
         # the same int8 kernel on a shape large enough to fill the machine (the Llama-7B FFN shape at M=2048)
         rng = np.random.default_rng(11)
@@ -209,8 +350,10 @@ def main():
             epg = mx.Epilogue(yg, mx.PP_DEQUANT, deq_scale_per_oc=sg)
             ms = avg_ms(xg, packs, wg["N"], epg, 240, b_dtype=mx.I8)
             wbytes = float(wg["K"]) * wg["N"]
-            gemv[str(Mg)] = {"us": round(ms * 1e3, 2), "weight_GBps": round(wbytes / ms / 1e6, 0),
-                             "frac_of_hbm_peak": round(wbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "kernel": mx.last_kernel()}
+            gemv[str(Mg)] = {"us": round(ms * 1e3, 2), "median_us": med_us(xg, packs, wg["N"], epg, b_dtype=mx.I8),
+                             "weight_GBps": round(wbytes / ms / 1e6, 0),
+                             "frac_of_hbm_peak": round(wbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "kernel": mx.last_kernel(),
+                             "traffic": measured_traffic(mx.last_kernel()) if Mg == 1 else None, "algorithmic_bytes": wbytes}
             del packs, Wg
         extra["decode_gemv_int8w_K4096_N11008"] = gemv
 
@@ -242,6 +385,36 @@ def main():
                               "frac_of_hbm_peak": round(wbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "kernel": mx.last_kernel()}
         del packs, P4, W4
         extra["decode_gemv_int4w_K4096_N11008"] = gemv4
+
+        # bf16 activations on int8-compressed weights at large M: the shape the reference publishes its
+        # weight-compressed figure on (perf.log:36: M=896, K=2560, N=10240); the int8 fragments are converted on the fly
+        Mw, Kw, Nw = 896, 2560, 10240
+        Aw = torch.randn((Mw, Kw), dtype=torch.float32, device="cuda").to(torch.bfloat16)
+        Ww = mx.repack_b(torch.randint(-127, 128, (Kw, Nw), dtype=torch.int8, device="cuda"))
+        Cw = torch.zeros((Mw, Nw), dtype=torch.float32, device="cuda")
+        epw = mx.Epilogue(Cw, mx.PP_DEQUANT, deq_scale=0.01)
+        ms = avg_ms(Aw, [Ww], Nw, epw, 100, b_dtype=mx.I8)
+        extra["bf16_x_int8w_gemm_M896_K2560_N10240"] = {
+            "us": round(ms * 1e3, 2), "tflops": round(2.0 * Mw * Kw * Nw / ms / 1e9, 1),
+            "frac_of_bf16_peak": round(2.0 * Mw * Kw * Nw / ms / 1e9 / PEAK_BF16_TFLOPS, 4), "kernel": mx.last_kernel(),
+            "weight_bytes_resident": int(Ww.numel())}
+        del Aw, Ww, Cw
+
+        # shapes with few output tiles, where K is split over several workgroups per tile (the MLP's down
+        # projection at prefill sizes below a full machine): with and without the split
+        ksp = {}
+        Wdn = mx.repack_b((torch.randn((11008, 4096), dtype=torch.float32, device="cuda") * 0.02).to(torch.bfloat16))
+        for Ms in (64, 256):
+            hs = torch.randn((Ms, 11008), dtype=torch.float32, device="cuda").to(torch.bfloat16)
+            ys = torch.zeros((Ms, 4096), dtype=torch.bfloat16, device="cuda")
+            eps = mx.Epilogue(ys, mx.PP_NONE)
+            t_split = avg_ms(hs, [Wdn], 4096, eps, 100)
+            k_split = mx.last_kernel()
+            t_plain = avg_ms(hs, [Wdn], 4096, eps, 100, k_splits=1)
+            ksp[str(Ms)] = {"us": round(t_split * 1e3, 2), "kernel": k_split, "us_without_split": round(t_plain * 1e3, 2),
+                            "kernel_without_split": mx.last_kernel(), "tflops": round(2.0 * Ms * 11008 * 4096 / t_split / 1e9, 1)}
+        extra["bf16_down_proj_K11008_N4096_ksplit"] = ksp
+        del Wdn
 
         # fused Llama-7B MLP
         mlp = {}
@@ -351,7 +524,11 @@ def main():
             rate, mhz = mx.probe_mfma(dt, rnd, 20000)
             ceil[key] = {"rate": round(rate, 1), "unit": "TFLOP/s" if dt == mx.BF16 else "TOP/s", "shader_mhz": round(mhz)}
         extra["mfma_issue_loop"] = ceil
+        if cpu_other:
+            extra["cpu_baselines"] = cpu_other
         out["extra"] = extra
+    elif cpu_other:
+        out["extra"] = {"cpu_baselines": cpu_other}
 
     print(json.dumps(out))
 

@@ -58,7 +58,10 @@ enum {
  *            saturate to [-128,127]; MMX_I32 (only with steps == 0 on int8 inputs) raw accumulator.
  * With MMX_PP_SILU_GATE the packed weights hold gate and up projections in alternating
  * 32-column panels (see mmx_repack_gate_up) and the output has half as many columns:
- *     C[m, c] = bf16( silu(acc_gate[m, c]) * acc_up[m, c] )   (DEQUANT/BIAS/GELU/QUANT must be off)
+ *     C[m, c] = bf16( silu(acc_gate[m, c]) * acc_up[m, c] )   (BIAS/GELU/QUANT must be off)
+ * over compressed weights (int8, int4) MMX_PP_DEQUANT may be set with it (an extension, the reference's MLP is
+ * bf16 only): each sum is first multiplied by the dequant scale of its own packed column,
+ *     C[m, c] = bf16( silu(acc_gate * deq[gate column]) * (acc_up * deq[up column]) )
  * deq_scale_per_oc is an extension: the reference has a per-tensor dequant scale only.
  */
 typedef struct mmx_epilogue {
@@ -108,7 +111,9 @@ int mmx_quantize_weights(const void* W, int64_t ldw_bytes, int rows, int cols, v
  * (weight_compression/wcompress.hpp:90-134, README.md:216-244: "we haven't found efficient instructions to
  * implement a fully-functional dequant() for INT4"); this is the real thing for the decode path.  Per output
  * channel n, symmetric: a = max_k |w[k][n]|, q[k][n] = clamp(rint(w[k][n] * (7 / a)), -7, 7) in fp32 (q = 0 for
- * a = 0), deq_scales_out[n] = a / 7.  W is [K, N] bf16 (transpose = 0) or [N, K] (transpose = 1, torch layout),
+ * a = 0), deq_scales_out[n] = a / 7.  Non-finite weights: NaNs do not take part in the maximum; a NaN weight, and
+ * every infinite weight (its column has a = inf, so 7 / a = 0 and the product is NaN), quantises to 0, and such a
+ * column's deq scale is inf.  W is [K, N] bf16 (transpose = 0) or [N, K] (transpose = 1, torch layout),
  * row stride ldw_bytes.  packed receives mmx_packed_b_bytes(MMX_I4, K, N) bytes: 32-column panels of 1 KiB
  * fragments, a fragment = 32 columns x 64 of k; the lane g * 32 + c (c = column in the panel, g = 0, 1) owns
  * bytes [16 (g*32+c), +16): dword i holds k = 64 f + 32 g + 8 i + e in bits [4e, 4e+4), two's complement;

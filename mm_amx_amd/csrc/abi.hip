@@ -114,7 +114,9 @@ static int make_epilogue(const mmx_epilogue* in, int a_dtype, int b_dtype, int M
     // here the converse is enforced: an enabled step must have its operand
     if ((in->steps & MMX_PP_BIAS) && !in->bias) return set_error(MMX_E_INVALID, "epilogue: BIAS step without a bias pointer");
     if (in->steps & MMX_PP_SILU_GATE) {
-        if (in->steps != MMX_PP_SILU_GATE) return set_error(MMX_E_INVALID, "epilogue: SILU_GATE excludes every other step");
+        // compressed weights need their scales before the non-linearity: DEQUANT (alone) may come with it
+        if (in->steps & ~(uint32_t)(MMX_PP_SILU_GATE | MMX_PP_DEQUANT))
+            return set_error(MMX_E_INVALID, "epilogue: SILU_GATE excludes every other step but DEQUANT");
         if (in->out_dtype != MMX_BF16 && in->out_dtype != MMX_F32)
             return set_error(MMX_E_INVALID, "epilogue: SILU_GATE stores bf16 or fp32");
         if (a_dtype != MMX_BF16) return set_error(MMX_E_INVALID, "epilogue: SILU_GATE needs bf16 activations");

@@ -780,6 +780,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                         gt[v] = MF::to_f32(raw[v]);
                         up[v] = MF::to_f32(acc_read(acc[i][j + 1][v]));
                     }
+                    if (ep.steps & MMX_PP_DEQUANT) {  // compressed weights: gate and up each by the scale of its own column
+                        if (ep.deq_oc) {
+                            float dg[16], du[16];
+                            load_per_oc(ep.deq_oc, wave_col0 + 32 * j, dg);
+                            load_per_oc(ep.deq_oc, wave_col0 + 32 * j + 32, du);
+#pragma unroll
+                            for (int v = 0; v < 16; v++) gt[v] = gt[v] * dg[v], up[v] = up[v] * du[v];
+                        } else {
+#pragma unroll
+                            for (int v = 0; v < 16; v++) gt[v] = gt[v] * ep.deq, up[v] = up[v] * ep.deq;
+                        }
+                    }
                     silu_mul_x16(gt, up, r, seg_of_lane);
                     store_block(r, raw, m0 + wm * WM + 32 * i + l32, ((wave_col0 + 32 * j) >> 1));
                     __builtin_amdgcn_sched_barrier(0);

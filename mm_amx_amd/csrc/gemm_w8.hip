@@ -10,7 +10,6 @@ int launch_tiles_w8_out_i8(const GemmArgs& g, TileCfg t, int mode, int grid, hip
 
 int launch_gemm_tiles_w8(const void* A, int64_t lda, const void* Bp, int M, int K, int N, int n0, int n1,
                          const Epilogue& ep, const SplitRequest& rq, hipStream_t st) {
-    if (ep.steps & MMX_PP_SILU_GATE) return set_error(MMX_E_UNSUPPORTED, "SILU_GATE over int8 weights exists for M <= 32 only");
     GemmArgs g;
     TileCfg t;
     int mode;

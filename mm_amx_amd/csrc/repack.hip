@@ -355,6 +355,7 @@ __global__ __launch_bounds__(256) void quant4_pack_kernel(const char* W, int64_t
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             float q = rintf(wval(k0 + e, n0 + c) * qs);
+            q = (q != q) ? 0.0f : q;  // a NaN weight, or an infinite one (its column's scale is then 0): quantised to 0
             q = fminf(fmaxf(q, -7.0f), 7.0f);
             d |= ((uint32_t)(int)q & 0xfu) << (4 * e);
         }

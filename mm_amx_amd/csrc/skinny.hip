@@ -105,7 +105,7 @@ __device__ __forceinline__ void skinny_prefetch(const SkinnyArgs& s, int panel_f
 #pragma unroll
         for (int p = 0; p < NP; p++) {
             const int n = ((panel_first + p) << 5) + nloc;
-            const bool ok = row_live && n < s.n1 && !(ep.steps & MMX_PP_SILU_GATE);
+            const bool ok = row_live && n < s.n1;  // (with SILU_GATE the only other step is DEQUANT, of gate and up each)
             o.deq[t][p] = ep.deq;
             o.bias[t][p] = 0.0f;
             o.q[t][p] = ep.q;
@@ -154,7 +154,12 @@ __device__ __forceinline__ void skinny_finish(const SkinnyArgs& s, const float (
         } else if (ep.steps & MMX_PP_SILU_GATE) {
             if constexpr (NP == 2) {
                 const int n = ((panel_first >> 1) << 5) + nloc;  // output column (half width)
-                if (n < (s.n1 >> 1)) store_out(ep, m, n, silu(sum[0]) * sum[1]);
+                float gate = sum[0], up = sum[1];
+                if (ep.steps & MMX_PP_DEQUANT) {  // compressed weights: each of the two sums by the scale of its own column
+                    gate = gate * o.deq[t][0];
+                    up = up * o.deq[t][1];
+                }
+                if (n < (s.n1 >> 1)) store_out(ep, m, n, silu(gate) * up);
             }
         } else {
 #pragma unroll
@@ -708,7 +713,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #pragma unroll
         for (int p = 0; p < NP; p++) {
             const int n = ((panel_first + p) << 5) + nloc;
-            const bool ok = l32 < s.M && n < s.n1 && !(ep.steps & MMX_PP_SILU_GATE);
+            const bool ok = l32 < s.M && n < s.n1;
             o_deq[t][p] = ep.deq;
             o_bias[t][p] = 0.0f;
             o_q[t][p] = ep.q;
@@ -828,7 +833,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         if (ep.steps & MMX_PP_SILU_GATE) {
             if constexpr (NP == 2) {
                 const int n = ((panel_first >> 1) << 5) + nloc;  // output column (half width)
-                if (n < (s.n1 >> 1)) store_out(ep, m, n, silu(sum[0]) * sum[1]);
+                float gate = sum[0], up = sum[1];
+                if (ep.steps & MMX_PP_DEQUANT) {
+                    gate = gate * o_deq[t][0];
+                    up = up * o_deq[t][1];
+                }
+                if (n < (s.n1 >> 1)) store_out(ep, m, n, silu(gate) * up);
             }
         } else {
 #pragma unroll
@@ -900,16 +910,26 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
     }
     if (wk == 2) {
         // int4 weights: the streaming kernel if x fits in LDS and K fills whole fragments, else the general one
-        if (pairs) return set_error(MMX_E_UNSUPPORTED, "SILU_GATE over int4 weights is not built");
+        if (pairs && (panels & 1)) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
         const int zoff = (M * K * 2 + 1023) & ~1023;
         const int xb = zoff + K * 2;
         if (s.nfrag * 64 == K && xb <= 46 * 1024 && s.x_vec_ok) {
-            note_kernel("skinny_stream_w4");
-            if ((s.nfrag + 7) / 8 <= 8)
+            note_kernel(pairs ? "skinny_stream_w4_gateup" : "skinny_stream_w4");
+            if (pairs) {  // gate and up panels side by side: four fragments of each in flight per wave
+                if ((s.nfrag + 7) / 8 <= 4)
+                    hipLaunchKernelGGL((skinny_stream_kernel<2, 2, true>), dim3(panels / 2), dim3(512), stream_lds_bytes(xb, 2), st, s, zoff);
+                else
+                    hipLaunchKernelGGL((skinny_stream_kernel<2, 2, false>), dim3(panels / 2), dim3(512), stream_lds_bytes(xb, 2), st, s, zoff);
+            } else if ((s.nfrag + 7) / 8 <= 8)
                 hipLaunchKernelGGL((skinny_stream_kernel<2, 1, true>), dim3(panels), dim3(512), stream_lds_bytes(xb, 1), st, s, zoff);
             else
                 hipLaunchKernelGGL((skinny_stream_kernel<2, 1, false>), dim3(panels), dim3(512), stream_lds_bytes(xb, 1), st, s, zoff);
             return check_hip(hipGetLastError(), "skinny_stream_kernel launch");
+        }
+        if (pairs) {  // x too large for LDS or a ragged K: the general kernel
+            note_kernel("skinny_w4_gateup");
+            hipLaunchKernelGGL((skinny_kernel<2, 2>), dim3(panels / 2), dim3(512), 0, st, s);
+            return check_hip(hipGetLastError(), "skinny_kernel launch");
         }
         if (s.nfrag * 64 == K && s.x_vec_ok) {
             // x too large for LDS: through LDS chunk by chunk (two buffers of 16 or 32 rows x 1 KiB)
@@ -957,10 +977,10 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
             if (rc) return rc;
         }
     }
-    if (kpad == K && (xbytes <= 46 * 1024 || bigx) && s.x_vec_ok && !(pairs && w8)) {
+    if (kpad == K && (xbytes <= 46 * 1024 || bigx) && s.x_vec_ok) {
         // the activations fit in LDS: streaming variant
         if (pairs && (panels & 1)) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
-        note_kernel(pairs ? "skinny_stream_bf16_gateup" : (w8 ? "skinny_stream_w8" : "skinny_stream_bf16"));
+        note_kernel(pairs ? (w8 ? "skinny_stream_w8_gateup" : "skinny_stream_bf16_gateup") : (w8 ? "skinny_stream_w8" : "skinny_stream_bf16"));
         const int per_wave = (s.nfrag + 7) / 8;
         // Half-panel workgroups pay off for up to 4 rows of x (cheap enough to stage per workgroup) if each still has at least
         // 128 KiB of weights to stream (measured: 64 KiB units lose more to the fixed cost of a workgroup than the
@@ -971,7 +991,8 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         const int wg_per_cu = (160 * 1024 / lds_wg) < 4 ? (160 * 1024 / lds_wg) : 4;
         const int64_t unit_bytes = (int64_t)s.nfrag * 512 * (pairs ? 2 : 1);
         const int force = decode_halves();  // -1: by the rule above, 0: never, 1: for every M <= 4 (tests pin the path with it)
-        const bool halves = M <= 4 && !bigx && force != 0 && (force == 1 || (2 * units <= 2 * num_cus() * wg_per_cu && unit_bytes >= 128 * 1024));
+        const bool halves = M <= 4 && !bigx && !(pairs && w8) && force != 0 &&
+                            (force == 1 || (2 * units <= 2 * num_cus() * wg_per_cu && unit_bytes >= 128 * 1024));
         const int per_wave_h = ((s.nfrag >> 1) + 3) / 4;
 #define MMX_STREAM(W8, NP, GRID)                                                                                     \
     do {                                                                                                             \
@@ -985,7 +1006,10 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
             hipLaunchKernelGGL((skinny_stream_kernel<W8, NP, false>), dim3(GRID), dim3(512), stream_lds_bytes(xbytes, NP), st, s, zero_off); \
     } while (0)
         if (halves) note_kernel(pairs ? "skinny_half_bf16_gateup" : (w8 ? "skinny_half_w8" : "skinny_half_bf16"));
-        if (pairs) MMX_STREAM(false, 2, panels / 2);
+        if (pairs && w8) {
+            if (per_wave <= 8) hipLaunchKernelGGL((skinny_stream_kernel<1, 2, true>), dim3(panels / 2), dim3(512), stream_lds_bytes(xbytes, 2), st, s, zero_off);
+            else hipLaunchKernelGGL((skinny_stream_kernel<1, 2, false>), dim3(panels / 2), dim3(512), stream_lds_bytes(xbytes, 2), st, s, zero_off);
+        } else if (pairs) MMX_STREAM(false, 2, panels / 2);
         else if (w8) MMX_STREAM(true, 1, panels);
         else MMX_STREAM(false, 1, panels);
 #undef MMX_STREAM

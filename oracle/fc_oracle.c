@@ -203,6 +203,7 @@ void orc_quantize_int4(const uint16_t* W, int64_t ldw, int K, int N, int transpo
         deq[n] = a / 7.0f;
         for (int k = 0; k < K; k++) {
             float r = rintf(orc_bf16_to_f32(transpose ? W[(size_t)n * ldw + k] : W[(size_t)k * ldw + n]) * qs);
+            if (r != r) r = 0.0f; /* NaN weight, or an infinite one in a column whose maximum (NaN aside) is infinite: 0 */
             r = r < -7.0f ? -7.0f : (r > 7.0f ? 7.0f : r);
             q[(size_t)k * N + n] = (int8_t)r;
         }

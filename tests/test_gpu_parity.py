@@ -790,6 +790,25 @@ def test_int4_quantise_and_pack_match_the_definition(po, shape, transpose):
     assert np.array_equal(host_bits(packed), want)
 
 
+def test_int4_quantise_non_finite_weights(po):
+    """NaN and infinite weights quantise to 0, NaNs are left out of the column maximum, an infinity makes the
+    column's dequant scale infinite: the kernel and the definition agree bit for bit."""
+    K, N = 300, 45
+    rng = np.random.default_rng(7)
+    Wf = (rng.standard_normal((K, N)) * 0.03).astype(np.float32)
+    Wf[5, 0] = np.nan
+    Wf[7, 1] = np.inf
+    Wf[9, 2] = -np.inf
+    Wf[11, 2] = np.nan
+    Wf[:, 3] = np.nan
+    W = po.f32_to_bf16(Wf)
+    q, deq = po.quantize_int4(W)
+    assert q[5, 0] == 0 and not q[:, 1].any() and not q[:, 2].any() and not q[:, 3].any() and np.isinf(deq[1]) and deq[3] == 0
+    packed, deq_gpu = mx.quantize_pack_int4(dev_bf16(W))
+    assert np.array_equal(host_bits(deq_gpu).view(np.uint32), deq.view(np.uint32))
+    assert np.array_equal(host_bits(packed), po.pack_int4(q))
+
+
 @pytest.mark.parametrize("shape", [(1, 256, 64), (3, 320, 100), (16, 337, 96), (32, 2560, 192), (2, 4096, 352), (4, 8192, 64),
                                    (8, 4096, 352), (20, 1024, 100), (16, 11008, 64)])
 def test_int4_decode_shapes(po, shape):
@@ -839,8 +858,8 @@ def test_int4_is_a_decode_path_only():
     y = torch.zeros((40, 64), dtype=torch.float32, device="cuda")
     with pytest.raises(mx.MmxError, match="decode path"):
         mx.gemm(x, packed, 64, mx.Epilogue(y, mx.PP_NONE), b_dtype=mx.I4)
-    with pytest.raises(mx.MmxError):
-        mx.gemm(x[:4], packed, 64, mx.Epilogue(y[:4, :32], mx.PP_SILU_GATE), b_dtype=mx.I4)
+    with pytest.raises(mx.MmxError, match="every other step but DEQUANT"):
+        mx.gemm(x[:4], packed, 64, mx.Epilogue(y[:4, :32], mx.PP_SILU_GATE | mx.PP_BIAS, bias=deq), b_dtype=mx.I4)
     with pytest.raises(mx.MmxError):
         mx.quantize_pack_int4(torch.zeros((256, 64), dtype=torch.float32, device="cuda"))
 
@@ -1068,3 +1087,61 @@ def test_mlp_down_projection_split(po, ws, M):
     assert np.array_equal(ys[0], ys[1])
     y_ref = po.mlp_down(host_bits(h), w["w_down"], split_k=True)
     check_float_parity(bf16_to_f32(ys[0]), bf16_to_f32(y_ref), f"mlp down split M={M}")
+
+
+# ---- SiLU(gate) * up over compressed weights (an extension: the reference's MLP is bf16 only) ----------------------
+def _interleave_panels(Wg, Wu):
+    """[K, N] gate and up -> [K, 2N] with gate and up alternating in 32-column panels (the layout of mmx_repack_gate_up)."""
+    K, N = Wg.shape
+    out = np.empty((K, 2 * N), Wg.dtype)
+    out.reshape(K, N // 32, 2, 32)[:, :, 0, :] = Wg.reshape(K, N // 32, 32)
+    out.reshape(K, N // 32, 2, 32)[:, :, 1, :] = Wu.reshape(K, N // 32, 32)
+    return out
+
+
+@pytest.mark.parametrize("shape", [(1, 512, 128), (3, 1024, 96), (4, 4096, 352), (16, 768, 64), (32, 2560, 192), (5, 300, 64), (2, 11008, 64),
+                                   (48, 512, 256), (300, 1024, 384)])
+@pytest.mark.parametrize("wk", ["w8", "w4"])
+def test_silu_gate_over_compressed_weights(po, shape, wk):
+    """bf16(silu(acc_gate * deq[gate column]) * (acc_up * deq[up column])): accumulators against the oracle's bf16 GEMM
+    on the integer weights, the fused store bit for bit against the oracle's SiLU on the GPU's own accumulators."""
+    M, K, N = shape
+    if wk == "w4" and M > 32:
+        pytest.skip("int4 weights are a decode path (M <= 32)")
+    rng = np.random.default_rng(M * 7 + K + N)
+    x = rand_bf16(rng, (M, K), 1.0)
+    if wk == "w8":
+        Wg = np.clip(np.rint(rng.standard_normal((K, N)) * 40.0), -127, 127).astype(np.int8)
+        Wu = np.clip(np.rint(rng.standard_normal((K, N)) * 40.0), -127, 127).astype(np.int8)
+        Wgu = _interleave_panels(Wg, Wu)
+        deq = rng.uniform(2e-4, 6e-4, 2 * N).astype(np.float32)
+        packed, deq_d, b_dt = mx.repack_b(dev(Wgu)), dev(deq), mx.I8
+        q_int = Wgu
+    else:
+        Wgu_f = _interleave_panels(rand_bf16(rng, (K, N), 0.02), rand_bf16(rng, (K, N), 0.02))
+        q_int, deq = po.quantize_int4(Wgu_f)
+        packed, deq_d = mx.quantize_pack_int4(dev_bf16(Wgu_f))
+        assert np.array_equal(host_bits(deq_d), deq)
+        b_dt = mx.I4
+    xd = dev_bf16(x)
+    acc = torch.zeros((M, 2 * N), dtype=torch.float32, device="cuda")
+    mx.gemm(xd, packed, 2 * N, mx.Epilogue(acc, mx.PP_NONE), b_dtype=b_dt)
+    k_plain = mx.last_kernel()
+    _, acc_ref = po.gemv_w8(x, q_int.astype(np.int8), np.ones(2 * N, np.float32), want_acc=True)
+    check_float_parity(host_bits(acc), acc_ref, f"{wk} gate/up accumulators {shape}")
+    h = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    mx.gemm(xd, packed, 2 * N, mx.Epilogue(h, mx.PP_SILU_GATE | mx.PP_DEQUANT, deq_scale_per_oc=deq_d), b_dtype=b_dt)
+    k_fused = mx.last_kernel()
+    a = (host_bits(acc) * deq[None, :]).astype(np.float32).reshape(M, N // 32, 2, 32)
+    gate, up = np.ascontiguousarray(a[:, :, 0, :]).reshape(M, N), np.ascontiguousarray(a[:, :, 1, :]).reshape(M, N)
+    want = po.silu_mul_bf16(gate, up)
+    if k_fused.replace("_gateup", "").replace("out_bf16", "out_f32") == k_plain:
+        assert np.array_equal(host_bits(h), want), (k_plain, k_fused)
+    else:
+        # the plain and the fused call took different kernels (different order of the partial sums): compare with the
+        # oracle's SiLU on the oracle's accumulators, to the floating-point bar
+        a = (acc_ref * deq[None, :]).astype(np.float32).reshape(M, N // 32, 2, 32)
+        ref = po.silu_mul_bf16(np.ascontiguousarray(a[:, :, 0, :]).reshape(M, N), np.ascontiguousarray(a[:, :, 1, :]).reshape(M, N))
+        check_float_parity(bf16_to_f32(host_bits(h)), bf16_to_f32(ref), f"{wk} silu-gate {shape} ({k_plain} / {k_fused})")
+    if K % 256 == 0 and M <= 32 and (M + 1) * K * 2 <= 40 * 1024:   # x and its zero row fit in LDS beside the pair's scratch
+        assert "stream" in k_fused and "gateup" in k_fused, k_fused

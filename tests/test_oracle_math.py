@@ -198,3 +198,17 @@ def test_gelu_deep_negative_tail_is_ill_conditioned(po):
         return np.mean(np.abs(y - y1) > ulp)
     assert frac_beyond_one_bf16_ulp(-4.9, -4.3) > 0.25
     assert frac_beyond_one_bf16_ulp(-3.0, 5.0) == 0.0
+
+
+def test_int4_non_finite_weights_are_defined(po):
+    """NaNs do not take part in a column's maximum; a NaN weight and every infinite weight quantise to 0; a column
+    holding an infinity has an infinite dequant scale (so its finite weights quantise to 0 as well)."""
+    W = np.full((8, 4), 0.5, np.float32)
+    W[:, 0] = [1.0, -2.0, np.nan, 0.5, 0.25, -1.0, 2.0, 0.0]         # a NaN among finite weights: max 2
+    W[:, 1] = [1.0, np.inf, -3.0, 0.5, 0.25, -1.0, 2.0, 0.0]          # an infinity
+    W[:, 2] = [np.nan] * 8                                            # nothing but NaNs: max 0
+    q, deq = po.quantize_int4(po.f32_to_bf16(W))
+    assert list(q[:, 0]) == [4, -7, 0, 2, 1, -4, 7, 0] and deq[0] == np.float32(2.0) / np.float32(7.0)
+    assert not q[:, 1].any() and np.isinf(deq[1])
+    assert not q[:, 2].any() and deq[2] == 0.0
+    assert list(q[:, 3]) == [7] * 8
