@@ -85,24 +85,32 @@ __device__ __forceinline__ float gelu_erf_minimax(float x) {
     return p;
 }
 
-// The same function on the 16 accumulators a lane holds of one 32x32 block.  A wavefront that is
-// alone on its SIMD cannot issue a dependent vector instruction back to back, so the 16 Horner
-// chains advance in lockstep, one coefficient at a time.  The three selects only matter outside
-// 2^-24 < |x| <= 5; they are skipped when no element of any lane of the wavefront is out there
-// (v_max/v_min drop a NaN operand: a NaN then comes out of the polynomial as NaN, as it would
-// out of the select).  Same result bit for bit.
-__device__ __forceinline__ void gelu_erf_minimax_x16(float (&r)[16]) {
-    constexpr uint32_t coef[14] = {0xa3198977u, 0x268a7927u, 0xa998c963u, 0x2c67ddb2u, 0xaf013b2cu, 0x315d4a4fu, 0xb3969b11u,
-                                   0x35a776e9u, 0xb79b0914u, 0x3970b255u, 0xbb1b7399u, 0x3ca3621fu, 0xbe082bc7u, 0x3f4c4228u};
+// The coefficients once more, for the 16-wide form below: read through a pointer they are fetched by scalar loads
+// and live in scalar registers, which makes each Horner step a plain v_fma_f32; written as literals they become
+// 64-bit v_fmaak_f32 instructions, which a lone wavefront issues 17 % slower (measured: 1495 against 1261 cycles
+// per 16 values).  (The caller passes each word through an empty asm statement, or the compiler folds the known
+// values back into literals.)
+__constant__ static const uint32_t kGeluCoef[15] = {0x1f1c83fdu, 0xa3198977u, 0x268a7927u, 0xa998c963u, 0x2c67ddb2u,
+                                                    0xaf013b2cu, 0x315d4a4fu, 0xb3969b11u, 0x35a776e9u, 0xb79b0914u,
+                                                    0x3970b255u, 0xbb1b7399u, 0x3ca3621fu, 0xbe082bc7u, 0x3f4c4228u};
+
+// The same function on the 16 accumulators a lane holds of one 32x32 block.  A wavefront that is alone on its SIMD
+// issues one vector instruction every 4 to 5 cycles whatever their dependences, so the 16 Horner chains simply
+// advance in lockstep, one coefficient at a time (cf: the 15 coefficients, in scalar registers).  The three
+// selects only matter outside 2^-24 < |x| <= 5; they are skipped when no element of any lane of the wavefront is
+// out there (v_max/v_min drop a NaN operand: a NaN then comes out of the polynomial as NaN, as it would out of
+// the select).  Same result bit for bit.  (Inside the GEMM's epilogue the test and branch cost less than applying
+// the selects to every element: 26.9k against 28.7k cycles per 256x192 tile.)
+__device__ __forceinline__ void gelu_erf_minimax_x16(float (&r)[16], const float (&cf)[15]) {
     float x2[16], p[16];
 #pragma unroll
     for (int v = 0; v < 16; v++) x2[v] = r[v] * r[v];
 #pragma unroll
-    for (int v = 0; v < 16; v++) p[v] = __builtin_fmaf(u2f(0x1f1c83fdu), x2[v], u2f(coef[0]));
+    for (int v = 0; v < 16; v++) p[v] = __builtin_fmaf(cf[0], x2[v], cf[1]);
 #pragma unroll
-    for (int c = 1; c < 14; c++) {
+    for (int c = 2; c < 15; c++) {
 #pragma unroll
-        for (int v = 0; v < 16; v++) p[v] = __builtin_fmaf(p[v], x2[v], u2f(coef[c]));
+        for (int v = 0; v < 16; v++) p[v] = __builtin_fmaf(p[v], x2[v], cf[c]);
     }
 #pragma unroll
     for (int v = 0; v < 16; v++) p[v] = __builtin_fmaf(p[v], r[v], 1.0f);
@@ -115,7 +123,9 @@ __device__ __forceinline__ void gelu_erf_minimax_x16(float (&r)[16]) {
         amin = __builtin_fminf(amin, __builtin_fabsf(r[v]));
     }
     const bool needs_select = !(amax <= 5.0f) || !(amin > u2f(0x33800000u));
-    if (__builtin_amdgcn_ballot_w64(needs_select) != 0) {
+    // (unlikely: the selects are laid out away from the straight path, which then has no taken branch - the epilogue's
+    // code runs once per tile, out of a cold instruction cache, and every taken branch restarts the fetch)
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(needs_select) != 0, 0)) {
 #pragma unroll
         for (int v = 0; v < 16; v++) {
             float x = r[v];

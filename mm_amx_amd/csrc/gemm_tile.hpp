@@ -230,6 +230,40 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0;
 
+    // The per-column operands of the post-op (bias, per-channel dequant and quant scales) of this tile's BN columns
+    // go into LDS behind the operand buffers, straight from memory (global_load_lds_dword: 64 columns per
+    // instruction, no registers) and ahead of every operand load, so they have long landed when the epilogue
+    // reads them: fetched at the point of use, each column block paid a trip to memory with the matrix pipe idle.
+    constexpr int OC_OFF = MODE == 2 ? Ring<BM, BN, W8>::BYTES : 2 * STAGE;
+    {
+        const Epilogue& e0 = g.ep;
+        const float* const src_of[3] = {(e0.steps & MMX_PP_BIAS) ? e0.bias : nullptr,
+                                        (e0.steps & MMX_PP_DEQUANT) ? e0.deq_oc : nullptr,
+                                        (e0.steps & MMX_PP_QUANT) ? e0.q_oc : nullptr};
+        const uint32_t oc_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)(smem + OC_OFF));
+        const int wave_s = __builtin_amdgcn_readfirstlane(wave);  // (uniform: the LDS address goes through M0)
+        if (wave_s * 64 < BN) {
+            int n = ntile0 + wave_s * 64 + lane;
+            n = n < g.n1 ? n : g.n1 - 1;  // columns past the range are never stored: any valid address will do
+#pragma unroll
+            for (int a = 0; a < 3; a++) {
+                if (src_of[a]) {
+                    const float* src = src_of[a] + n;
+                    const uint32_t m0v = oc_lds + a * BN * 4 + wave_s * 256;
+                    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(m0v), "v"(src) : "memory");
+                }
+            }
+        }
+    }
+
+    float gelu_c[15];  // the GELU polynomial's coefficients, fetched into scalar registers ahead of the main loop
+#pragma unroll
+    for (int c = 0; c < 15; c++) {
+        uint32_t bits = kGeluCoef[c];
+        asm volatile("" : "+s"(bits));  // opaque: keeps the coefficient in a scalar register (see gelu_erf_minimax_x16)
+        gelu_c[c] = u2f(bits);
+    }
+
     u32x4 ra[MODE == 2 ? 1 : A_IT], rb[MODE == 2 ? 1 : B_IT];  // staging registers of modes 0 and 3
 
     auto fetch = [&](int kt) {
@@ -698,19 +732,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int out_n1 = silu_gate ? (g.n1 >> 1) : g.n1;
     const int wave_col0 = ntile0 + wn * WN;  // first column of this wave, in accumulator columns
 
-    // 16 per-column values of block column bcol for this lane: index v <-> column bcol + 8(v/4) + 4 g32 + v%4
-    auto load_per_oc = [&](const float* p, int bcol, float (&dst)[16]) {
+    // 16 per-column values (array a of the LDS copy: 0 bias, 1 dequant scale, 2 quant scale) of the block column that
+    // starts at column lcol of the tile, for this lane: index v <-> column lcol + 8(v/4) + 4 g32 + v%4
+    auto load_per_oc = [&](int a, int lcol, float (&dst)[16]) {
+        const char* base = smem + OC_OFF + a * BN * 4 + (lcol + 4 * g32) * 4;
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-            const int n = bcol + 8 * q + 4 * g32;
-            if (n + 4 <= g.n1 && (reinterpret_cast<uintptr_t>(p) & 15) == 0) {
-                const f32x4 t = *reinterpret_cast<const f32x4*>(p + n);
+            const f32x4 t = *reinterpret_cast<const f32x4*>(base + q * 32);
 #pragma unroll
-                for (int e = 0; e < 4; e++) dst[4 * q + e] = t[e];
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; e++) dst[4 * q + e] = (n + e < g.n1) ? p[n + e] : 0.0f;
-            }
+            for (int e = 0; e < 4; e++) dst[4 * q + e] = t[e];
         }
     };
     // stores the 16 values r[] (or the raw int32 sums) of one block: row grow, output columns
@@ -783,8 +813,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     if (ep.steps & MMX_PP_DEQUANT) {  // compressed weights: gate and up each by the scale of its own column
                         if (ep.deq_oc) {
                             float dg[16], du[16];
-                            load_per_oc(ep.deq_oc, wave_col0 + 32 * j, dg);
-                            load_per_oc(ep.deq_oc, wave_col0 + 32 * j + 32, du);
+                            load_per_oc(1, wn * WN + 32 * j, dg);
+                            load_per_oc(1, wn * WN + 32 * j + 32, du);
 #pragma unroll
                             for (int v = 0; v < 16; v++) gt[v] = gt[v] * dg[v], up[v] = up[v] * du[v];
                         } else {
@@ -807,9 +837,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             constexpr int j = decltype(jc)::value;
             const int bcol = wave_col0 + 32 * j;
             float deq_v[16], bias_v[16], q_v[16];
-            if ((ep.steps & MMX_PP_DEQUANT) && ep.deq_oc) load_per_oc(ep.deq_oc, bcol, deq_v);
-            if (ep.steps & MMX_PP_BIAS) load_per_oc(ep.bias, bcol, bias_v);
-            if ((ep.steps & MMX_PP_QUANT) && ep.q_oc) load_per_oc(ep.q_oc, bcol, q_v);
+            if ((ep.steps & MMX_PP_DEQUANT) && ep.deq_oc) load_per_oc(1, wn * WN + 32 * j, deq_v);
+            if (ep.steps & MMX_PP_BIAS) load_per_oc(0, wn * WN + 32 * j, bias_v);
+            if ((ep.steps & MMX_PP_QUANT) && ep.q_oc) load_per_oc(2, wn * WN + 32 * j, q_v);
             static_for<0, MI>([&](auto ic) __attribute__((always_inline)) {
                 constexpr int i = decltype(ic)::value;
                 constexpr int step = j * MI + i;
@@ -835,7 +865,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
                     for (int v = 0; v < 16; v++) r[v] = r[v] + bias_v[v];
                 }
-                if (ep.steps & MMX_PP_GELU) gelu_erf_minimax_x16(r);
+                if (ep.steps & MMX_PP_GELU) gelu_erf_minimax_x16(r, gelu_c);
                 if (ep.steps & MMX_PP_QUANT) {
                     if (ep.q_oc) {
 #pragma unroll
@@ -933,7 +963,9 @@ template <> constexpr const char* type_tag<float>() { return "f32"; }
 template <typename TIn, int BM, int BN, int MODE, typename TOut, int SMAX>
 static int launch_cfg(const GemmArgs& g, int grid, hipStream_t st) {
     constexpr bool W8 = Mfma<TIn>::W8;
-    constexpr int lds = MODE == 2 ? Ring<BM, BN, W8>::BYTES : 2 * (BM * 128 + BN * (W8 ? 64 : 128));
+    // operand buffers, then three arrays of BN per-column post-op operands
+    constexpr int lds = (MODE == 2 ? Ring<BM, BN, W8>::BYTES : 2 * (BM * 128 + BN * (W8 ? 64 : 128))) + 3 * BN * 4;
+    static_assert(lds <= 160 * 1024, "LDS of a CU");
     auto kern = gemm_kernel<TIn, BM, BN, MODE, TOut, SMAX>;
     static std::atomic<uint64_t> attr_done{0};  // one per instantiation: the devices whose LDS limit has been raised
     int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, attr_done);
