@@ -178,8 +178,14 @@ struct Ring {
 #define MMX_STAMP(i) do {} while (0)
 #endif
 
-template <typename TIn, int BM, int BN, int MODE, typename TOut, int SMAX>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_kernel(const GemmArgs g) {
+// NW: wavefronts per workgroup.  4 = one per SIMD, each with up to 512 registers (the large accumulator blocks need
+// them); 8 = two per SIMD with 256 registers each, half as large a block per wave: the second wave of a SIMD
+// fills the issue slots the first leaves empty, above all in the epilogue, whose vector instructions a lone
+// wave issues at under half the rate the SIMD executes them (ring pipeline only).
+template <typename TIn, int BM, int BN, int MODE, typename TOut, int SMAX, int NW = 4>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4))) void gemm_kernel(const GemmArgs g) {
+    static_assert(NW == 4 || (NW == 8 && MODE == 2), "eight wavefronts exist for the ring pipeline only");
+    constexpr int NT = NW * 64;  // threads
     using MF = Mfma<TIn>;
     using frag = typename MF::frag;
     using accv = typename MF::accv;
@@ -187,8 +193,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     constexpr bool W8 = MF::W8;
     // per panel and k-iteration the packed weights hold 4 KiB (four fragments; two of 32 k each for int8 under bf16 A)
     constexpr int BP_IT = W8 ? 2048 : 4096;
-    // the four waves form a 2x2 grid over the tile, or 4x1 when the tile is only 64 columns wide
-    constexpr int WGN = BN >= 128 ? 2 : 1, WGM = 4 / WGN;
+    // the waves form a (NW/2) x 2 grid over the tile, or NW x 1 when the tile is only 64 columns wide
+    constexpr int WGN = BN >= 128 ? 2 : 1, WGM = NW / WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int MI = WM / 32, NJ = WN / 32;
     constexpr int A_BYTES = BM * 128, B_BYTES = BN / 32 * BP_IT, STAGE = A_BYTES + B_BYTES;
@@ -356,8 +362,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         using RG = Ring<BM, BN, W8>;
         constexpr int R = RG::R, RA = RG::RA, BH = RG::BH, A_ST = RG::A_ST, B0 = RG::B0;
         constexpr int BP_HS = BP_IT / 2;                  // bytes per panel and half-stage
-        static_assert(BH % 4096 == 0, "a half-stage of B must be whole 4 KiB loads of the workgroup");
-        constexpr int A_IT2 = BM / 64, B_IT2 = BH / 4096; // 16-byte chunks per thread per window
+        // A window's B chunks are NBI wave-wide loads of 1 KiB, dealt to the waves in turn: wave w issues loads
+        // w, w + NW, ...  Where NBI is not a multiple of NW the first NBI % NW waves issue one more than the
+        // others ("class 0" / "class 1"): the pipeline below exists once per class, because the number of a
+        // wave's loads in flight is part of its wait counts.
+        constexpr int NBI = BH / 1024;
+        constexpr int NCLS0 = NBI % NW == 0 ? NW : NBI % NW;   // waves of class 0
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+        auto ring = [&](auto cls_c) __attribute__((always_inline)) {
+        constexpr int CLS = decltype(cls_c)::value;
+        constexpr int A_IT2 = BM * 4 / NT, B_IT2 = CLS == 0 ? (NBI + NW - 1) / NW : NBI / NW; // 16-byte chunks per thread per window
         constexpr int MN = MI * NJ;                       // MFMAs per k-step
         constexpr int NL = A_IT2 + B_IT2;                 // HBM->LDS loads per thread per window
         constexpr int H = (NL + 1) / 2;                   // issued in two groups, one load per MFMA slot
@@ -374,14 +388,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         for (int half = 0; half < 2; half++)
 #pragma unroll
             for (int it = 0; it < A_IT2; it++) {
-                const int row = half * (BM / 2) + it * 32 + (tid >> 3);
+                const int row = half * (BM / 2) + it * (NT / 8) + (tid >> 3);
                 int grow = m0 + row;
                 grow = grow < g.M ? grow : g.M - 1;
                 aoff[half][it] = (uint32_t)grow * (uint32_t)g.lda + (uint32_t)(((tid & 7) ^ ((tid >> 4) & 7)) * 16);
             }
 #pragma unroll
         for (int it = 0; it < B_IT2; it++) {
-            const int c = it * 256 + tid;
+            const int c = it * NT + tid;
             int panel = panel0 + c / (BP_HS / 16);  // 128 chunks = one panel's two fragments of this half-stage (64 = one int8 fragment)
             panel = panel < g.npanels ? panel : g.npanels - 1;
             boff[it] = (uint32_t)(panel - panel0) * (uint32_t)g.panel_stride + (uint32_t)((c % (BP_HS / 16)) * 16);
@@ -459,13 +473,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 const uint32_t off = boff[Q];
                 asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                              :
-                             : "s"(kp.m0B), "v"(off), "s"(kp.srcB), "n"(Q * 4096)
+                             : "s"(kp.m0B), "v"(off), "s"(kp.srcB), "n"(Q * NT * 16)
                              : "memory", "scc");
             } else {
                 const uint32_t off = aoff[HALF][Q - B_IT2];
                 asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                              :
-                             : "s"(kp.m0A), "v"(off), "s"(kp.srcA), "n"((Q - B_IT2) * 4096)
+                             : "s"(kp.m0A), "v"(off), "s"(kp.srcA), "n"((Q - B_IT2) * NT * 16)
                              : "memory", "scc");
             }
         };
@@ -579,6 +593,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             as = nas;
         }
         asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // the re-fetched slots past the end must land before the wave ends
+        };  // ring
+        if constexpr (NCLS0 == NW) {
+            ring(std::integral_constant<int, 0>{});
+        } else {
+            if (wave_u < NCLS0) ring(std::integral_constant<int, 0>{});
+            else ring(std::integral_constant<int, 1>{});
+        }
     } else {
     fetch(kt0);
     commit(0);
@@ -891,6 +912,7 @@ struct TileCfg {
 };
 TileCfg forced_tile();
 int load_mode();
+int wave_count();
 int ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done_on_device);
 
 // Where the partial sums of a K split live: the first WS_COUNTER_BYTES hold one arrival counter per tile
@@ -960,22 +982,22 @@ template <> constexpr const char* type_tag<int8_t>() { return "i8"; }
 template <> constexpr const char* type_tag<int32_t>() { return "i32"; }
 template <> constexpr const char* type_tag<float>() { return "f32"; }
 
-template <typename TIn, int BM, int BN, int MODE, typename TOut, int SMAX>
+template <typename TIn, int BM, int BN, int MODE, typename TOut, int SMAX, int NW = 4>
 static int launch_cfg(const GemmArgs& g, int grid, hipStream_t st) {
     constexpr bool W8 = Mfma<TIn>::W8;
     // operand buffers, then three arrays of BN per-column post-op operands
     constexpr int lds = (MODE == 2 ? Ring<BM, BN, W8>::BYTES : 2 * (BM * 128 + BN * (W8 ? 64 : 128))) + 3 * BN * 4;
     static_assert(lds <= 160 * 1024, "LDS of a CU");
-    auto kern = gemm_kernel<TIn, BM, BN, MODE, TOut, SMAX>;
+    auto kern = gemm_kernel<TIn, BM, BN, MODE, TOut, SMAX, NW>;
     static std::atomic<uint64_t> attr_done{0};  // one per instantiation: the devices whose LDS limit has been raised
     int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds, attr_done);
     if (rc) return rc;
     static const char* const loads[] = {"regs", "", "ring", "masked"};
     char name[96];
-    snprintf(name, sizeof name, "gemm_%s_%dx%d_%s_out_%s%s", type_tag<TIn>(), BM, BN, loads[MODE], type_tag<TOut>(),
+    snprintf(name, sizeof name, "gemm_%s_%dx%d_%s%s_out_%s%s", type_tag<TIn>(), BM, BN, loads[MODE], NW == 8 ? "8w" : "", type_tag<TOut>(),
              g.ksplit == 2 ? "_ksplit2" : g.ksplit == 3 ? "_ksplit3" : g.ksplit == 4 ? "_ksplit4" : "");
     note_kernel(name);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, g);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, st, g);
     return check_hip(hipGetLastError(), name);
 }
 
@@ -994,7 +1016,11 @@ static int launch_tiles(const GemmArgs& g, TileCfg t, int mode, int grid, hipStr
     if (t.bm == 128 && t.bn == 256) return MMX_LAUNCH_MODES(TIn, 128, 256, TOut);
     if (t.bm == 128 && t.bn == 128) return MMX_LAUNCH_MODES(TIn, 128, 128, TOut);
     if constexpr (!Mfma<TIn>::W8) {  // (int8 weights under bf16 A come in tiles of 128 or 256 columns)
-        if (t.bm == 256 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 256, 192, TOut);
+        if (t.bm == 256 && t.bn == 192) {
+            // two waves per SIMD, half the accumulator block each (ring pipeline, no K split)
+            if (wave_count() == 8 && mode == 2 && g.ksplit == 1) return launch_cfg<TIn, 256, 192, 2, TOut, 1, 8>(g, grid, st);
+            return MMX_LAUNCH_MODES(TIn, 256, 192, TOut);
+        }
         if (t.bm == 128 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 128, 192, TOut);
         if (t.bm == 128 && t.bn == 64 && mode == 2 && g.ksplit == 1) return MMX_LAUNCH(TIn, 128, 64, 2, TOut, 1);  // ring pipeline only
     }
