@@ -205,7 +205,11 @@ const char* mmx_last_kernel(void);
  * loads use a masked kernel whatever this is set to.  "decode_halves": whether the streaming decode
  * kernel for M <= 4 splits every 32-column panel over two workgroups — -1 (default) where that fills the
  * CUs better, 0 never, 1 always while x takes at most 46 KiB of LDS (the two forms add the partial sums in
- * different orders). */
+ * different orders).  "waves": 8 (default) lets the 256x192 tile kernel run as eight wavefronts per
+ * workgroup, 4 keeps the four-wavefront form (same results).  "decode_valu": whether the
+ * streaming decode kernel at M = 1 over int8-compressed weights uses v_dot2_f32_bf16 and a cross-lane add
+ * instead of the matrix cores — -1 (default) where at most one workgroup per CU is launched (it is the faster form
+ * there), 0 never, 1 always; the two forms agree to fp32 summation order. */
 int mmx_set_option(const char* name, int value);  /* like mmx_set_tile: affects the calling thread's later calls only */
 /* HIP-event timing of `iters` back-to-back launches of the given gemm on `stream`, launch i
  * using the packed weights Bpacked_rot[i % n_rot] (rotate over several copies so that a

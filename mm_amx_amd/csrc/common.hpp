@@ -11,6 +11,7 @@
 namespace mmx {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 typedef __attribute__((__vector_size__(4 * sizeof(int)))) int i32x4;

@@ -961,7 +961,10 @@ static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, bool w
                 if (rq.k_splits == 0 && (tiles * S > cus || kq < 8)) continue;
             }
             const int kit = S > 1 ? slice_kiters(nk, S) : nk;
-            const float mfma = (float)(c.bm * c.bn / 32) / c.eff, bytes = (float)((c.bm + c.bn) * 128) / l1_bytes_per_clk;
+            // int8 weights under bf16 A: every wave converts its own fragments, 12 vector instructions per MFMA operand,
+            // which a small block per wave cannot hide behind its MFMAs (measured issue efficiencies)
+            const float eff = !wide_only ? c.eff : (c.bm == 256 ? 0.80f : (c.bn == 256 ? 0.50f : 0.42f));
+            const float mfma = (float)(c.bm * c.bn / 32) / eff, bytes = (float)((c.bm + c.bn) * 128) / l1_bytes_per_clk;
             const float loop = (float)kit * (mfma > bytes ? mfma : bytes);
             const float epi = (float)(c.bm * c.bn / 256) * 100.0f;  // between a plain store (45) and a GELU (170): the plan must
                                                                    // not depend on the post-op, or a GEMM and its fused form would sum differently

@@ -526,6 +526,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 template <int WK, int NP, bool ONE>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void skinny_stream_kernel(const SkinnyArgs s, int zero_off) {
     constexpr bool W8 = WK == 1, W4 = WK == 2, I8A = WK == 3;  // 3: int8 weights AND int8 activations, int32 sums
+    // 4: int8 weights and ONE row of x without the matrix cores: every lane owns one column and half of a fragment's
+    // k, v_dot2_f32_bf16 on the converted pairs, and one cross-lane add at the end.  Kept as the measured
+    // counterpart of WK = 1 (option "decode_valu"); the post-op is the same code.
+    constexpr bool W8V = WK == 4, VALU = W8V;
+    static_assert(!VALU || NP == 1, "the VALU form is a single-panel kernel");
     using accv = std::conditional_t<I8A, i32x16, f32x16>;
     // fragments per panel per wave in flight at once (16 KiB of weights; int4: 8 KiB, a fragment holds 64 of k
     // and unpacking it costs more than streaming it)
@@ -564,6 +569,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     __builtin_amdgcn_sched_barrier(0);
 
     accv acc[NP];
+    float vacc[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // VALU form: four independent chains per lane
 #pragma unroll
     for (int p = 0; p < NP; p++)
 #pragma unroll
@@ -582,7 +588,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         wbase[p] = s.Wp + (int64_t)panel * s.panel_stride + lane * 16;
     }
     const char* zrow = xs + zero_off;
-    const char* xrow = l32 < s.M ? xs + l32 * row_bytes : zrow;
+    const char* xrow = (VALU || l32 < s.M) ? xs + (VALU ? 0 : l32) * row_bytes : zrow;
     const int nbatch = (per_wave + U - 1) / U;  // same for every wave
     // U fragments per panel are in flight per wave at all times: register set u holds fragment u of a
     // batch and is re-requested for the next batch as soon as it has been multiplied
@@ -609,6 +615,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
                 const bf16x8 xq_ = *reinterpret_cast<const bf16x8*>(xr_ + (64 * fc_ + 32 * g32 + 8 * i_) * 2);  \
                 _Pragma("unroll") for (int p = 0; p < NP; p++)                                                  \
                     acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s4x8_to_bf16_div16(w[p][UU][i_]), xq_, acc[p], 0, 0, 0); \
+            }                                                                                                   \
+        } else if constexpr (W8V) {                                                                             \
+            const u32x4 xa_ = *reinterpret_cast<const u32x4*>(xr_ + (32 * fc_ + 16 * g32) * 2);                 \
+            const u32x4 xb_ = *reinterpret_cast<const u32x4*>(xr_ + (32 * fc_ + 16 * g32 + 8) * 2);             \
+            const u32x4 wa_ = __builtin_bit_cast(u32x4, s8x8_to_bf16(w[0][UU].x, w[0][UU].y));                  \
+            const u32x4 wb_ = __builtin_bit_cast(u32x4, s8x8_to_bf16(w[0][UU].z, w[0][UU].w));                  \
+            _Pragma("unroll") for (int i_ = 0; i_ < 4; i_++) {                                                  \
+                const uint32_t wa1_ = wa_[i_], xa1_ = xa_[i_], wb1_ = wb_[i_], xb1_ = xb_[i_];                  \
+                vacc[i_] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, wa1_), __builtin_bit_cast(bf16x2, xa1_), vacc[i_], false); \
+                vacc[i_] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, wb1_), __builtin_bit_cast(bf16x2, xb1_), vacc[i_], false); \
             }                                                                                                   \
         } else if constexpr (W8) {                                                                              \
             const bf16x8 xa_ = *reinterpret_cast<const bf16x8*>(xr_ + (32 * fc_ + 16 * g32) * 2);               \
@@ -655,13 +671,21 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #undef MMX_MULTIPLY
 
     __syncthreads();  // every wave has read its last x: the buffer becomes the reduction scratch
+    if constexpr (VALU) {
+        // lane (column l32, k half g32): add the other half's sum, then put the column's value where the
+        // matrix-core form would hold it (output row 0 of a 32x32 block), so that the post-op below is shared
+        float sum = (vacc[0] + vacc[1]) + (vacc[2] + vacc[3]);
+        sum += __shfl_xor(sum, 32);
+        if (g32 == 0) red[wave][0][4 * (l32 >> 3) + (l32 & 3)][32 * ((l32 >> 2) & 1)] = sum;
+    } else {
 #pragma unroll
-    for (int p = 0; p < NP; p++)
+        for (int p = 0; p < NP; p++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            if constexpr (I8A) reinterpret_cast<int*>(&red[wave][p][v][lane])[0] = acc[p][v];  // the sums travel as bits
-            else red[wave][p][v][lane] = W4 ? acc[p][v] * 16.0f : acc[p][v];  // int4 operands were q / 16
-        }
+            for (int v = 0; v < 16; v++) {
+                if constexpr (I8A) reinterpret_cast<int*>(&red[wave][p][v][lane])[0] = acc[p][v];  // the sums travel as bits
+                else red[wave][p][v][lane] = W4 ? acc[p][v] * 16.0f : acc[p][v];  // int4 operands were q / 16
+            }
+    }
     __syncthreads();
     skinny_finish<NP, I8A>(s, red, panel_first, tid, fin);
 }
@@ -857,6 +881,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 }
 
 int decode_halves();
+int decode_valu();
 
 // int8 x int8 at M <= 32 can use the decode kernels if x is 16-byte aligned and K fills whole 128-byte groups of
 // the packed weights: the streaming form if x fits in LDS, else the chunked one, which walks K in chunks of 256
@@ -982,9 +1007,9 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         if (pairs && (panels & 1)) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
         note_kernel(pairs ? (w8 ? "skinny_stream_w8_gateup" : "skinny_stream_bf16_gateup") : (w8 ? "skinny_stream_w8" : "skinny_stream_bf16"));
         const int per_wave = (s.nfrag + 7) / 8;
-        // Half-panel workgroups pay off for up to 4 rows of x (cheap enough to stage per workgroup) if each still has at least
-        // 128 KiB of weights to stream (measured: 64 KiB units lose more to the fixed cost of a workgroup than the
-        // better balance gains) and the list is short enough for balance to matter: at most two rounds of resident
+        // Half-panel workgroups pay off for up to 4 rows of x (cheap enough to stage per workgroup) if each still has enough
+        // weights to stream (measured at M = 1: bf16 units of 80 KiB gain 8 %, of 64 KiB lose to the fixed cost of a
+        // workgroup; int8 units of 172 KiB gain 16 %, of 128 KiB lose 1 %, of 64 KiB 20 %) and the list is short enough for balance to matter: at most two rounds of resident
         // workgroups (four waves each; LDS allows min(4, 160 KiB / (reduction scratch + x)) per CU)
         const int units = pairs ? panels / 2 : panels;
         const int lds_wg = 16 * 1024 * (pairs ? 2 : 1) + xbytes;
@@ -992,7 +1017,7 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         const int64_t unit_bytes = (int64_t)s.nfrag * 512 * (pairs ? 2 : 1);
         const int force = decode_halves();  // -1: by the rule above, 0: never, 1: for every M <= 4 (tests pin the path with it)
         const bool halves = M <= 4 && !bigx && !(pairs && w8) && force != 0 &&
-                            (force == 1 || (2 * units <= 2 * num_cus() * wg_per_cu && unit_bytes >= 128 * 1024));
+                            (force == 1 || (2 * units <= 2 * num_cus() * wg_per_cu && unit_bytes >= (pairs ? 128 : (w8 ? 160 : 80)) * 1024));
         const int per_wave_h = ((s.nfrag >> 1) + 3) / 4;
 #define MMX_STREAM(W8, NP, GRID)                                                                                     \
     do {                                                                                                             \
@@ -1006,7 +1031,19 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
             hipLaunchKernelGGL((skinny_stream_kernel<W8, NP, false>), dim3(GRID), dim3(512), stream_lds_bytes(xbytes, NP), st, s, zero_off); \
     } while (0)
         if (halves) note_kernel(pairs ? "skinny_half_bf16_gateup" : (w8 ? "skinny_half_w8" : "skinny_half_bf16"));
-        if (pairs && w8) {
+        // One row of x over int8 weights: a lane can own a column and half of a fragment's k (v_dot2_f32_bf16, one
+        // cross-lane add), which costs half the issue cycles of a 32x32 MFMA that fills 31 unused rows.  It wins while a
+        // CU holds a single workgroup (no second one to hide the int8 conversion behind: 4096 x 4096 6.6 against 7.6 us,
+        // 4096 x 8192 8.4 against 8.8) and loses once two share a CU (4096 x 11008: 11.3 against 10.6 us).  With bf16
+        // weights there is no conversion and the two forms take the same time, so only this one exists.
+        // decode_valu(): -1 by that rule, 0 never, 1 always.
+        const int vforce = decode_valu();
+        const bool valu = w8 && M == 1 && !pairs && !halves && !bigx && vforce != 0 && (vforce == 1 || panels <= num_cus());
+        if (valu) {
+            note_kernel("skinny_stream_w8_valu");
+            if (per_wave <= 16) hipLaunchKernelGGL((skinny_stream_kernel<4, 1, true>), dim3(panels), dim3(512), stream_lds_bytes(xbytes, 1), st, s, zero_off);
+            else hipLaunchKernelGGL((skinny_stream_kernel<4, 1, false>), dim3(panels), dim3(512), stream_lds_bytes(xbytes, 1), st, s, zero_off);
+        } else if (pairs && w8) {
             if (per_wave <= 8) hipLaunchKernelGGL((skinny_stream_kernel<1, 2, true>), dim3(panels / 2), dim3(512), stream_lds_bytes(xbytes, 2), st, s, zero_off);
             else hipLaunchKernelGGL((skinny_stream_kernel<1, 2, false>), dim3(panels / 2), dim3(512), stream_lds_bytes(xbytes, 2), st, s, zero_off);
         } else if (pairs) MMX_STREAM(false, 2, panels / 2);

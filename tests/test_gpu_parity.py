@@ -346,6 +346,52 @@ def test_decode_half_panel_form(po, shape, w8):
     assert np.linalg.norm(a - b) <= 1e-5 * np.linalg.norm(b)
 
 
+# One row of x over int8 weights without the matrix cores (v_dot2_f32_bf16 per lane + a cross-lane add): same sums
+# up to fp32 order, the post-op is the shared code, so the fused result equals the oracle's post-op on the GPU's own sums.
+# Shapes: a single batch per wave and the rolling window, ragged N, a column range, K of the long down projection.
+@pytest.mark.parametrize("shape", [(256, 64), (4096, 352), (4096, 4096), (11008, 160), (8192, 100), (2560, 10240)])
+@pytest.mark.parametrize("out", ["f32", "bf16", "i8"])
+def test_decode_valu_form(po, shape, out):
+    K, N = shape
+    if out != "f32" and K * N > 4096 * 352:
+        pytest.skip("the large shapes with the fp32 store only")
+    rng = np.random.default_rng(11 * sum(shape))
+    x = rand_bf16(rng, (1, K), 1.0)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    W = np.clip(np.rint(rng.standard_normal((K, N)) * 40), -127, 127).astype(np.int8)
+    scale = rng.uniform(1e-3, 5e-3, N).astype(np.float32)
+    _, acc_ref = po.gemv_w8(x, W, scale, want_acc=True)
+    packed = mx.repack_b(dev(W))
+    steps = mx.PP_DEQUANT | mx.PP_BIAS | mx.PP_GELU | (mx.PP_QUANT if out == "i8" else 0)
+    tdt, odt = {"f32": (torch.float32, po.F32), "bf16": (torch.bfloat16, po.BF16), "i8": (torch.int8, po.I8)}[out]
+    n0, n1 = (32, N - 5) if N > 96 and N < 4096 else (0, N)
+    res = {}
+    try:
+        for valu in (1, 0):
+            mx.set_option("decode_valu", valu)
+            mx.set_option("decode_halves", 0)
+            y = torch.full((1, N), 7, dtype=tdt, device="cuda")
+            mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, steps, bias=dev(bias), deq_scale_per_oc=dev(scale), q_scale=20.0),
+                    n0=n0, n1=n1, b_dtype=mx.I8)
+            assert ("valu" in mx.last_kernel()) == (valu == 1), mx.last_kernel()
+            acc = torch.zeros((1, N), dtype=torch.float32, device="cuda")
+            mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc, mx.PP_NONE), b_dtype=mx.I8)
+            assert ("valu" in mx.last_kernel()) == (valu == 1), mx.last_kernel()
+            res[valu] = (host_bits(y), host_bits(acc))
+    finally:
+        mx.set_option("decode_valu", -1)
+        mx.set_option("decode_halves", -1)
+    posteps = po.PP_DEQUANT | po.PP_BIAS | po.PP_GELU | (po.PP_QUANT if out == "i8" else 0)
+    for valu, (got, acc) in res.items():
+        check_float_parity(acc, acc_ref, f"accumulators {shape} valu={valu}")
+        again = po.pp(acc, posteps, odt, bias=bias, deq_per_oc=scale, q=20.0)
+        assert np.array_equal(got[:, n0:n1], again[:, n0:n1]), f"valu={valu}"
+        fill = host_bits(torch.full((1, 1), 7, dtype=tdt, device="cuda"))[0, 0]
+        assert np.all(got[:, :n0] == fill) and np.all(got[:, n1:] == fill)   # nothing outside the range is written
+    a, b = res[1][1].astype(np.float64), res[0][1].astype(np.float64)
+    assert np.linalg.norm(a - b) <= 1e-5 * np.linalg.norm(b)
+
+
 # 2-4 rows of a long x (the MLP's down projection: K = 11008) still go whole into LDS for the half-panel form when
 # there is at most one half-panel per CU; "decode_halves" = 0 gives the per-lane form to compare with
 @pytest.mark.parametrize("shape", [(2, 11008, 256), (3, 11008, 100), (4, 11008, 4096), (4, 8192, 160)])
