@@ -33,9 +33,9 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # when the kernel that ran is the one profiled AND its source is the one that was profiled (first 16 hex digits of
 # the SHA-256 of the kernel's source file): after a change of the kernel the figure reads null until it is re-measured.
 MEASURED_TRAFFIC = {
-    "gemm_bf16_256x192_ring_out_bf16": {"bytes": (81969 * 2.000 + 27915 * 1.000) * 1024, "source": "mm_amx_amd/csrc/gemm_tile.hpp",
-                                        "sha": "@GEMM_SHA@"},
-    "skinny_stream_w8": {"bytes": 22174 * 2.000 * 1024 + 22 * 1.000 * 1024, "source": "mm_amx_amd/csrc/skinny.hip", "sha": "@SKINNY_SHA@"},
+    "gemm_bf16_256x192_ring8w_out_bf16": {"bytes": (81715.7 * 2.000 + 27523.7 * 1.000) * 1024, "source": "mm_amx_amd/csrc/gemm_tile.hpp",
+                                          "sha": "ecd456f5b7103bb4"},
+    "skinny_stream_w8": {"bytes": (22175 * 2.000 + 49 * 1.000) * 1024, "source": "mm_amx_amd/csrc/skinny.hip", "sha": "5d55891ec393aa12"},
 }
 
 
@@ -130,15 +130,18 @@ def main():
     kernel_name = mx.last_kernel()
     value = flops / (ms_per_step * 1e-3) / 1e12
     achieved = flops / (kernel_ms * 1e-3) / 1e12
-    # the same launches once more with an event between every two of them: the median launch (not part of `value`)
-    evs = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    # the same launches once more in chunks of ten with an event between the chunks: the median chunk mean (not part
+    # of `value`; an event between every two launches would add its own gap to each of them)
+    nchunk = max(1, args.steps // 10)
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(nchunk + 1)]
     evs[0].record()
-    for i in range(args.steps):
-        step()
+    for i in range(nchunk):
+        for _ in range(10):
+            step()
         evs[i + 1].record()
     torch.cuda.synchronize()
-    per_launch = sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(args.steps))
-    kernel_median_ms = per_launch[len(per_launch) // 2]
+    per_chunk = sorted(evs[i].elapsed_time(evs[i + 1]) / 10 for i in range(nchunk))
+    kernel_median_ms = per_chunk[len(per_chunk) // 2]
 
     out = {
         "metric": "bf16 FC GEMM TFLOP/s (M=1024, K=4096, N=11008, fused BIAS+GELU, bf16 out)",
@@ -313,6 +316,31 @@ def main():
             del As, Cs
         extra["bf16_fc_bias_gelu_sweep_M"] = sweep
 
+        # The headline FC launched alternately on two streams (independent requests, separate outputs): a launch of
+        # 232 workgroups leaves 24 CUs idle and successive launches on one stream are ~5 us apart; two streams let the
+        # next launch start on the idle CUs.  Throughput only - a launch on its own is not faster this way.
+        s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+        C2 = torch.zeros_like(C)
+        ep_2 = mx.Epilogue(C2, mx.PP_BIAS | mx.PP_GELU, bias=bias)
+
+        def pair():
+            with torch.cuda.stream(s1):
+                mx.gemm(A, Bp, N, ep)
+            with torch.cuda.stream(s2):
+                mx.gemm(A, Bp, N, ep_2)
+        torch.cuda.synchronize()
+        for _ in range(50):
+            pair()
+        torch.cuda.synchronize()
+        tp0 = time.perf_counter()
+        for _ in range(100):
+            pair()
+        torch.cuda.synchronize()
+        us2 = (time.perf_counter() - tp0) * 1e6 / 200
+        extra["bf16_fc_bias_gelu_M1024_two_streams"] = {"us_per_launch": round(us2, 2), "tflops": round(flops / us2 / 1e6, 1),
+                                                        "frac_of_bf16_peak": round(flops / us2 / 1e6 / PEAK_BF16_TFLOPS, 4)}
+        del C2
+
         # int8 FC with dequant/bias/requant
         wi = wl.int8_fc()
         Ai, Bi = dev(wi["A"]), mx.repack_b(dev(wi["B"]))
@@ -354,8 +382,83 @@ def main():
                              "weight_GBps": round(wbytes / ms / 1e6, 0),
                              "frac_of_hbm_peak": round(wbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "kernel": mx.last_kernel(),
                              "traffic": measured_traffic(mx.last_kernel()) if Mg == 1 else None, "algorithmic_bytes": wbytes}
+            if Mg == 1:
+                # the same launch in its other form (matrix cores <-> v_dot2_f32_bf16 per lane), for the record
+                auto_valu = "valu" in mx.last_kernel()
+                mx.set_option("decode_valu", 0 if auto_valu else 1)
+                try:
+                    ms2 = avg_ms(xg, packs, wg["N"], epg, 240, b_dtype=mx.I8)
+                    gemv["1"]["other_form"] = {"us": round(ms2 * 1e3, 2), "kernel": mx.last_kernel()}
+                finally:
+                    mx.set_option("decode_valu", -1)
             del packs, Wg
         extra["decode_gemv_int8w_K4096_N11008"] = gemv
+
+        # The same GEMV (M=1) over the number of output columns, in each of its forms: per-launch cost and rate, and
+        # what the balance of 32-column panels over 256 CUs is worth (N = 8192 and 16384 are exactly 1 and 2 panels per CU)
+        sweepn = {}
+        xg1 = torch.randn((1, 4096), dtype=torch.float32, device="cuda").to(torch.bfloat16)
+        for Nn in (4096, 8192, 11008, 16384, 32768):
+            ncopy = max(2, int(540e6 // (4096 * Nn)))
+            Wn = mx.repack_b(torch.randint(-127, 128, (4096, Nn), dtype=torch.int8, device="cuda"))
+            packs = [Wn] + [Wn.clone() for _ in range(ncopy - 1)]
+            yn = torch.zeros((1, Nn), dtype=torch.bfloat16, device="cuda")
+            epn = mx.Epilogue(yn, mx.PP_DEQUANT, deq_scale=1e-3)
+            ent = {}
+            for form, (valu, halves) in (("mfma", (0, 0)), ("valu", (1, 0)), ("half_panels", (0, 1)), ("auto", (-1, -1))):
+                mx.set_option("decode_valu", valu)
+                mx.set_option("decode_halves", halves)
+                try:
+                    msn = avg_ms(xg1, packs, Nn, epn, 200, b_dtype=mx.I8)
+                    ent[form] = {"us": round(msn * 1e3, 2), "kernel": mx.last_kernel()}
+                finally:
+                    mx.set_option("decode_valu", -1)
+                    mx.set_option("decode_halves", -1)
+            ent["panels_per_cu"] = round(Nn / 32 / 256, 2)
+            ent["auto_weight_GBps"] = round(4096.0 * Nn / ent["auto"]["us"] / 1e3, 0)
+            sweepn[str(Nn)] = ent
+            del packs, Wn
+        extra["decode_gemv_int8w_K4096_M1_sweep_N"] = sweepn
+
+        # Steady state of a chain of decode layers (the topology of main.cpp:660-711: A1 x B1 -> A2, A2 x B2 -> A1, ...,
+        # one set of weights per layer): 12 pairs of [1,4096] x [4096,11008] and [1,11008] x [11008,4096] over int8
+        # weights (1.08 GB, nothing repeats within the cache), every layer reading the previous layer's output,
+        # replayed from a HIP graph so that no host time is in the figure
+        Kc, Nc, pairs = 4096, 11008, 12
+        rngc = torch.Generator(device="cuda").manual_seed(5)
+        W1 = [mx.repack_b(torch.randint(-127, 128, (Kc, Nc), dtype=torch.int8, device="cuda", generator=rngc)) for _ in range(pairs)]
+        W2 = [mx.repack_b(torch.randint(-127, 128, (Nc, Kc), dtype=torch.int8, device="cuda", generator=rngc)) for _ in range(pairs)]
+        xa = torch.randn((1, Kc), dtype=torch.float32, device="cuda").to(torch.bfloat16)
+        hb = torch.zeros((1, Nc), dtype=torch.bfloat16, device="cuda")
+        ep1, ep2 = mx.Epilogue(hb, mx.PP_DEQUANT, deq_scale=2e-4), mx.Epilogue(xa, mx.PP_DEQUANT, deq_scale=2e-4)
+
+        def chain():
+            for i in range(pairs):
+                mx.gemm(xa, W1[i], Nc, ep1, b_dtype=mx.I8)
+                mx.gemm(hb, W2[i], Kc, ep2, b_dtype=mx.I8)
+        cstream = torch.cuda.Stream()
+        with torch.cuda.stream(cstream):
+            chain()
+            torch.cuda.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr, stream=cstream):
+                chain()
+        torch.cuda.synchronize()
+        reps = []
+        for _ in range(12):
+            a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a0.record()
+            gr.replay()
+            a1.record()
+            torch.cuda.synchronize()
+            reps.append(a0.elapsed_time(a1) * 1e3 / (2 * pairs))
+        reps = sorted(reps[2:])
+        us = reps[len(reps) // 2]
+        extra["decode_chain_int8w_24_layers_K4096_N11008"] = {
+            "us_per_layer": round(us, 2), "weight_GBps": round(float(Kc) * Nc / us / 1e3, 0),
+            "frac_of_hbm_peak": round(float(Kc) * Nc / us / 1e3 / PEAK_HBM_GBS, 4), "layers": 2 * pairs,
+            "note": "graph replay, M=1, each layer reads the previous layer's output; median of 10 replays"}
+        del gr, W1, W2
 
         # int8 activations x int8 weights at M=1 (int32 sums), same weights and rotation
         w8b = wl.decode_gemv_w8(M=1)

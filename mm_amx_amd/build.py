@@ -1,9 +1,11 @@
 """Builds libmm_amx_amd.so (HIP kernels + C ABI) in-tree for gfx950 with hipcc.
 
-    python -m mm_amx_amd.build [--incremental]
+    python -m mm_amx_amd.build [--incremental] [--stamps]
 
 By default every source is compiled again; --incremental keeps the object files of earlier runs and
-recompiles only what is older than its source or than a header.
+recompiles only what is older than its source or than a header.  --stamps builds a second library,
+libmm_amx_amd_stamps.so, whose tile kernels record the shader clock at the phase boundaries of every
+workgroup (-DMMX_STAMPS; read by mm_amx_amd.phase_stamps); the shipped library holds no such code.
 """
 import os
 import subprocess
@@ -35,8 +37,10 @@ def _stale(obj, src):
     return any(os.path.getmtime(d) > t for d in deps)
 
 
-def build(verbose=False, incremental=False):
-    objs = [os.path.join(CSRC, src.replace(".hip", ".o")) for src in SOURCES]
+def build(verbose=False, incremental=False, stamps=False):
+    lib = LIB.replace(".so", "_stamps.so") if stamps else LIB
+    flags = FLAGS + (["-DMMX_STAMPS"] if stamps else [])
+    objs = [os.path.join(CSRC, src.replace(".hip", ".stamps.o" if stamps else ".o")) for src in SOURCES]
     todo = [(src, obj) for src, obj in zip(SOURCES, objs)
             if not incremental or _stale(obj, os.path.join(CSRC, src))]
     failed = False
@@ -55,7 +59,7 @@ def build(verbose=False, incremental=False):
     for src, obj in todo:
         while len(running) >= JOBS:
             reap(*running.pop(0))
-        cmd = ["hipcc"] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = ["hipcc"] + flags + ["-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         running.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
@@ -63,12 +67,12 @@ def build(verbose=False, incremental=False):
         reap(*item)
     if failed:
         raise RuntimeError("hipcc failed")
-    subprocess.check_call(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
+    subprocess.check_call(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs)
     if not incremental:
         for obj in objs:
             os.remove(obj)
-    return LIB
+    return lib
 
 
 if __name__ == "__main__":
-    print(build(verbose=True, incremental="--incremental" in sys.argv[1:]))
+    print(build(verbose=True, incremental="--incremental" in sys.argv[1:], stamps="--stamps" in sys.argv[1:]))

@@ -1,0 +1,100 @@
+"""Per-workgroup phase timings of the MFMA tile kernels, from the instrumented build.
+
+    python -m mm_amx_amd.build --stamps
+    python -m mm_amx_amd.phase_stamps bf16,1024,4096,11008,256x192,1,8 i8,512,4096,4096,128x64,1
+
+Each argument is  dtype,M,K,N,tile,k_splits[,waves]  (dtype bf16: the FC with BIAS+GELU and a bf16 store; i8: the int8 FC
+with DEQUANT+BIAS+QUANT and an int8 store; tile as for mmx_set_tile, empty = the library's choice; waves 4 or 8).
+The instrumented library (libmm_amx_amd_stamps.so, -DMMX_STAMPS) makes thread 0 of every workgroup write the shader
+clock at its phase boundaries behind the K-split workspace; this module launches the shape, reads the stamps back and
+prints medians over the workgroups: cycles from start to the first data in LDS, of the main loop, of parking and
+combining K slices, of the epilogue, and the clock (cycles per wall-clock tick).  The shipped library has no stamps;
+the instrumented one runs the same code plus eight 8-byte stores per workgroup.
+"""
+import os
+import sys
+
+import numpy as np
+import torch
+
+import mm_amx_amd as mx
+from mm_amx_amd import _lib
+
+# the library is loaded on first use: point the binding at the instrumented build before that
+if "MMX_LIB_PATH" not in os.environ:
+    _lib._LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmm_amx_amd_stamps.so")
+
+STAMP_OFFSET = 96 << 20          # the kernels write at workspace partials + 96 MiB + 64 * unit index
+COUNTER_BYTES = 16 << 10
+STAMP_BYTES = 1 << 20
+
+
+def run(ws, dt, M, K, N, tile, S, waves=8, out=sys.stdout):
+    mx.set_option("waves", waves)
+    if dt == "i8":
+        A = torch.randint(-127, 128, (M, K), dtype=torch.int8, device="cuda")
+        Bp = mx.repack_b(torch.randint(-127, 128, (K, N), dtype=torch.int8, device="cuda"))
+        C = torch.zeros((M, N), dtype=torch.int8, device="cuda")
+        ep = mx.Epilogue(C, mx.PP_DEQUANT | mx.PP_BIAS | mx.PP_QUANT, bias=torch.zeros(N, device="cuda"),
+                         deq_scale_per_oc=torch.full((N,), 1e-4, device="cuda"), q_scale=20.0)
+    else:
+        A = torch.randn((M, K), device="cuda").to(torch.bfloat16)
+        Bp = mx.repack_b((torch.randn((K, N), device="cuda") * 0.02).to(torch.bfloat16))
+        C = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+        ep = mx.Epilogue(C, mx.PP_BIAS | mx.PP_GELU, bias=torch.zeros(N, device="cuda"))
+    stamp_off = COUNTER_BYTES + STAMP_OFFSET
+    mx.set_tile(tile)
+    try:
+        mx.time_gemm(A, [Bp], N, ep, 100, k_splits=S, ws=ws)
+        ms = mx.time_gemm(A, [Bp], N, ep, 100, k_splits=S, ws=ws)
+        torch.cuda.synchronize()
+        ws[stamp_off:].zero_()
+        for _ in range(3):
+            mx.gemm(A, Bp, N, ep, k_splits=S, ws=ws)
+        torch.cuda.synchronize()
+        kern = mx.last_kernel()
+    finally:
+        mx.set_tile("")
+        mx.set_option("waves", 8)
+    st = ws[stamp_off:].view(torch.int64).cpu().numpy().reshape(-1, 8)
+    st = st[st[:, 0] != 0]
+    fin = st[st[:, 7] != 0]               # workgroups that ran an epilogue (with a K split: the last to arrive at their tile)
+    rt0 = st[:, 0].min()
+    wall_us = (fin[:, 7] - fin[:, 0]) / 100.0   # 100 MHz wall-clock ticks
+    ghz = np.median((fin[:, 5] - fin[:, 1]) / wall_us) / 1e3
+
+    def ph(a, b, rows=fin):
+        rows = rows[(rows[:, a] != 0) & (rows[:, b] != 0)]   # a workgroup that skipped a phase left its stamp at zero
+        if not len(rows):
+            return "       -"
+        d = rows[:, b] - rows[:, a]
+        return f"{np.median(d):8.0f} ({d.min():.0f}..{d.max():.0f})"
+    print(f"== {dt} {M}x{K}x{N} {kern}: {ms * 1e3:.2f} us/launch, {len(st)} workgroups, {len(fin)} with an epilogue, "
+          f"clock ~{ghz:.2f} GHz", file=out)
+    print(f"   workgroup life us: median {np.median(wall_us):.2f} max {wall_us.max():.2f}; last end "
+          f"{(fin[:, 7].max() - rt0) / 100.0:.2f} us after the first start", file=out)
+    line = f"   cycles, median (min..max): start->first data {ph(1, 2)}   main loop {ph(2, 3)}   "
+    if S > 1:
+        line += f"park+count {ph(3, 4)}   combine+epilogue {ph(4, 5)}"
+        parked = st[(st[:, 6] != 0) & (st[:, 3] != 0)]
+        if len(parked):
+            d = parked[:, 6] - parked[:, 3]
+            line += f"\n   parked slices: {len(parked)}, park+count {np.median(d):.0f} ({d.min():.0f}..{d.max():.0f})"
+    else:
+        line += f"epilogue {ph(3, 5)}"
+    print(line, file=out, flush=True)
+
+
+def main(argv):
+    if "stamps" not in os.path.basename(mx.lib_path()):
+        sys.exit("phase_stamps: the instrumented library is needed (python -m mm_amx_amd.build --stamps)")
+    mx.init(0)
+    ws = torch.zeros(COUNTER_BYTES + STAMP_OFFSET + STAMP_BYTES, dtype=torch.uint8, device="cuda")
+    for a in argv:
+        parts = a.split(",")
+        dt, M, K, N, tile, S = parts[:6]
+        run(ws, dt, int(M), int(K), int(N), tile, int(S), waves=int(parts[6]) if len(parts) > 6 else 8)
+
+
+if __name__ == "__main__":
+    main(sys.argv[1:])

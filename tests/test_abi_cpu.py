@@ -208,3 +208,14 @@ def test_tuning_knobs_are_per_thread(lib):
     t1.start(), t2.start(), t1.join(), t2.join()
     assert seen["good"][0] == 0 and seen["bad"][0] == -1 and b"17x3" in seen["bad"][1]
     assert b"17x3" not in lib.mmx_last_error()  # this thread's error string is its own
+
+
+def test_bench_traffic_figures_belong_to_the_current_kernel_sources():
+    """bench.py reports a measured HBM traffic only for the kernel source it was measured on (keyed by a hash of the
+    file): after a change of such a file the figure has to be measured again, or the bench reports null."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_for_test", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    for kernel in bench.MEASURED_TRAFFIC:
+        assert bench.measured_traffic(kernel) is not None, f"{kernel}: its source changed after the traffic was measured"
