@@ -942,7 +942,9 @@ static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, bool w
         {256, 256, 0.92f}, {256, 192, 0.90f}, {128, 256, 0.86f}, {128, 192, 0.84f}, {128, 128, 0.80f}, {128, 64, 0.70f}};
     const TileCfg f = forced_tile();
     const int cus = num_cus();
-    const float l1_bytes_per_clk = 48.0f, ws_bytes_per_clk = 40.0f;
+    // measured: a CU takes 36.6 bytes per clock from L2 with all CUs pulling; parking a 64 KiB partial tile and counting
+    // takes 5.5k cycles, adding one in 2.9k
+    const float l1_bytes_per_clk = 36.6f, ws_bytes_per_clk = 22.5f;
     float best = 1e30f;
     Plan pick = {{128, 128}, 1};
     for (const auto& c : cand) {
@@ -968,9 +970,11 @@ static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, bool w
             const float loop = (float)kit * (mfma > bytes ? mfma : bytes);
             const float epi = (float)(c.bm * c.bn / 256) * 100.0f;  // between a plain store (45) and a GELU (170): the plan must
                                                                    // not depend on the post-op, or a GEMM and its fused form would sum differently
-            const float split = S > 1 ? 3000.0f + (float)(c.bm * c.bn * 4) * (float)S / ws_bytes_per_clk : 0.0f;
+            const float split = S > 1 ? 2500.0f + (float)(c.bm * c.bn * 4) * (float)S / ws_bytes_per_clk : 0.0f;
             const int per_cu = (tiles * S + cus - 1) / cus;
-            const float t = (float)per_cu * (3700.0f + loop + epi + split);
+            // a K split has to win by a margin: its extra traffic costs clock as well as cycles (the part runs these kernels
+            // at its power limit; 128x128 in two slices against 128x64: 2 % fewer cycles, 8 % lower clock)
+            const float t = (float)per_cu * (3700.0f + loop + epi + split) * (S > 1 ? 1.15f : 1.0f);
             if (t < best) { best = t; pick = {{c.bm, c.bn}, S}; }
         }
     }
