@@ -149,7 +149,11 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "llama7b_ffn_up_bf16_bias_gelu", "M": M, "K": K, "N": N, "kernel": kernel_name,
-                   "inputs": "A~N(0,1) bf16, B~N(0,0.02) bf16 repacked once, bias~N(0,0.1) fp32, all resident in HBM"},
+                   "inputs": "A~N(0,1) bf16, B~N(0,0.02) bf16 repacked once, bias~N(0,0.1) fp32, all resident in HBM",
+                   "parity": "vs the CPU oracle at this size: relative Frobenius <= 1e-3; 99.87 % of all elements within 1 bf16 ulp "
+                             "(the stated bar is 99.9 %: met where the pre-activation is > -3.5, 99.99 %; below it GELU's bracket cancels and "
+                             "one fp32 ulp of summation order moves a bf16 ulp); the fused epilogue equals the oracle's bit for bit on the "
+                             "GPU's own accumulators (tests/test_gpu_parity.py::test_ffn_up_bias_gelu_full_size)"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                      "traffic": measured_traffic(kernel_name),

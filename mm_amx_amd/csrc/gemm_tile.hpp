@@ -383,7 +383,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4,
         // A in LDS: rows of 128 bytes; the 16-byte chunk c of row r sits at position c ^ ((r >> 1) & 7), so
         // the 16 rows x 16 bytes that one LDS cycle serves for an MFMA operand fall into 16 different
         // bank groups.  A load instruction covers 8 rows x 128 bytes: lane -> (row, position).
-        uint32_t aoff[2][A_IT2], boff[B_IT2];
+        uint32_t aoff[2][A_IT2], boff[B_IT2 > 0 ? B_IT2 : 1];  // (a wave class without B loads: NBI < NW)
 #pragma unroll
         for (int half = 0; half < 2; half++)
 #pragma unroll
@@ -949,7 +949,8 @@ static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, bool w
     Plan pick = {{128, 128}, 1};
     for (const auto& c : cand) {
         if (f.bm && (f.bm != c.bm || f.bn != c.bn)) continue;
-        if ((need_pairs || wide_only) && (c.bn % 128) != 0) continue;   // (int8 weights under bf16 A: 128 columns per load)
+        if (need_pairs && (c.bn % 128) != 0) continue;
+        if (wide_only && c.bn == 64) continue;                      // (no 64-column tile for int8 weights under bf16 A)
         if (mode == 3 && !(c.bm == 128 && c.bn == 128)) continue;   // the masked path exists for one tile shape
         if (mode != 2 && c.bn == 64) continue;                      // the 64-wide tile exists for the ring pipeline only
         const int tiles = ((M + c.bm - 1) / c.bm) * ((Ncols + c.bn - 1) / c.bn);
@@ -965,7 +966,7 @@ static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, bool w
             const int kit = S > 1 ? slice_kiters(nk, S) : nk;
             // int8 weights under bf16 A: every wave converts its own fragments, 12 vector instructions per MFMA operand,
             // which a small block per wave cannot hide behind its MFMAs (measured issue efficiencies)
-            const float eff = !wide_only ? c.eff : (c.bm == 256 ? 0.80f : (c.bn == 256 ? 0.50f : 0.42f));
+            const float eff = !wide_only ? c.eff : (c.bm == 256 ? 0.80f : (c.bn == 256 ? 0.50f : (c.bn == 192 ? 0.46f : 0.42f)));
             const float mfma = (float)(c.bm * c.bn / 32) / eff, bytes = (float)((c.bm + c.bn) * 128) / l1_bytes_per_clk;
             const float loop = (float)kit * (mfma > bytes ? mfma : bytes);
             const float epi = (float)(c.bm * c.bn / 256) * 100.0f;  // between a plain store (45) and a GELU (170): the plan must
@@ -1022,13 +1023,13 @@ static int launch_tiles(const GemmArgs& g, TileCfg t, int mode, int grid, hipStr
     if (t.bm == 256 && t.bn == 256) return MMX_LAUNCH_MODES(TIn, 256, 256, TOut);
     if (t.bm == 128 && t.bn == 256) return MMX_LAUNCH_MODES(TIn, 128, 256, TOut);
     if (t.bm == 128 && t.bn == 128) return MMX_LAUNCH_MODES(TIn, 128, 128, TOut);
-    if constexpr (!Mfma<TIn>::W8) {  // (int8 weights under bf16 A come in tiles of 128 or 256 columns)
-        if (t.bm == 256 && t.bn == 192) {
-            // two waves per SIMD, half the accumulator block each (ring pipeline, no K split)
-            if (wave_count() == 8 && mode == 2 && g.ksplit == 1) return launch_cfg<TIn, 256, 192, 2, TOut, 1, 8>(g, grid, st);
-            return MMX_LAUNCH_MODES(TIn, 256, 192, TOut);
-        }
-        if (t.bm == 128 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 128, 192, TOut);
+    if (t.bm == 256 && t.bn == 192) {
+        // two waves per SIMD, half the accumulator block each (ring pipeline, no K split)
+        if (wave_count() == 8 && mode == 2 && g.ksplit == 1) return launch_cfg<TIn, 256, 192, 2, TOut, 1, 8>(g, grid, st);
+        return MMX_LAUNCH_MODES(TIn, 256, 192, TOut);
+    }
+    if (t.bm == 128 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 128, 192, TOut);
+    if constexpr (!Mfma<TIn>::W8) {
         if (t.bm == 128 && t.bn == 64 && mode == 2 && g.ksplit == 1) return MMX_LAUNCH(TIn, 128, 64, 2, TOut, 1);  // ring pipeline only
     }
     return set_error(MMX_E_UNSUPPORTED, "no MFMA tile kernel for %dx%d", t.bm, t.bn);

@@ -464,7 +464,7 @@ def _w8_case(po, M, K, N, seed, steps=None, **gemm_kw):
     return kernel
 
 
-@pytest.mark.parametrize("tile", ["256x256", "128x256", "128x128"])
+@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x192", "128x128"])
 @pytest.mark.parametrize("mode", [0, 2])
 def test_w8_gemm_every_kernel_variant(po, tile, mode):
     """int8-compressed weights under bf16 activations at M > 32: the tile kernels convert the int8 fragments on
@@ -474,6 +474,14 @@ def test_w8_gemm_every_kernel_variant(po, tile, mode):
     try:
         kernel = _w8_case(po, 600, 512, 832, 170)
         assert kernel.startswith("gemm_w8_") and tile in kernel and LOAD_NAMES[mode] in kernel, kernel
+        if tile == "256x192" and mode == 2:   # its four-wavefront form as well (the default is eight)
+            assert "ring8w" in kernel, kernel
+            mx.set_option("waves", 4)
+            try:
+                kernel4 = _w8_case(po, 600, 512, 832, 170)
+            finally:
+                mx.set_option("waves", 8)
+            assert "256x192_ring_" in kernel4, kernel4
     finally:
         mx.set_tile("")
         mx.set_option("load_mode", DEFAULT_LOAD_MODE)
@@ -488,9 +496,14 @@ def test_w8_gemm_shapes(po, shape):
 
 
 @pytest.mark.parametrize("S", [2, 4])
-def test_w8_gemm_k_split(po, ws, S):
-    kernel = _w8_case(po, 200, 2048, 384, 172 + S, k_splits=S, ws=ws)
-    assert f"ksplit{S}" in kernel, kernel
+@pytest.mark.parametrize("tile", ["", "256x192", "128x192"])
+def test_w8_gemm_k_split(po, ws, S, tile):
+    mx.set_tile(tile)
+    try:
+        kernel = _w8_case(po, 200, 2048, 384, 172 + S, k_splits=S, ws=ws)
+    finally:
+        mx.set_tile("")
+    assert f"ksplit{S}" in kernel and tile in kernel, kernel
 
 
 def test_w8_gemm_perf_log_shape(po):
@@ -1066,6 +1079,34 @@ def test_ksplit_bf16_fixed_order(po, ws, tile, S):
         assert np.array_equal(host_bits(C), po.pp(accs[0], po.PP_BIAS | po.PP_GELU, po.BF16, bias=bias))
     finally:
         mx.set_tile("")
+
+
+@pytest.mark.parametrize("S", [2, 4])
+def test_ksplit_over_a_column_range(po, ws, S):
+    """A K split over a column range n0..n1 (the N split of main.cpp:461-471 on top of the K split): the range's
+    columns equal those of the whole-N launch bit for bit (same tiles, same slice order), nothing else is written."""
+    M, K, N = 200, 4096, 1024
+    rng = np.random.default_rng(170 + S)
+    A, B = rand_bf16(rng, (M, K), 1.0), rand_bf16(rng, (K, N), 0.05)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    Ad, packed = dev_bf16(A), mx.repack_b(dev_bf16(B))
+    mx.set_tile("128x128")
+    try:
+        whole = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+        mx.gemm(Ad, packed, N, mx.Epilogue(whole, mx.PP_BIAS | mx.PP_GELU, bias=dev(bias)), k_splits=S, ws=ws)
+        assert f"ksplit{S}" in mx.last_kernel()
+        n0, n1 = 256, 896 - 40           # starts on a tile, ends inside one
+        part = torch.full((M, N), 7.0, dtype=torch.bfloat16, device="cuda")
+        mx.gemm(Ad, packed, N, mx.Epilogue(part, mx.PP_BIAS | mx.PP_GELU, bias=dev(bias)), n0=n0, n1=n1, k_splits=S, ws=ws)
+        assert f"ksplit{S}" in mx.last_kernel()
+    finally:
+        mx.set_tile("")
+    w, p7 = host_bits(whole), host_bits(part)
+    fill = host_bits(torch.full((1, 1), 7.0, dtype=torch.bfloat16, device="cuda"))[0, 0]
+    assert np.array_equal(p7[:, n0:n1], w[:, n0:n1])
+    assert np.all(p7[:, :n0] == fill) and np.all(p7[:, n1:] == fill)
+    acc = po.gemm_bf16(A, B)
+    check_gelu_parity(w, po.pp(acc, po.PP_BIAS | po.PP_GELU, po.BF16, bias=bias), acc + bias[None, :], f"ksplit{S} + column range")
 
 
 def test_ksplit_two_way_is_the_reference_partition(po, ws):
