@@ -4,7 +4,7 @@
     python -m mm_amx_amd.phase_stamps bf16,1024,4096,11008,256x192,1,8 i8,512,4096,4096,128x64,1
 
 Each argument is  dtype,M,K,N,tile,k_splits[,waves]  (dtype bf16: the FC with BIAS+GELU and a bf16 store; i8: the int8 FC
-with DEQUANT+BIAS+QUANT and an int8 store; tile as for mmx_set_tile, empty = the library's choice; waves 4 or 8).
+with DEQUANT+BIAS+QUANT and an int8 store; w8: bf16 activations on int8-compressed weights, DEQUANT, fp32 store; tile as for mmx_set_tile, empty = the library's choice; waves 4 or 8).
 The instrumented library (libmm_amx_amd_stamps.so, -DMMX_STAMPS) makes thread 0 of every workgroup write the shader
 clock at its phase boundaries behind the K-split workspace; this module launches the shape, reads the stamps back and
 prints medians over the workgroups: cycles from start to the first data in LDS, of the main loop, of parking and
@@ -31,12 +31,19 @@ STAMP_BYTES = 1 << 20
 
 def run(ws, dt, M, K, N, tile, S, waves=8, out=sys.stdout):
     mx.set_option("waves", waves)
+    kw = {}
     if dt == "i8":
         A = torch.randint(-127, 128, (M, K), dtype=torch.int8, device="cuda")
         Bp = mx.repack_b(torch.randint(-127, 128, (K, N), dtype=torch.int8, device="cuda"))
         C = torch.zeros((M, N), dtype=torch.int8, device="cuda")
         ep = mx.Epilogue(C, mx.PP_DEQUANT | mx.PP_BIAS | mx.PP_QUANT, bias=torch.zeros(N, device="cuda"),
                          deq_scale_per_oc=torch.full((N,), 1e-4, device="cuda"), q_scale=20.0)
+    elif dt == "w8":
+        A = torch.randn((M, K), device="cuda").to(torch.bfloat16)
+        Bp = mx.repack_b(torch.randint(-127, 128, (K, N), dtype=torch.int8, device="cuda"))
+        C = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        ep = mx.Epilogue(C, mx.PP_DEQUANT, deq_scale=0.01)
+        kw = {"b_dtype": mx.I8}
     else:
         A = torch.randn((M, K), device="cuda").to(torch.bfloat16)
         Bp = mx.repack_b((torch.randn((K, N), device="cuda") * 0.02).to(torch.bfloat16))
@@ -45,11 +52,11 @@ def run(ws, dt, M, K, N, tile, S, waves=8, out=sys.stdout):
     stamp_off = COUNTER_BYTES + STAMP_OFFSET
     mx.set_tile(tile)
     try:
-        mx.time_gemm(A, [Bp], N, ep, 100, k_splits=S, ws=ws)
-        ms = mx.time_gemm(A, [Bp], N, ep, 100, k_splits=S, ws=ws)
+        mx.time_gemm(A, [Bp], N, ep, 100, k_splits=S, ws=ws, **kw)
+        ms = mx.time_gemm(A, [Bp], N, ep, 100, k_splits=S, ws=ws, **kw)
         torch.cuda.synchronize()
         ws[stamp_off:].zero_()
-        mx.gemm(A, Bp, N, ep, k_splits=S, ws=ws)   # one launch: with a K split, which workgroup of a tile arrives last varies
+        mx.gemm(A, Bp, N, ep, k_splits=S, ws=ws, **kw)   # one launch: with a K split, which workgroup of a tile arrives last varies
         torch.cuda.synchronize()
         kern = mx.last_kernel()
         S = int(kern.rsplit("ksplit", 1)[1]) if "ksplit" in kern else 1
