@@ -290,6 +290,24 @@ __device__ __forceinline__ bf16x8 s8x8_to_bf16(uint32_t lo, uint32_t hi) {
     return r;
 }
 
+// One dword of the above: the bf16 pair of bytes 2 PAIR and 2 PAIR + 1 of src (three instructions), for callers that
+// spread a fragment's conversion over several issue slots.
+template <int PAIR>
+__device__ __forceinline__ uint32_t s8x2_to_bf16(uint32_t src) {
+    float a, b;
+    if constexpr (PAIR == 0) {
+        asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(a) : "v"(src));
+        asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1" : "=v"(b) : "v"(src));
+    } else {
+        asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(a) : "v"(src));
+        asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3" : "=v"(b) : "v"(src));
+    }
+    bf16x2 r;
+    r[0] = (__bf16)a;
+    r[1] = (__bf16)b;
+    return __builtin_bit_cast(uint32_t, r);
+}
+
 // fp32 -> bf16, round to nearest even (vcvtne2ps2bf16, include/kernels_amx.hpp:654)
 __device__ __forceinline__ uint16_t to_bf16(float x) {
     __bf16 b = (__bf16)x;

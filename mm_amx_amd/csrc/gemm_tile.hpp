@@ -503,14 +503,29 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4,
                     if constexpr (rd < NJ) {
                         if constexpr (!W8) {
                             nb[rd] = *reinterpret_cast<const frag*>(sB + rd * BP_HS);
-                        } else if constexpr (KS == 1) {  // next: k-step 0 of the next half-stage - fetch its fragment, use the first half
+                        } else if constexpr (KS == 1) {  // next: k-step 0 of the next half-stage - fetch its int8 fragment
                             braw[rd] = *reinterpret_cast<const u32x4*>(sB + rd * BP_HS);
-                            nb[rd] = s8x8_to_bf16(braw[rd][0], braw[rd][1]);
-                        } else {                         // next: k-step 1 of this half-stage - the second half of what is here
-                            nb[rd] = s8x8_to_bf16(braw[rd][2], braw[rd][3]);
                         }
                     } else if constexpr (rd < NJ + MI) na[rd - NJ] = *reinterpret_cast<const frag*>(sA + (rd - NJ) * 32 * 128);
                 });
+                // int8 fragments -> the next k-step's bf16 operands, one dword (two weights, three instructions) at a time
+                // and spread over the k-step's MFMA slots: a wave issues in order, and a whole fragment's conversion in
+                // one slot (12 instructions) takes twice as long as the MFMA it should hide behind.  k-step 1 converts
+                // the first halves of the fragments it has just fetched, so it starts a few slots behind their reads.
+                if constexpr (W8) {
+                    constexpr int D = 4 * NJ;                                       // dwords to produce
+                    constexpr int S0 = KS == 1 ? (NJ + 1 < MN / 2 ? NJ + 1 : MN / 2) : 0;  // first slot that converts
+                    static_for<0, D>([&](auto d_c) {
+                        constexpr int d = decltype(d_c)::value;
+                        if constexpr (S0 + d * (MN - S0) / D == t) {
+                            constexpr int j = d / 4, e = d % 4;
+                            const uint32_t src = braw[j][(KS == 1 ? 0 : 2) + e / 2];
+                            u32x4 w = __builtin_bit_cast(u32x4, nb[j]);
+                            w[e] = s8x2_to_bf16<e % 2>(src);
+                            nb[j] = __builtin_bit_cast(frag, w);
+                        }
+                    });
+                }
                 if constexpr (Q0 + t < Q1) dma(integral_constant<int, Q0 + t>{}, half_c, kp);
                 // four parts of the next k-step's parameters in the last four slots (all in the last one
                 // where a k-step has fewer)
@@ -968,8 +983,8 @@ static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, bool w
             }
             const int kit = S > 1 ? slice_kiters(nk, S) : nk;
             // int8 weights under bf16 A: every wave converts its own fragments, 12 vector instructions per MFMA operand,
-            // which a small block per wave cannot hide behind its MFMAs (measured issue efficiencies)
-            const float eff = !wide_only ? c.eff : (c.bm == 256 ? 0.80f : (c.bn == 256 ? 0.50f : (c.bn == 192 ? 0.46f : 0.42f)));
+            // which a block of only two row-blocks per wave cannot hide behind its MFMAs (measured issue efficiencies)
+            const float eff = !wide_only ? c.eff : (c.bm == 256 ? 0.85f : (c.bn == 256 ? 0.62f : (c.bn == 192 ? 0.60f : 0.50f)));
             const float mfma = (float)(c.bm * c.bn / 32) / eff, bytes = (float)((c.bm + c.bn) * 128) / l1_bytes_per_clk;
             const float loop = (float)kit * (mfma > bytes ? mfma : bytes);
             const float epi = (float)(c.bm * c.bn / 256) * 100.0f;  // between a plain store (45) and a GELU (170): the plan must
@@ -1025,7 +1040,9 @@ static int launch_tiles(const GemmArgs& g, TileCfg t, int mode, int grid, hipStr
     if (mode == 3) return MMX_LAUNCH(TIn, 128, 128, 3, TOut, 1);  // the masked path exists for one tile shape
     if (t.bm == 256 && t.bn == 256) {
         // two waves per SIMD (a 64x128 block each): MLP gate/up at M = 2048 325 -> 312 us, same bits
-        if (wave_count() == 8 && mode == 2 && g.ksplit == 1) return launch_cfg<TIn, 256, 256, 2, TOut, 1, 8>(g, grid, st);
+        // (not over int8 weights: there the four-wavefront forms are as fast or faster, 91.5 against 98.2 us for 256x192)
+        if constexpr (!Mfma<TIn>::W8)
+            if (wave_count() == 8 && mode == 2 && g.ksplit == 1) return launch_cfg<TIn, 256, 256, 2, TOut, 1, 8>(g, grid, st);
         return MMX_LAUNCH_MODES(TIn, 256, 256, TOut);
     }
     // (eight wavefronts were measured on the 128-row tiles as well: within +-3 % of four, not instantiated)
@@ -1033,7 +1050,8 @@ static int launch_tiles(const GemmArgs& g, TileCfg t, int mode, int grid, hipStr
     if (t.bm == 128 && t.bn == 128) return MMX_LAUNCH_MODES(TIn, 128, 128, TOut);
     if (t.bm == 256 && t.bn == 192) {
         // two waves per SIMD, half the accumulator block each (ring pipeline, no K split)
-        if (wave_count() == 8 && mode == 2 && g.ksplit == 1) return launch_cfg<TIn, 256, 192, 2, TOut, 1, 8>(g, grid, st);
+        if constexpr (!Mfma<TIn>::W8)
+            if (wave_count() == 8 && mode == 2 && g.ksplit == 1) return launch_cfg<TIn, 256, 192, 2, TOut, 1, 8>(g, grid, st);
         return MMX_LAUNCH_MODES(TIn, 256, 192, TOut);
     }
     if (t.bm == 128 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 128, 192, TOut);
