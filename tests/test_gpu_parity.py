@@ -960,6 +960,46 @@ def test_mlp_replays_from_a_hip_graph(M):
         assert np.array_equal(got, host_bits(y2)), rep
 
 
+@pytest.mark.parametrize("S", [2, 4])
+def test_ksplit_replays_from_a_hip_graph(po, ws, S):
+    """The K split under graph replay: the arrival counters reset themselves with the last arrival of every tile, so a
+    captured launch can be replayed without anything being cleared in between (no memset node in the graph).  Every
+    replay, with new inputs and eager split launches on the same workspace between the replays, gives the eager bits."""
+    M, K, N = 200, 4096, 640
+    rng = np.random.default_rng(180 + S)
+    B = rand_bf16(rng, (K, N), 0.05)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    packed, biasd = mx.repack_b(dev_bf16(B)), dev(bias)
+    x = dev_bf16(rand_bf16(rng, (M, K), 1.0)).clone()
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    ep = mx.Epilogue(y, mx.PP_BIAS | mx.PP_GELU, bias=biasd)
+    mx.set_tile("128x128")
+    try:
+        g = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            mx.gemm(x, packed, N, ep, k_splits=S, ws=ws)   # warm-up on the capture stream
+            side.synchronize()
+            with torch.cuda.graph(g, stream=side):
+                mx.gemm(x, packed, N, ep, k_splits=S, ws=ws)
+        assert f"ksplit{S}" in mx.last_kernel()
+        torch.cuda.synchronize()
+        for rep in range(4):
+            x.copy_(dev_bf16(rand_bf16(rng, (M, K), 1.0)))
+            y.zero_()
+            g.replay()
+            torch.cuda.synchronize()
+            got = host_bits(y).copy()
+            assert not ws[:16 << 10].any().item(), "counters not back at zero after a replay"
+            y2 = torch.zeros_like(y)
+            mx.gemm(x, packed, N, mx.Epilogue(y2, mx.PP_BIAS | mx.PP_GELU, bias=biasd), k_splits=S, ws=ws)   # eager, same workspace
+            torch.cuda.synchronize()
+            assert np.array_equal(got, host_bits(y2)), rep
+    finally:
+        mx.set_tile("")
+
+
 # ---- int8 activations at M <= 32: the streaming decode form (int32 sums, order-free) --------------------------
 @pytest.mark.parametrize("shape", [(1, 128, 64), (5, 1024, 100), (32, 1152, 192), (4, 4096, 352), (9, 4096, 33),
                                    (2, 8192, 96), (16, 4096, 352), (32, 2560, 100), (12, 11008, 64), (32, 4224, 96)])
