@@ -622,6 +622,35 @@ def main():
             del gr, ks, scf
         extra["streaming_read_floor"] = floor
 
+        # The vendor library on the same shapes, same box (torch.matmul / torch._int_mm -> hipBLASLt; the bare product,
+        # no bias, no GELU, no requantisation), for context only
+        vend = {}
+
+        def t_us(fn, iters=100):
+            for _ in range(30):
+                fn()
+            torch.cuda.synchronize()
+            a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a0.record()
+            for _ in range(iters):
+                fn()
+            a1.record()
+            torch.cuda.synchronize()
+            return a0.elapsed_time(a1) * 1e3 / iters
+        try:
+            At = torch.randn((M, K), dtype=torch.float32, device="cuda").to(torch.bfloat16)
+            Bt = (torch.randn((K, N), dtype=torch.float32, device="cuda") * 0.02).to(torch.bfloat16)
+            us = t_us(lambda: torch.matmul(At, Bt))
+            vend["bf16_matmul_M1024_K4096_N11008"] = {"us": round(us, 2), "tflops": round(flops / us / 1e6, 1)}
+            Ai8 = torch.randint(-127, 128, (512, 4096), dtype=torch.int8, device="cuda")
+            Bi8 = torch.randint(-127, 128, (4096, 4096), dtype=torch.int8, device="cuda")
+            us = t_us(lambda: torch._int_mm(Ai8, Bi8))
+            vend["int8_int_mm_M512_K4096_N4096"] = {"us": round(us, 2), "tops": round(2.0 * 512 * 4096 * 4096 / us / 1e6, 1)}
+            del At, Bt, Ai8, Bi8
+        except Exception as e:  # an op this torch build lacks: say so
+            vend["note"] = f"{type(e).__name__}: {e}"[:160]
+        extra["torch_hipblaslt_same_shapes"] = vend
+
         # what the matrix pipes deliver with nothing else going on: an issue-bound loop of independent MFMAs,
         # all-zero operands vs operands like the benchmark's (the clock under matrix load depends on the data)
         ceil = {}
