@@ -209,7 +209,10 @@ const char* mmx_last_kernel(void);
  * workgroup, 4 keeps the four-wavefront form (same results).  "decode_valu": whether the
  * streaming decode kernel at M = 1 over int8-compressed weights uses v_dot2_f32_bf16 and a cross-lane add
  * instead of the matrix cores — -1 (default) where at most one workgroup per CU is launched (it is the faster form
- * there), 0 never, 1 always; the two forms agree to fp32 summation order. */
+ * there), 0 never, 1 always; the two forms agree to fp32 summation order.  "decode_resident": whether a decode
+ * launch (M <= 32, bf16 or int8-compressed weights, K a multiple of 512) whose x fits in one CU's LDS but not twice
+ * runs as one workgroup per CU that keeps x there and walks the panels — -1 (default) where the streaming kernel does
+ * not apply (x above 80 KiB), 0 never, 1 wherever x fits (same results as the streaming kernel). */
 int mmx_set_option(const char* name, int value);  /* like mmx_set_tile: affects the calling thread's later calls only */
 /* HIP-event timing of `iters` back-to-back launches of the given gemm on `stream`, launch i
  * using the packed weights Bpacked_rot[i % n_rot] (rotate over several copies so that a

@@ -89,11 +89,13 @@ static thread_local TileCfg g_forced = {0, 0};
 static thread_local int g_load_mode = 2;
 static thread_local int g_decode_halves = -1;
 static thread_local int g_decode_valu = -1;
+static thread_local int g_decode_resident = -1;
 static thread_local int g_waves = 8;
 TileCfg forced_tile() { return g_forced; }
 int load_mode() { return g_load_mode; }
 int decode_halves() { return g_decode_halves; }
 int decode_valu() { return g_decode_valu; }
+int decode_resident() { return g_decode_resident; }
 int wave_count() { return g_waves; }
 
 static int elesz_of(int dtype) { return dtype == MMX_BF16 ? 2 : dtype == MMX_I8 ? 1 : 0; }
@@ -374,6 +376,11 @@ int mmx_set_option(const char* name, int value) {
     if (name && !strcmp(name, "decode_valu")) {
         if (value < -1 || value > 1) return set_error(MMX_E_INVALID, "mmx_set_option: decode_valu is -1, 0 or 1");
         g_decode_valu = value;
+        return MMX_OK;
+    }
+    if (name && !strcmp(name, "decode_resident")) {
+        if (value < -1 || value > 1) return set_error(MMX_E_INVALID, "mmx_set_option: decode_resident is -1, 0 or 1");
+        g_decode_resident = value;
         return MMX_OK;
     }
     if (name && !strcmp(name, "waves")) {

@@ -690,6 +690,175 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     skinny_finish<NP, I8A>(s, red, panel_first, tid, fin);
 }
 
+// ---- resident-x variant: more rows than two workgroups per CU can hold a copy of ----------------------
+// For 10-16 rows of a 4096-wide x the activations are 80-128 KiB: one copy fits in a CU's LDS, two do not.  So there
+// is one workgroup per CU, x goes to LDS once, and the workgroup walks its panels (blockIdx.x + i * gridDim.x) with the
+// weight stream running across panel boundaries: a register set is re-requested for the next batch of fragments, of
+// this panel or the next, as soon as it has been multiplied, so 16 KiB per wave are in flight until the last panel
+// ends.  (The chunked kernel re-stages x per workgroup, 44 MB for 344 panels, behind a barrier per chunk with 24 KiB
+// of weights in flight per workgroup.)
+// A wave multiplies the same share of K in every panel, so it needs only that share of every row of x: each wave
+// fetches its own slice (global_load_lds, no registers) into its own LDS region and waits for nothing but its own
+// loads -- no barrier before the first multiply.  A region holds [M rows][SB + 16 bytes], SB = the slice of a row;
+// the 16 bytes of padding make the row pitch an odd number of 16-byte pieces, so the 16 rows x 16 bytes that one LDS
+// cycle serves for an MFMA operand fall into different banks.  Lanes of rows >= M read row 0 (their outputs are
+// never stored).  K fills whole batches of fragments (the launcher checks).
+// Every load of the kernel is issued and waited for by hand: the rolling window crosses loop iterations and
+// branches, where the compiler's own count of outstanding loads falls back to "wait for all of them" (measured:
+// 14.7 us at M = 1 against 10.8 for the streaming kernel).  Loads return in order, so "at most n outstanding" names
+// the n youngest; the counts below follow from the order of issue.  The wait hands the register set on as its
+// output, so nothing that reads it can be scheduled ahead of the wait.
+// Per-column post-op operands go to LDS the same way (wave 0, global_load_lds_dword) at the start of a panel.
+// Cross-wave reduction per panel through red[8 waves][16][2][MR] (MR = 16 or 32 rows), behind the regions.
+template <bool W8, int U>  // U: fragments per panel and wave (K = 8 waves x U fragments)
+__global__ __launch_bounds__(512) void skinny_resident_kernel(const SkinnyArgs s, int region, int red_off, int mr_log2) {
+    // Fragments (KiB) a wave keeps in flight.  More is worse: a wave is held at a request until the CU accepts it
+    // (4096 x 11008 int8 at M = 16: 13.0 us with 4, 13.1 with 8, 14.1 with 16; 3: 13.3, 2: 14.3).
+    constexpr int D = 4;
+    constexpr int XB = W8 ? 64 : 32;    // bytes of a row of x that one fragment covers
+    extern __shared__ __attribute__((aligned(1024))) char xs[];
+    float* const red = reinterpret_cast<float*>(xs + red_off);
+    const float* const oc = reinterpret_cast<const float*>(xs + red_off + (1024 << mr_log2));  // [3][64]
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, g32 = lane >> 5;
+    const int row_bytes = s.K * 2;
+    const int G = gridDim.x;
+    const int panel0 = (s.n0 >> 5) + (int)blockIdx.x;
+    const int panels = ((s.n1 + 31) >> 5) - (s.n0 >> 5);
+    const int npan = (panels - (int)blockIdx.x + G - 1) / G;  // >= 1: the launcher keeps gridDim.x <= panels
+    const Epilogue& ep = s.ep;
+    const bool deq_oc = (ep.steps & MMX_PP_DEQUANT) && ep.deq_oc, bias_oc = (ep.steps & MMX_PP_BIAS) != 0,
+               q_oc = (ep.steps & MMX_PP_QUANT) && ep.q_oc;
+
+    constexpr int per_wave = U;  // the launcher checks: nfrag = 8 * U
+    const int f_begin = wave * per_wave;
+    const int SB = per_wave * XB;
+    const int rowp = SB + 16;
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)xs);
+    {   // this wave's slice of x -> its LDS region, 64 pieces of 16 bytes per instruction (piece = row-major index over
+        // [M][SB / 16 + 1]; the padding piece and the pieces past the end re-read a neighbour)
+        const uint32_t lds_w = lds_base + (uint32_t)(wave * region);
+        const int cpr1 = SB / 16 + 1;
+        const int npieces = s.M * cpr1;
+        const int slice0 = f_begin * XB;
+        int r = lane / cpr1, c = lane - r * cpr1;
+        for (int i0 = 0; i0 < npieces; i0 += 64) {
+            const int rr = r < s.M ? r : s.M - 1;
+            int cb = slice0 + (c < cpr1 - 1 ? c : cpr1 - 2) * 16;
+            cb = cb < row_bytes - 16 ? cb : row_bytes - 16;
+            const char* src = s.x + (int64_t)rr * s.ldx + cb;
+            const uint32_t m0v = lds_w + (uint32_t)(i0 * 16);
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0v), "v"(src) : "memory");
+            c += 64;
+            while (c >= cpr1) {
+                c -= cpr1;
+                r++;
+            }
+        }
+    }
+    // per-column post-op operands of a panel -> oc (wave 0; lanes 32-63 repeat the 32 columns)
+    auto stage_operands = [&](int panel) __attribute__((always_inline)) {
+        if (wave != 0) return;
+        int n = (panel << 5) + l32;
+        n = n < s.n1 ? n : s.n1 - 1;
+        const uint32_t dst = lds_base + (uint32_t)(red_off + (1024 << mr_log2));
+        if (deq_oc) {
+            const float* src = ep.deq_oc + n;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(dst), "v"(src) : "memory");
+        }
+        if (bias_oc) {
+            const float* src = ep.bias + n;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(dst + 256), "v"(src) : "memory");
+        }
+        if (q_oc) {
+            const float* src = ep.q_oc + n;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(dst + 512), "v"(src) : "memory");
+        }
+    };
+
+    const int mrow = l32 < s.M ? l32 : 0;
+    const char* const xrow = xs + wave * region + mrow * rowp + g32 * (XB / 2);
+    const int64_t wstep = (int64_t)G * s.panel_stride;
+    const char* wcur = s.Wp + (int64_t)panel0 * s.panel_stride + (int64_t)f_begin * 1024 + lane * 16;  // this wave's first fragment
+
+    u32x4 w[D];
+    f32x16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+
+    // Fragment g of this wave's stream (g / U = panel of the workgroup, g % U = fragment of the wave's share) lives in
+    // register set g % D.  (Nontemporal: the weights are read once.  The scheduler barrier keeps the requests in the
+    // order written, which the compiler's waits then follow: left alone it reorders them and waits for the youngest.)
+#define MMX_REQUEST(GG)                                                                     \
+    do {                                                                                    \
+        w[(GG) % D] = MMX_WLOAD(((GG) / U ? wcur + wstep : wcur) + ((GG) % U) * 1024);      \
+        __builtin_amdgcn_sched_barrier(0);                                                  \
+    } while (0)
+
+    // The first fragments behind x.  A wave is held at a request until the CU accepts it, so only U0 go out before the
+    // wait for x ("at most these outstanding": this wave's slice of x has landed).
+    constexpr int U0 = D < 4 ? D : 4;
+    skinny_static_for<0, U0>([&](auto g_c) __attribute__((always_inline)) { MMX_REQUEST(decltype(g_c)::value); });
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(U0) : "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    skinny_static_for<U0, D>([&](auto g_c) __attribute__((always_inline)) { MMX_REQUEST(decltype(g_c)::value); });
+
+    const int MR = 1 << mr_log2;
+    // cross-wave sum of the panel's partial blocks, post-op, store.  (Barriers by hand: __syncthreads() would also
+    // wait for the weight loads of the next panel.)
+    auto finish = [&](int panel) __attribute__((always_inline)) {
+        if (l32 < MR) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) red[((((wave * 16 + v) * 2) + g32) << mr_log2) + l32] = acc[v];
+        }
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory");
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            const int idx = tid + 512 * t;
+            const int v = idx >> (mr_log2 + 1), g = (idx >> mr_log2) & 1, m = idx & (MR - 1);
+            const int nloc = 8 * (v >> 2) + 4 * g + (v & 3);
+            const int n = (panel << 5) + nloc;
+            if (v >= 16 || m >= s.M || n >= s.n1) continue;
+            float r = 0.0f;
+#pragma unroll
+            for (int w8 = 0; w8 < 8; w8++) r += red[((((w8 * 16 + v) * 2) + g) << mr_log2) + m];
+            if (ep.steps & MMX_PP_DEQUANT) r = r * (deq_oc ? oc[nloc] : ep.deq);
+            if (ep.steps & MMX_PP_BIAS) r = r + oc[64 + nloc];
+            if (ep.steps & MMX_PP_GELU) r = gelu_erf_minimax(r);
+            if (ep.steps & MMX_PP_QUANT) r = r * (q_oc ? oc[128 + nloc] : ep.q);
+            store_out(ep, m, n, r);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory");  // the next panel overwrites scratch and operands
+    };
+    // One batch of U fragments per panel and at most two panels per workgroup (the launcher checks): straight-line
+    // code, so the compiler counts the outstanding loads exactly.  Each multiply is followed by the request for the
+    // fragment D places further on, of this panel or the next.
+    auto run = [&](auto npan_c) __attribute__((always_inline)) {
+        constexpr int TOTAL = decltype(npan_c)::value * U;
+        skinny_static_for<0, TOTAL>([&](auto g_c) __attribute__((always_inline)) {
+            constexpr int g = decltype(g_c)::value, u = g % U;
+            if constexpr (u == 0) stage_operands(panel0 + (g / U) * G);
+            const bf16x8 xa = *reinterpret_cast<const bf16x8*>(xrow + u * XB);
+            if constexpr (W8) {
+                const bf16x8 xc = *reinterpret_cast<const bf16x8*>(xrow + u * XB + 16);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(w[g % D].x, w[g % D].y), xa, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(w[g % D].z, w[g % D].w), xc, acc, 0, 0, 0);
+            } else {
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w[g % D]), xa, acc, 0, 0, 0);
+            }
+            if constexpr (g + D < TOTAL) MMX_REQUEST(g + D);
+            if constexpr (u == U - 1) finish(panel0 + (g / U) * G);
+        });
+    };
+    if (npan > 1) run(std::integral_constant<int, 2>{});
+    else run(std::integral_constant<int, 1>{});
+#undef MMX_REQUEST
+}
+
 // Half-panel variant of the streaming kernel for 1-4 rows of x.  A list of 32-column panels that is only 1-2
 // per CU long leaves some CUs with twice the work of others (or idle), and how fast one CU can pull
 // weights in is what bounds this kernel.  Here a workgroup (four waves) multiplies HALF a panel
@@ -882,6 +1051,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 
 int decode_halves();
 int decode_valu();
+int decode_resident();
 
 // int8 x int8 at M <= 32 can use the decode kernels if x is 16-byte aligned and K fills whole 128-byte groups of
 // the packed weights: the streaming form if x fits in LDS, else the chunked one, which walks K in chunks of 256
@@ -987,6 +1157,41 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         else
             hipLaunchKernelGGL((skinny_half_kernel<false, 1, false, 16>), dim3(2 * panels), dim3(256), xbytes, st, s, zero_off);
         return check_hip(hipGetLastError(), "skinny_half_kernel launch");
+    }
+    {
+        // x fits in one CU's LDS once: one workgroup per CU keeps it there and walks its one or two panels.  Taken where the
+        // streaming form cannot hold x twice per CU (4096 x 11008 int8 at M = 10 / 16: 12.3 / 13.1 us against 13.5 / 14.6 for
+        // the chunked form; 8192 x 4096 at M = 6: 10.4 against 17.1; over bf16 weights only while no workgroup has a second
+        // panel: 4096 x 4096 at M = 12 9.9 against 12.0, but 4096 x 11008 at M = 16 21.2 against 20.9), and over int8
+        // weights wherever no workgroup has a second panel (4096 x 4096: M = 1 6.1 against 6.7 us, M = 4 6.4 against 8.0;
+        // 8192 x 4096: M = 1 9.5 against 10.9); with two panels on some CUs and few rows the streaming form's two
+        // workgroups per CU are ahead (11008 columns, M = 1: 10.8 against 11.4 us).
+        // decode_resident(): -1 by that rule (and only while decode_valu and decode_halves are left alone), 0 never,
+        // 1 wherever the shape allows.
+        const int rforce = decode_resident();
+        const int mr_log2 = M <= 16 ? 4 : 5;
+        const int slice = (s.nfrag >> 3) * (w8 ? 64 : 32);                 // bytes of a row of x per wave
+        const int region = (M * (slice + 16) + 1023) & ~1023;              // LDS per wave
+        const int red_off = 8 * region;
+        const int lds = red_off + (1024 << mr_log2) + 2048;   // regions, reduction scratch, post-op operands
+        const bool shape_ok = kpad == K && s.x_vec_ok && !pairs && (s.nfrag == 128 || s.nfrag == 256) && panels > 0 &&
+                              panels <= 2 * num_cus() && lds <= 160 * 1024;
+        const bool one_each = panels <= num_cus();
+        const bool by_rule = (xbytes > 80 * 1024 && (w8 || one_each)) || (w8 && one_each && decode_valu() == -1 && decode_halves() == -1);
+        if (shape_ok && rforce != 0 && (rforce == 1 || by_rule)) {
+            typedef void (*ResidentKernel)(const SkinnyArgs, int, int, int);
+            static std::atomic<uint64_t> attr_done[4];
+            const ResidentKernel kerns[4] = {skinny_resident_kernel<false, 16>, skinny_resident_kernel<false, 32>,
+                                             skinny_resident_kernel<true, 16>, skinny_resident_kernel<true, 32>};
+            const int ki = (w8 ? 2 : 0) + (s.nfrag == 256 ? 1 : 0);
+            const ResidentKernel kern = kerns[ki];
+            const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, attr_done[ki]);
+            if (rc) return rc;
+            note_kernel(w8 ? "skinny_resident_w8" : "skinny_resident_bf16");
+            const int grid = panels < num_cus() ? panels : num_cus();
+            hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, st, s, region, red_off, mr_log2);
+            return check_hip(hipGetLastError(), "skinny_resident_kernel launch");
+        }
     }
     // The streaming form needs all of x in LDS and at least two workgroups per CU (344 panels of N = 11008 must all
     // be resident): 80 KiB of x each (4096 x 11008 int8 GEMV at M = 5-8: 13.0-13.4 -> 11.5-12.0 us against the chunked

@@ -54,13 +54,14 @@ def test_sizes_and_argument_validation(lib):
     assert lib.mmx_set_option(b"nonsense", 1) != 0
     # every documented option takes its documented values and nothing else
     for name, good, bad in ((b"load_mode", (0, 2), (1, 3)), (b"waves", (4, 8), (2, 16)), (b"decode_halves", (-1, 0, 1), (-2, 2)),
-                            (b"decode_valu", (-1, 0, 1), (-2, 2))):
+                            (b"decode_valu", (-1, 0, 1), (-2, 2)), (b"decode_resident", (-1, 0, 1), (-2, 2))):
         for v in bad:
             assert lib.mmx_set_option(name, v) != 0, (name, v)
         for v in good:
             assert lib.mmx_set_option(name, v) == 0, (name, v)
     assert lib.mmx_set_option(b"load_mode", 2) == 0 and lib.mmx_set_option(b"waves", 8) == 0
     assert lib.mmx_set_option(b"decode_halves", -1) == 0 and lib.mmx_set_option(b"decode_valu", -1) == 0
+    assert lib.mmx_set_option(b"decode_resident", -1) == 0
     # NULL operands are rejected by validation, before any HIP call
     assert lib.mmx_gemm(1, 1, None, C.c_int64(0), None, 1, 64, 64, 0, 64, None, None) == -1
     assert b"NULL" in lib.mmx_last_error()

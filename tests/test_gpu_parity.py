@@ -256,11 +256,19 @@ def test_decode_gemv_w8_full_size(po, M):
     print(f"gemv_w8 M={M}: rel_fro={err:.2e} within_1ulp={frac * 100:.4f}%")
 
 
+@pytest.fixture
+def no_resident_form():
+    """Keeps the decode launches of a test on the kernels they were written for (the resident-x form has its own tests)."""
+    mx.set_option("decode_resident", 0)
+    yield
+    mx.set_option("decode_resident", -1)
+
+
 # the last three: 46-80 KiB of x, which the streaming form still holds in LDS (the reduction scratch reuses the space)
 @pytest.mark.parametrize("shape", [(1, 256, 64), (3, 320, 100), (16, 337, 96), (32, 2560, 192), (7, 70, 45),
                                    (8, 4096, 96), (9, 4096, 160), (5, 6144, 64)])
 @pytest.mark.parametrize("w8", [False, True])
-def test_decode_small_shapes(po, shape, w8):
+def test_decode_small_shapes(po, shape, w8, no_resident_form):
     M, K, N = shape
     rng = np.random.default_rng(sum(shape) + int(w8))
     x = rand_bf16(rng, (M, K), 1.0)
@@ -390,6 +398,92 @@ def test_decode_valu_form(po, shape, out):
         assert np.all(got[:, :n0] == fill) and np.all(got[:, n1:] == fill)   # nothing outside the range is written
     a, b = res[1][1].astype(np.float64), res[0][1].astype(np.float64)
     assert np.linalg.norm(a - b) <= 1e-5 * np.linalg.norm(b)
+
+
+# One workgroup per CU that keeps x in LDS and walks its one or two panels ("decode_resident"): K of exactly 8 waves x 16 or
+# 32 fragments, one and two panels per workgroup (N up to and beyond 256 x 32 columns), ragged N, a column range,
+# every post-op operand and output type; the accumulators against the oracle, the fused store = the oracle's post-op on
+# the GPU's own sums, and the same bits as the streaming kernel wherever both run (same split of K over the waves,
+# same order of the cross-wave sum).
+@pytest.mark.parametrize("case", [(True, 1, 4096, 352), (True, 16, 4096, 4096), (True, 10, 4096, 11008), (True, 16, 4096, 16384),
+                                  (True, 5, 8192, 1000), (True, 4, 4096, 8200), (False, 12, 4096, 2000), (False, 16, 2048, 9000),
+                                  (False, 3, 4096, 96)])
+@pytest.mark.parametrize("out", ["f32", "bf16", "i8"])
+def test_decode_resident_form(po, case, out):
+    w8, M, K, N = case
+    if out != "f32" and K * N > 4096 * 4096:
+        pytest.skip("the large shapes with the fp32 store only")
+    rng = np.random.default_rng(13 * (M + K + N) + int(w8))
+    x = rand_bf16(rng, (M, K), 1.0)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    qs = rng.uniform(10.0, 30.0, N).astype(np.float32)
+    if w8:
+        W = np.clip(np.rint(rng.standard_normal((K, N)) * 40), -127, 127).astype(np.int8)
+        scale = rng.uniform(1e-3, 5e-3, N).astype(np.float32)
+        _, acc_ref = po.gemv_w8(x, W, scale, want_acc=True)
+        packed, kw = mx.repack_b(dev(W)), {"b_dtype": mx.I8}
+    else:
+        W = rand_bf16(rng, (K, N), 0.05)
+        scale = rng.uniform(0.5, 2.0, N).astype(np.float32)
+        acc_ref = po.gemm_bf16(x, W)
+        packed, kw = mx.repack_b(dev_bf16(W)), {}
+    steps = mx.PP_DEQUANT | mx.PP_BIAS | mx.PP_GELU | (mx.PP_QUANT if out == "i8" else 0)
+    posteps = po.PP_DEQUANT | po.PP_BIAS | po.PP_GELU | (po.PP_QUANT if out == "i8" else 0)
+    tdt, odt = {"f32": (torch.float32, po.F32), "bf16": (torch.bfloat16, po.BF16), "i8": (torch.int8, po.I8)}[out]
+    n0, n1 = (64, N - 5) if N > 160 else (0, N)   # a column range that starts on a panel and ends inside one
+    res = {}
+    try:
+        for resident in (1, 0):
+            mx.set_option("decode_resident", resident)
+            mx.set_option("decode_halves", 0)
+            mx.set_option("decode_valu", 0)
+            y = torch.full((M, N), 7, dtype=tdt, device="cuda")
+            mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, steps, bias=dev(bias), deq_scale_per_oc=dev(scale), q_scale_per_oc=dev(qs)),
+                    n0=n0, n1=n1, **kw)
+            k1 = mx.last_kernel()
+            acc = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+            mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc, mx.PP_NONE), **kw)
+            assert ("resident" in k1) == (resident == 1) and ("resident" in mx.last_kernel()) == (resident == 1), (k1, mx.last_kernel())
+            res[resident] = (host_bits(y), host_bits(acc), mx.last_kernel())
+    finally:
+        mx.set_option("decode_resident", -1)
+        mx.set_option("decode_halves", -1)
+        mx.set_option("decode_valu", -1)
+    fill = host_bits(torch.full((1, 1), 7, dtype=tdt, device="cuda"))[0, 0]
+    for resident, (got, acc, kernel) in res.items():
+        check_float_parity(acc, acc_ref, f"accumulators {case} {kernel}")
+        again = po.pp(acc, posteps, odt, bias=bias, deq_per_oc=scale, q_per_oc=qs)
+        assert np.array_equal(got[:, n0:n1], again[:, n0:n1]), kernel
+        assert np.all(got[:, :n0] == fill) and np.all(got[:, n1:] == fill), kernel   # nothing outside the range is written
+    if "stream" in res[0][2]:
+        assert np.array_equal(res[1][1].view(np.uint32), res[0][1].view(np.uint32)), res[0][2]
+        assert np.array_equal(res[1][0], res[0][0])
+
+
+def test_decode_resident_rule(po):
+    """Left alone, the library takes the resident form where x is too large for two workgroups per CU and, over int8
+    weights, wherever no workgroup has a second panel; shapes it does not cover keep their kernels."""
+    rng = np.random.default_rng(3)
+
+    def kernel_for(w8, M, K, N):
+        x = dev_bf16(rand_bf16(rng, (M, K), 1.0))
+        if w8:
+            packed, kw = mx.repack_b(dev(rng.integers(-127, 128, (K, N), dtype=np.int8))), {"b_dtype": mx.I8}
+        else:
+            packed, kw = mx.repack_b(dev_bf16(rand_bf16(rng, (K, N), 0.05))), {}
+        y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        mx.gemm(x, packed, N, mx.Epilogue(y, mx.PP_NONE), **kw)
+        return mx.last_kernel()
+
+    assert kernel_for(True, 16, 4096, 11008) == "skinny_resident_w8"
+    assert kernel_for(True, 1, 4096, 4096) == "skinny_resident_w8"
+    assert kernel_for(True, 1, 4096, 11008) == "skinny_stream_w8"          # two panels on some CUs, few rows
+    assert kernel_for(True, 16, 4096, 16416) == "skinny_chunk_w8"          # more than two panels per CU
+    assert kernel_for(True, 16, 4160 - 64, 512) == "skinny_resident_w8"    # K = 4096
+    assert kernel_for(True, 16, 5120, 512) == "skinny_chunk_w8"            # K not 8 x 16 or 8 x 32 fragments
+    assert kernel_for(False, 12, 4096, 4096) == "skinny_resident_bf16"
+    assert kernel_for(False, 16, 4096, 11008) == "skinny_chunk_bf16"       # bf16 weights, two panels on some CUs
+    assert "resident" not in kernel_for(False, 1, 4096, 4096)              # bf16 weights, x fits twice: as before
 
 
 # 2-4 rows of a long x (the MLP's down projection: K = 11008) still go whole into LDS for the half-panel form when
