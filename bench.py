@@ -409,15 +409,18 @@ def main():
             yn = torch.zeros((1, Nn), dtype=torch.bfloat16, device="cuda")
             epn = mx.Epilogue(yn, mx.PP_DEQUANT, deq_scale=1e-3)
             ent = {}
-            for form, (valu, halves) in (("mfma", (0, 0)), ("valu", (1, 0)), ("half_panels", (0, 1)), ("auto", (-1, -1))):
+            for form, (valu, halves, resident) in (("mfma", (0, 0, 0)), ("valu", (1, 0, 0)), ("half_panels", (0, 1, 0)),
+                                                   ("resident_x", (-1, -1, 1)), ("auto", (-1, -1, -1))):
                 mx.set_option("decode_valu", valu)
                 mx.set_option("decode_halves", halves)
+                mx.set_option("decode_resident", resident)
                 try:
                     msn = avg_ms(xg1, packs, Nn, epn, 200, b_dtype=mx.I8)
                     ent[form] = {"us": round(msn * 1e3, 2), "kernel": mx.last_kernel()}
                 finally:
                     mx.set_option("decode_valu", -1)
                     mx.set_option("decode_halves", -1)
+                    mx.set_option("decode_resident", -1)
             ent["panels_per_cu"] = round(Nn / 32 / 256, 2)
             ent["auto_weight_GBps"] = round(4096.0 * Nn / ent["auto"]["us"] / 1e3, 0)
             sweepn[str(Nn)] = ent

@@ -713,7 +713,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 template <bool W8, int U>  // U: fragments per panel and wave (K = 8 waves x U fragments)
 __global__ __launch_bounds__(512) void skinny_resident_kernel(const SkinnyArgs s, int region, int red_off, int mr_log2) {
     // Fragments (KiB) a wave keeps in flight.  More is worse: a wave is held at a request until the CU accepts it
-    // (4096 x 11008 int8 at M = 16: 13.0 us with 4, 13.1 with 8, 14.1 with 16; 3: 13.3, 2: 14.3).
+    // (4096 x 11008 int8 at M = 16: 13.0 us with 4, 13.1 with 8, 14.1 with 16; 3: 13.3, 2: 14.3; a deeper window for the
+    // workgroups with two panels only: 6: 13.0, 8: 13.1, 12: 13.6).
     constexpr int D = 4;
     constexpr int XB = W8 ? 64 : 32;    // bytes of a row of x that one fragment covers
     extern __shared__ __attribute__((aligned(1024))) char xs[];
@@ -797,14 +798,6 @@ __global__ __launch_bounds__(512) void skinny_resident_kernel(const SkinnyArgs s
         __builtin_amdgcn_sched_barrier(0);                                                  \
     } while (0)
 
-    // The first fragments behind x.  A wave is held at a request until the CU accepts it, so only U0 go out before the
-    // wait for x ("at most these outstanding": this wave's slice of x has landed).
-    constexpr int U0 = D < 4 ? D : 4;
-    skinny_static_for<0, U0>([&](auto g_c) __attribute__((always_inline)) { MMX_REQUEST(decltype(g_c)::value); });
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(U0) : "memory");
-    __builtin_amdgcn_sched_barrier(0);
-    skinny_static_for<U0, D>([&](auto g_c) __attribute__((always_inline)) { MMX_REQUEST(decltype(g_c)::value); });
-
     const int MR = 1 << mr_log2;
     // cross-wave sum of the panel's partial blocks, post-op, store.  (Barriers by hand: __syncthreads() would also
     // wait for the weight loads of the next panel.)
@@ -839,6 +832,13 @@ __global__ __launch_bounds__(512) void skinny_resident_kernel(const SkinnyArgs s
     // fragment D places further on, of this panel or the next.
     auto run = [&](auto npan_c) __attribute__((always_inline)) {
         constexpr int TOTAL = decltype(npan_c)::value * U;
+        // The first fragments behind x.  A wave is held at a request until the CU accepts it, so only U0 go out before
+        // the wait for x ("at most these outstanding": this wave's slice of x has landed).
+        constexpr int U0 = D < 4 ? D : 4;
+        skinny_static_for<0, U0>([&](auto g_c) __attribute__((always_inline)) { MMX_REQUEST(decltype(g_c)::value); });
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(U0) : "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        skinny_static_for<U0, D>([&](auto g_c) __attribute__((always_inline)) { MMX_REQUEST(decltype(g_c)::value); });
         skinny_static_for<0, TOTAL>([&](auto g_c) __attribute__((always_inline)) {
             constexpr int g = decltype(g_c)::value, u = g % U;
             if constexpr (u == 0) stage_operands(panel0 + (g / U) * G);
@@ -1174,16 +1174,20 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         const int region = (M * (slice + 16) + 1023) & ~1023;              // LDS per wave
         const int red_off = 8 * region;
         const int lds = red_off + (1024 << mr_log2) + 2048;   // regions, reduction scratch, post-op operands
-        const bool shape_ok = kpad == K && s.x_vec_ok && !pairs && (s.nfrag == 128 || s.nfrag == 256) && panels > 0 &&
+        // K = 8 waves x U fragments for the U that exist: 16, 32 (K = 2048, 4096 of bf16 weights; 4096, 8192 of int8 weights) and,
+        // for int8 weights, 20 and 43 (K = 5120, 11008)
+        const bool k_ok = s.nfrag == 128 || s.nfrag == 256 || (w8 && (s.nfrag == 160 || s.nfrag == 344));
+        const bool shape_ok = kpad == K && s.x_vec_ok && !pairs && k_ok && panels > 0 &&
                               panels <= 2 * num_cus() && lds <= 160 * 1024;
         const bool one_each = panels <= num_cus();
         const bool by_rule = (xbytes > 80 * 1024 && (w8 || one_each)) || (w8 && one_each && decode_valu() == -1 && decode_halves() == -1);
         if (shape_ok && rforce != 0 && (rforce == 1 || by_rule)) {
             typedef void (*ResidentKernel)(const SkinnyArgs, int, int, int);
-            static std::atomic<uint64_t> attr_done[4];
-            const ResidentKernel kerns[4] = {skinny_resident_kernel<false, 16>, skinny_resident_kernel<false, 32>,
-                                             skinny_resident_kernel<true, 16>, skinny_resident_kernel<true, 32>};
-            const int ki = (w8 ? 2 : 0) + (s.nfrag == 256 ? 1 : 0);
+            static std::atomic<uint64_t> attr_done[6];
+            const ResidentKernel kerns[6] = {skinny_resident_kernel<false, 16>, skinny_resident_kernel<false, 32>,
+                                             skinny_resident_kernel<true, 16>, skinny_resident_kernel<true, 32>,
+                                             skinny_resident_kernel<true, 20>, skinny_resident_kernel<true, 43>};
+            const int ki = !w8 ? (s.nfrag == 256 ? 1 : 0) : (s.nfrag == 128 ? 2 : (s.nfrag == 256 ? 3 : (s.nfrag == 160 ? 4 : 5)));
             const ResidentKernel kern = kerns[ki];
             const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, attr_done[ki]);
             if (rc) return rc;

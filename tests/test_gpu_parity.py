@@ -400,14 +400,14 @@ def test_decode_valu_form(po, shape, out):
     assert np.linalg.norm(a - b) <= 1e-5 * np.linalg.norm(b)
 
 
-# One workgroup per CU that keeps x in LDS and walks its one or two panels ("decode_resident"): K of exactly 8 waves x 16 or
-# 32 fragments, one and two panels per workgroup (N up to and beyond 256 x 32 columns), ragged N, a column range,
+# One workgroup per CU that keeps x in LDS and walks its one or two panels ("decode_resident"): K of exactly 8 waves x 16,
+# 20, 32 or 43 fragments, one and two panels per workgroup (N up to and beyond 256 x 32 columns), ragged N, a column range,
 # every post-op operand and output type; the accumulators against the oracle, the fused store = the oracle's post-op on
 # the GPU's own sums, and the same bits as the streaming kernel wherever both run (same split of K over the waves,
 # same order of the cross-wave sum).
 @pytest.mark.parametrize("case", [(True, 1, 4096, 352), (True, 16, 4096, 4096), (True, 10, 4096, 11008), (True, 16, 4096, 16384),
-                                  (True, 5, 8192, 1000), (True, 4, 4096, 8200), (False, 12, 4096, 2000), (False, 16, 2048, 9000),
-                                  (False, 3, 4096, 96)])
+                                  (True, 5, 8192, 1000), (True, 4, 4096, 8200), (True, 6, 11008, 1000), (True, 1, 11008, 4096),
+                                  (True, 12, 5120, 704), (False, 12, 4096, 2000), (False, 16, 2048, 9000), (False, 3, 4096, 96)])
 @pytest.mark.parametrize("out", ["f32", "bf16", "i8"])
 def test_decode_resident_form(po, case, out):
     w8, M, K, N = case
@@ -480,7 +480,8 @@ def test_decode_resident_rule(po):
     assert kernel_for(True, 1, 4096, 11008) == "skinny_stream_w8"          # two panels on some CUs, few rows
     assert kernel_for(True, 16, 4096, 16416) == "skinny_chunk_w8"          # more than two panels per CU
     assert kernel_for(True, 16, 4160 - 64, 512) == "skinny_resident_w8"    # K = 4096
-    assert kernel_for(True, 16, 5120, 512) == "skinny_chunk_w8"            # K not 8 x 16 or 8 x 32 fragments
+    assert kernel_for(True, 12, 5120, 512) == "skinny_resident_w8"         # K = 8 x 20 fragments
+    assert kernel_for(True, 16, 6144, 512) == "skinny_chunk_w8"            # no kernel for 8 x 24 fragments
     assert kernel_for(False, 12, 4096, 4096) == "skinny_resident_bf16"
     assert kernel_for(False, 16, 4096, 11008) == "skinny_chunk_bf16"       # bf16 weights, two panels on some CUs
     assert "resident" not in kernel_for(False, 1, 4096, 4096)              # bf16 weights, x fits twice: as before
