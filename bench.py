@@ -356,7 +356,13 @@ def main():
         extra["int8_fc_requant_M512_K4096_N4096"] = {
             "us": round(ms * 1e3, 2), "median_us": med_us(Ai, [Bi], wi["N"], epi), "tops": round(ops / ms / 1e9, 1),
             "frac_of_int8_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4), "kernel": mx.last_kernel()}
-        del Ai, Bi, Ci
+        # the same launch with the rows of A 128 bytes further apart (a row stride that is a multiple of 4 KiB puts the 8 rows
+        # of a load instruction into one L2 channel; the C++ tensor2D pads such rows, this configuration's layout is compact)
+        Apad = torch.zeros((wi["M"], wi["K"] + 128), dtype=torch.int8, device="cuda")
+        Apad[:, :wi["K"]] = Ai
+        msp = avg_ms(Apad[:, :wi["K"]], [Bi], wi["N"], epi, 100)
+        extra["int8_fc_requant_M512_K4096_N4096"]["a_rows_padded_by_128B"] = {"us": round(msp * 1e3, 2), "tops": round(ops / msp / 1e9, 1)}
+        del Ai, Bi, Ci, Apad
         # the same int8 kernel on a shape large enough to fill the machine (the Llama-7B FFN shape at M=2048)
         rng = np.random.default_rng(11)
         Mi, Ki, Ni = 2048, 4096, 11008
