@@ -692,22 +692,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 
 // ---- resident-x variant: more rows than two workgroups per CU can hold a copy of ----------------------
 // For 10-16 rows of a 4096-wide x the activations are 80-128 KiB: one copy fits in a CU's LDS, two do not.  So there
-// is one workgroup per CU, x goes to LDS once, and the workgroup walks its panels (blockIdx.x + i * gridDim.x) with the
-// weight stream running across panel boundaries: a register set is re-requested for the next batch of fragments, of
-// this panel or the next, as soon as it has been multiplied, so 16 KiB per wave are in flight until the last panel
-// ends.  (The chunked kernel re-stages x per workgroup, 44 MB for 344 panels, behind a barrier per chunk with 24 KiB
-// of weights in flight per workgroup.)
+// is one workgroup per CU, x goes to LDS once, and the workgroup walks its one or two panels (blockIdx.x and
+// blockIdx.x + gridDim.x) with the weight stream running across the panel boundary: right after a fragment has been
+// multiplied the one D places further on is requested, of this panel or the next, so D KiB per wave are in flight
+// until the last panel ends.  (The chunked kernel re-stages x per workgroup, 44 MB for 344 panels, behind a barrier
+// per chunk with 24 KiB of weights in flight per workgroup.)
 // A wave multiplies the same share of K in every panel, so it needs only that share of every row of x: each wave
 // fetches its own slice (global_load_lds, no registers) into its own LDS region and waits for nothing but its own
 // loads -- no barrier before the first multiply.  A region holds [M rows][SB + 16 bytes], SB = the slice of a row;
 // the 16 bytes of padding make the row pitch an odd number of 16-byte pieces, so the 16 rows x 16 bytes that one LDS
 // cycle serves for an MFMA operand fall into different banks.  Lanes of rows >= M read row 0 (their outputs are
-// never stored).  K fills whole batches of fragments (the launcher checks).
-// Every load of the kernel is issued and waited for by hand: the rolling window crosses loop iterations and
-// branches, where the compiler's own count of outstanding loads falls back to "wait for all of them" (measured:
-// 14.7 us at M = 1 against 10.8 for the streaming kernel).  Loads return in order, so "at most n outstanding" names
-// the n youngest; the counts below follow from the order of issue.  The wait hands the register set on as its
-// output, so nothing that reads it can be scheduled ahead of the wait.
+// never stored).  K is exactly 8 waves x U fragments (the launcher checks).
+// Straight-line code for one or two panels: in a loop whose iterations hand loads on to the next one, the compiler's
+// count of outstanding loads falls back to "wait for all of them" (a loop over panels took 14.7 us at M = 1 against
+// 10.8 for the streaming kernel).  The requests are separated by scheduler barriers, which keeps them in the order
+// written: left alone, the compiler reorders independent loads and then waits for the youngest.  (Loads issued and
+// waited for by hand, asm loads and a vmcnt wait that hands the registers on, are not an option: the compiler copies or
+// spills the destination registers between the load and the wait, before the data has arrived.)
 // Per-column post-op operands go to LDS the same way (wave 0, global_load_lds_dword) at the start of a panel.
 // Cross-wave reduction per panel through red[8 waves][16][2][MR] (MR = 16 or 32 rows), behind the regions.
 template <bool W8, int U>  // U: fragments per panel and wave (K = 8 waves x U fragments)
@@ -1165,7 +1166,9 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         // panel: 4096 x 4096 at M = 12 9.9 against 12.0, but 4096 x 11008 at M = 16 21.2 against 20.9), and over int8
         // weights wherever no workgroup has a second panel (4096 x 4096: M = 1 6.1 against 6.7 us, M = 4 6.4 against 8.0;
         // 8192 x 4096: M = 1 9.5 against 10.9); with two panels on some CUs and few rows the streaming form's two
-        // workgroups per CU are ahead (11008 columns, M = 1: 10.8 against 11.4 us).
+        // workgroups per CU are ahead (11008 columns, M = 1: 10.8 against 11.4 us; so they are against this kernel with one
+        // panel per workgroup and two workgroups per CU: 11.2 with 4 KiB per wave in flight, 10.8 with 2, and ahead only
+        // when every CU holds two, 16384 columns: 13.3 against 13.9 us; not kept).
         // decode_resident(): -1 by that rule (and only while decode_valu and decode_halves are left alone), 0 never,
         // 1 wherever the shape allows.
         const int rforce = decode_resident();
