@@ -407,7 +407,8 @@ def test_decode_valu_form(po, shape, out):
 # same order of the cross-wave sum).
 @pytest.mark.parametrize("case", [(True, 1, 4096, 352), (True, 16, 4096, 4096), (True, 10, 4096, 11008), (True, 16, 4096, 16384),
                                   (True, 5, 8192, 1000), (True, 4, 4096, 8200), (True, 6, 11008, 1000), (True, 1, 11008, 4096),
-                                  (True, 12, 5120, 704), (False, 12, 4096, 2000), (False, 16, 2048, 9000), (False, 3, 4096, 96)])
+                                  (True, 12, 5120, 704), (False, 12, 4096, 2000), (False, 16, 2048, 9000), (False, 3, 4096, 96),
+                                  (False, 24, 2048, 1000), (False, 19, 2048, 8300)])   # (more than 16 rows: the wider reduction scratch)
 @pytest.mark.parametrize("out", ["f32", "bf16", "i8"])
 def test_decode_resident_form(po, case, out):
     w8, M, K, N = case
