@@ -366,12 +366,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 // get zero weights and a clamped (finite) x.
 // WK: weights are bf16 (0), int8 (1) or int4 (2), 3: int8 weights and int8 activations (int32 sums);
 // XD: 16-byte x loads per thread per chunk (8 KiB of x each)
-template <int WK, int NP, int FPW, int XD>
+template <int WK, int NP, int FPW, int XD, int WIN = 0>  // WIN: chunks in flight (0: what the case's registers hold)
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void skinny_chunk_kernel(const SkinnyArgs s) {
     constexpr bool W8 = WK == 1, W4 = WK == 2, I8A = WK == 3;
     using accv = std::conditional_t<I8A, i32x16, f32x16>;
     // chunks in flight (what 128 registers hold)
-    constexpr int W = W4 ? (XD >= 4 ? 2 : 3) : ((FPW == 2 && (W8 || NP == 2)) ? 2 : 3);
+    constexpr int W = WIN ? WIN : (W4 ? (XD >= 4 ? 2 : 3) : ((FPW == 2 && (W8 || NP == 2)) ? 2 : 3));
     constexpr int XB = W4 ? 128 : (W8 ? 64 : 32);  // bytes of a row of x one fragment covers (int8 x int8: 32)
     constexpr int FC = 8 * FPW;          // fragments per chunk
     constexpr int RB = FC * XB;          // bytes of a row of x per chunk
@@ -1286,7 +1286,12 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
             if (M <= 16) MMX_CHUNKED(false, 2, 2, 1, panels / 2);
             else MMX_CHUNKED(false, 2, 1, 1, panels / 2);
         } else if (w8) {
-            if (M <= 16) MMX_CHUNKED(true, 1, 1, 1, panels);
+            // With at most one workgroup per CU, six chunks in flight instead of three (11008 x 4096 at M = 8 / 32: 22.0 / 27.4
+            // -> 19.1 / 24.7 us; 4096 x 4096 at M = 16: 10.4 -> 9.5); with two per CU three are better (4096 x 11008 at
+            // M = 16: 14.6 against 15.0), and nine no longer fit the registers.
+            if (panels <= num_cus() && M <= 16) hipLaunchKernelGGL((skinny_chunk_kernel<true, 1, 1, 1, 6>), dim3(panels), dim3(512), 32768, st, s);
+            else if (panels <= num_cus()) hipLaunchKernelGGL((skinny_chunk_kernel<true, 1, 1, 2, 6>), dim3(panels), dim3(512), 32768, st, s);
+            else if (M <= 16) MMX_CHUNKED(true, 1, 1, 1, panels);
             else MMX_CHUNKED(true, 1, 1, 2, panels);
         } else {
             if (M <= 16) MMX_CHUNKED(false, 1, 2, 1, panels);

@@ -461,6 +461,28 @@ def test_decode_resident_form(po, case, out):
         assert np.array_equal(res[1][0], res[0][0])
 
 
+# The chunked kernel (x too large for LDS, or a K the resident-x kernel does not exist for) with at most one workgroup per CU
+# keeps six chunks in flight instead of three: both row counts of its x buffers, a K that is not a whole number of chunks
+@pytest.mark.parametrize("shape", [(12, 6144, 704), (20, 6144, 512), (32, 4224, 96), (16, 7168, 1000)])
+def test_decode_chunked_few_panels(po, shape):
+    M, K, N = shape
+    rng = np.random.default_rng(17 * sum(shape))
+    x = rand_bf16(rng, (M, K), 1.0)
+    W = np.clip(np.rint(rng.standard_normal((K, N)) * 40), -127, 127).astype(np.int8)
+    scale = rng.uniform(1e-3, 5e-3, N).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    _, acc_ref = po.gemv_w8(x, W, scale, want_acc=True)
+    packed = mx.repack_b(dev(W))
+    acc = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc, mx.PP_NONE), b_dtype=mx.I8)
+    assert mx.last_kernel() == "skinny_chunk_w8", mx.last_kernel()
+    check_float_parity(host_bits(acc), acc_ref, f"chunked accumulators {shape}")
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_DEQUANT | mx.PP_BIAS, bias=dev(bias), deq_scale_per_oc=dev(scale)), b_dtype=mx.I8)
+    assert mx.last_kernel() == "skinny_chunk_w8"
+    assert np.array_equal(host_bits(y), po.pp(host_bits(acc), po.PP_DEQUANT | po.PP_BIAS, po.BF16, bias=bias, deq_per_oc=scale))
+
+
 def test_decode_resident_rule(po):
     """Left alone, the library takes the resident form where x is too large for two workgroups per CU and, over int8
     weights, wherever no workgroup has a second panel; shapes it does not cover keep their kernels."""
