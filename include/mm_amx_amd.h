@@ -210,9 +210,11 @@ const char* mmx_last_kernel(void);
  * streaming decode kernel at M = 1 over int8-compressed weights uses v_dot2_f32_bf16 and a cross-lane add
  * instead of the matrix cores — -1 (default) where at most one workgroup per CU is launched (it is the faster form
  * there), 0 never, 1 always; the two forms agree to fp32 summation order.  "decode_resident": whether a decode
- * launch (M <= 32, bf16 or int8-compressed weights, K a multiple of 512) whose x fits in one CU's LDS but not twice
- * runs as one workgroup per CU that keeps x there and walks the panels — -1 (default) where the streaming kernel does
- * not apply (x above 80 KiB), 0 never, 1 wherever x fits (same results as the streaming kernel). */
+ * launch (M <= 32; K = 4096, 5120, 8192 or 11008 over int8-compressed weights, 2048 or 4096 over bf16 weights; at
+ * most two 32-column panels per CU; x within a CU's LDS) runs as one workgroup per CU that keeps x in LDS and walks
+ * its one or two panels — -1 (default) where x is too large for the streaming kernel's two workgroups per CU and,
+ * over int8 weights, wherever no workgroup gets a second panel (and only while decode_halves and decode_valu are
+ * left at -1); 0 never; 1 wherever the shape allows (same bits as the streaming kernel). */
 int mmx_set_option(const char* name, int value);  /* like mmx_set_tile: affects the calling thread's later calls only */
 /* HIP-event timing of `iters` back-to-back launches of the given gemm on `stream`, launch i
  * using the packed weights Bpacked_rot[i % n_rot] (rotate over several copies so that a
