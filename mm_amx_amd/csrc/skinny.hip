@@ -523,7 +523,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 // 128 VGPRs at most: two workgroups per CU, so that every panel of an 11008-column matrix is resident at once.
 // ONE: every wave's share of K is a single batch (the common decode shapes); a variant of its own so that
 // each kernel holds one code path and stays within its registers.
-template <int WK, int NP, bool ONE>
+// UW: batch of the rolling window if not the full register set (the last batch of a wave's share of K is filled up with
+// repeats of the last load, which cost what they are a share of the loads: the launcher picks the batch with the fewest)
+template <int WK, int NP, bool ONE, int UW = 0>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void skinny_stream_kernel(const SkinnyArgs s, int zero_off) {
     constexpr bool W8 = WK == 1, W4 = WK == 2, I8A = WK == 3;  // 3: int8 weights AND int8 activations, int32 sums
     // 4: int8 weights and ONE row of x without the matrix cores: every lane owns one column and half of a fragment's
@@ -534,7 +536,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     using accv = std::conditional_t<I8A, i32x16, f32x16>;
     // fragments per panel per wave in flight at once (16 KiB of weights; int4: 8 KiB, a fragment holds 64 of k
     // and unpacking it costs more than streaming it)
-    constexpr int U = (W4 ? 8 : 16) / NP;
+    constexpr int U = UW ? UW : (W4 ? 8 : 16) / NP;
     // [M][K] bf16, then at zero_off a row of zeros; once x has been used up, the cross-wave reduction scratch
     // (the launcher allocates the larger of the two: stream_lds_bytes)
     extern __shared__ __attribute__((aligned(1024))) char xs[];
@@ -1066,6 +1068,50 @@ bool skinny_i8_eligible(const void* x, int64_t ldx, int M, int K) {
            ((ldx & 15) == 0);
 }
 
+// The rolling-window form of the half-panel kernel re-requests its loads in batches of U; the last batch is filled up
+// with repeats of the last load.  The repeats cost as much as they are a share of the loads (bf16 2560 x 10240 at
+// M = 1, 20 loads per wave: 14.7 us with batches of 16, 10.8 with 10; 11008 x 4096, 86 loads: 18.3 with 16, 16.8 with 8,
+// 17.4 with 10), so the batch with the fewest repeats is used; at equal repeats the larger one (4096 x 11008, 32 loads:
+// 16.8 / 17.7 us at M = 1 / 4 with 16, 16.7 / 18.3 with 8), over int8 weights the smaller (11008 x 4096: 11.2 with 8, 11.8
+// with 12).  Gate/up pairs: batches of 4 per panel (3: +3 %, 2: +5 %, 6: +38 %).
+typedef void (*HalfKernel)(const SkinnyArgs, int);
+template <bool W8, int NP>
+static HalfKernel half_window_kernel(int nfrag) {
+    if constexpr (NP == 2) {
+        return skinny_half_kernel<W8, 2, false, 4>;
+    } else {
+        const int n = ((nfrag >> 1) + 3) / 4;  // loads per wave
+        auto repeats = [n](int u) { return (n + u - 1) / u * u - n; };
+        if constexpr (W8) {
+            return repeats(12) < repeats(8) ? skinny_half_kernel<true, 1, false, 12> : skinny_half_kernel<true, 1, false, 8>;
+        } else {
+            int best = 16;
+            for (int u : {10, 8, 6})
+                if (repeats(u) < repeats(best)) best = u;
+            return best == 16 ? skinny_half_kernel<false, 1, false, 16>
+                              : (best == 10 ? skinny_half_kernel<false, 1, false, 10>
+                                            : (best == 8 ? skinny_half_kernel<false, 1, false, 8> : skinny_half_kernel<false, 1, false, 6>));
+        }
+    }
+}
+
+// the rolling-window form of the streaming kernel for a wave's share of per_wave fragments: batches of 16, 10 or 8
+// (single panels), whichever repeats the fewest loads, the larger at equal repeats (a share of 20 fragments in batches
+// of 16 is 12 repeats in 32 loads: int8 5120 x 13824 at M = 1 20.0 us, 14.3 in batches of 10; bf16 2560 x 10752 16.2 -> 12.0)
+typedef void (*StreamKernel)(const SkinnyArgs, int);
+template <bool W8, int NP>
+static StreamKernel stream_window_kernel(int per_wave) {
+    if constexpr (NP == 2) {
+        return skinny_stream_kernel<W8, 2, false>;
+    } else {
+        auto repeats = [per_wave](int u) { return (per_wave + u - 1) / u * u - per_wave; };
+        int best = 16;
+        for (int u : {10, 8})
+            if (repeats(u) < repeats(best)) best = u;
+        return best == 16 ? skinny_stream_kernel<W8, 1, false> : (best == 10 ? skinny_stream_kernel<W8, 1, false, 10> : skinny_stream_kernel<W8, 1, false, 8>);
+    }
+}
+
 // wk: weights are bf16 (0), int8 (1) or int4 (2); 3: int8 weights and int8 activations
 int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
                   const Epilogue& ep, hipStream_t st) {
@@ -1145,10 +1191,11 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         decode_halves() != 0 && panels <= num_cus() && (int64_t)s.nfrag * 512 >= 128 * 1024) {
         // A few rows of a long x (the MLP's down projection at M = 2-4: 66-110 KiB with the zero row) and at
         // most one half-panel per CU: the half-panel form with one workgroup per CU still has all of x in LDS.
-        typedef void (*HalfKernel)(const SkinnyArgs, int);
-        static std::atomic<uint64_t> attr_done[2];
-        const HalfKernel kernels[2] = {skinny_half_kernel<false, 1, true, 16>, skinny_half_kernel<false, 1, false, 16>};
-        for (int i = 0; i < 2; i++) {
+        static std::atomic<uint64_t> attr_done[5];
+        const HalfKernel kernels[5] = {skinny_half_kernel<false, 1, true, 16>, skinny_half_kernel<false, 1, false, 16>,
+                                       skinny_half_kernel<false, 1, false, 10>, skinny_half_kernel<false, 1, false, 8>,
+                                       skinny_half_kernel<false, 1, false, 6>};
+        for (int i = 0; i < 5; i++) {
             const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernels[i]), 128 * 1024, attr_done[i]);
             if (rc) return rc;
         }
@@ -1156,7 +1203,7 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         if (((s.nfrag >> 1) + 3) / 4 <= 16)
             hipLaunchKernelGGL((skinny_half_kernel<false, 1, true, 16>), dim3(2 * panels), dim3(256), xbytes, st, s, zero_off);
         else
-            hipLaunchKernelGGL((skinny_half_kernel<false, 1, false, 16>), dim3(2 * panels), dim3(256), xbytes, st, s, zero_off);
+            hipLaunchKernelGGL((half_window_kernel<false, 1>(s.nfrag)), dim3(2 * panels), dim3(256), xbytes, st, s, zero_off);
         return check_hip(hipGetLastError(), "skinny_half_kernel launch");
     }
     {
@@ -1205,11 +1252,12 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
     // form; with one workgroup per CU, M = 12-16, it loses: 16.6-17.7 against 13.7-14.5 us).
     const bool bigx = !pairs && xbytes > 46 * 1024 && xbytes <= 80 * 1024;
     if (bigx) {
-        typedef void (*StreamKernel)(const SkinnyArgs, int);
-        static std::atomic<uint64_t> attr_done[4];
-        const StreamKernel kernels[4] = {skinny_stream_kernel<0, 1, true>, skinny_stream_kernel<0, 1, false>,
-                                         skinny_stream_kernel<1, 1, true>, skinny_stream_kernel<1, 1, false>};
-        for (int i = 0; i < 4; i++) {
+        static std::atomic<uint64_t> attr_done[8];
+        const StreamKernel kernels[8] = {skinny_stream_kernel<0, 1, true>, skinny_stream_kernel<0, 1, false>,
+                                         skinny_stream_kernel<1, 1, true>, skinny_stream_kernel<1, 1, false>,
+                                         skinny_stream_kernel<0, 1, false, 10>, skinny_stream_kernel<0, 1, false, 8>,
+                                         skinny_stream_kernel<1, 1, false, 10>, skinny_stream_kernel<1, 1, false, 8>};
+        for (int i = 0; i < 8; i++) {
             const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernels[i]), 80 * 1024, attr_done[i]);
             if (rc) return rc;
         }
@@ -1236,11 +1284,11 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         if (halves && per_wave_h <= 16 / NP)                                                                         \
             hipLaunchKernelGGL((skinny_half_kernel<W8, NP, true, 16 / NP>), dim3(2 * (GRID)), dim3(256), xbytes, st, s, zero_off); \
         else if (halves) /* the rolling window holds fewer registers where two accumulator pairs need them */      \
-            hipLaunchKernelGGL((skinny_half_kernel<W8, NP, false, (NP == 2 ? 4 : (W8 ? 12 : 16))>), dim3(2 * (GRID)), dim3(256), xbytes, st, s, zero_off); \
+            hipLaunchKernelGGL((half_window_kernel<W8, NP>(s.nfrag)), dim3(2 * (GRID)), dim3(256), xbytes, st, s, zero_off); \
         else if (per_wave <= 16 / NP)                                                                                \
             hipLaunchKernelGGL((skinny_stream_kernel<W8, NP, true>), dim3(GRID), dim3(512), stream_lds_bytes(xbytes, NP), st, s, zero_off); \
         else                                                                                                         \
-            hipLaunchKernelGGL((skinny_stream_kernel<W8, NP, false>), dim3(GRID), dim3(512), stream_lds_bytes(xbytes, NP), st, s, zero_off); \
+            hipLaunchKernelGGL((stream_window_kernel<W8, NP>(per_wave)), dim3(GRID), dim3(512), stream_lds_bytes(xbytes, NP), st, s, zero_off); \
     } while (0)
         if (halves) note_kernel(pairs ? "skinny_half_bf16_gateup" : (w8 ? "skinny_half_w8" : "skinny_half_bf16"));
         // One row of x over int8 weights: a lane can own a column and half of a fragment's k (v_dot2_f32_bf16, one
@@ -1294,7 +1342,11 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
             else if (M <= 16) MMX_CHUNKED(true, 1, 1, 1, panels);
             else MMX_CHUNKED(true, 1, 1, 2, panels);
         } else {
-            if (M <= 16) MMX_CHUNKED(false, 1, 2, 1, panels);
+            // (six chunks in flight with at most one workgroup per CU, as above: 11008 x 4096 at M = 16 / 32 28.9 / 39.3 ->
+            // 26.2 / 34.1 us, 4096 x 4096 at M = 32 16.4 -> 14.6)
+            if (panels <= num_cus() && M <= 16) hipLaunchKernelGGL((skinny_chunk_kernel<false, 1, 2, 1, 6>), dim3(panels), dim3(512), 32768, st, s);
+            else if (panels <= num_cus()) hipLaunchKernelGGL((skinny_chunk_kernel<false, 1, 1, 1, 6>), dim3(panels), dim3(512), 32768, st, s);
+            else if (M <= 16) MMX_CHUNKED(false, 1, 2, 1, panels);
             else MMX_CHUNKED(false, 1, 1, 1, panels);
         }
 #undef MMX_CHUNKED
