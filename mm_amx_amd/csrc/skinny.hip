@@ -1095,21 +1095,31 @@ static HalfKernel half_window_kernel(int nfrag) {
     }
 }
 
-// the rolling-window form of the streaming kernel for a wave's share of per_wave fragments: batches of 16, 10 or 8
-// (single panels), whichever repeats the fewest loads, the larger at equal repeats (a share of 20 fragments in batches
-// of 16 is 12 repeats in 32 loads: int8 5120 x 13824 at M = 1 20.0 us, 14.3 in batches of 10; bf16 2560 x 10752 16.2 -> 12.0)
+// The streaming kernel for single panels and a wave's share of per_wave fragments.  Up to 16: one batch, of the smallest
+// register set that holds the share (a share of 10 in a set of 16 is 6 repeated loads and 6 multiplies by zero in 16: int8
+// 2560 x 10240 at M = 1 10.0 us against 7.6 for its bytes).  Beyond: the rolling window in batches of 16, 10 or 8,
+// whichever repeats the fewest loads, the larger at equal repeats (a share of 20 fragments in batches of 16 is 12 repeats
+// in 32 loads: int8 5120 x 13824 at M = 1 20.0 us, 14.3 in batches of 10; bf16 2560 x 10752 16.2 -> 12.0).
+// *index: the kernel's place in a list of STREAM_KERNELS per weight type (for per-kernel set-up).
 typedef void (*StreamKernel)(const SkinnyArgs, int);
-template <bool W8, int NP>
-static StreamKernel stream_window_kernel(int per_wave) {
-    if constexpr (NP == 2) {
-        return skinny_stream_kernel<W8, 2, false>;
+constexpr int STREAM_KERNELS = 9;
+template <int WK>
+static StreamKernel stream_kernel_for(int per_wave, int* index) {
+    static const StreamKernel list[STREAM_KERNELS] = {
+        skinny_stream_kernel<WK, 1, true, 4>,  skinny_stream_kernel<WK, 1, true, 6>,  skinny_stream_kernel<WK, 1, true, 8>,
+        skinny_stream_kernel<WK, 1, true, 10>, skinny_stream_kernel<WK, 1, true, 12>, skinny_stream_kernel<WK, 1, true>,
+        skinny_stream_kernel<WK, 1, false>,    skinny_stream_kernel<WK, 1, false, 10>, skinny_stream_kernel<WK, 1, false, 8>};
+    int i;
+    if (per_wave <= 16) {
+        i = per_wave <= 4 ? 0 : (per_wave <= 6 ? 1 : (per_wave <= 8 ? 2 : (per_wave <= 10 ? 3 : (per_wave <= 12 ? 4 : 5))));
     } else {
         auto repeats = [per_wave](int u) { return (per_wave + u - 1) / u * u - per_wave; };
-        int best = 16;
-        for (int u : {10, 8})
-            if (repeats(u) < repeats(best)) best = u;
-        return best == 16 ? skinny_stream_kernel<W8, 1, false> : (best == 10 ? skinny_stream_kernel<W8, 1, false, 10> : skinny_stream_kernel<W8, 1, false, 8>);
+        i = 6;
+        if (repeats(10) < repeats(16)) i = 7;
+        if (repeats(8) < repeats(i == 7 ? 10 : 16)) i = 8;
     }
+    *index = i;
+    return list[i];
 }
 
 // wk: weights are bf16 (0), int8 (1) or int4 (2); 3: int8 weights and int8 activations
@@ -1144,10 +1154,8 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
             return check_hip(hipGetLastError(), "skinny_chunk_kernel launch");
         }
         note_kernel("skinny_stream_i8");
-        if ((s.nfrag + 7) / 8 <= 16)
-            hipLaunchKernelGGL((skinny_stream_kernel<3, 1, true>), dim3(panels), dim3(512), stream_lds_bytes(zoff + K, 1), st, s, zoff);
-        else
-            hipLaunchKernelGGL((skinny_stream_kernel<3, 1, false>), dim3(panels), dim3(512), stream_lds_bytes(zoff + K, 1), st, s, zoff);
+        int unused;
+        hipLaunchKernelGGL(stream_kernel_for<3>((s.nfrag + 7) / 8, &unused), dim3(panels), dim3(512), stream_lds_bytes(zoff + K, 1), st, s, zoff);
         return check_hip(hipGetLastError(), "skinny_stream_kernel launch");
     }
     if (wk == 2) {
@@ -1251,22 +1259,18 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
     // be resident): 80 KiB of x each (4096 x 11008 int8 GEMV at M = 5-8: 13.0-13.4 -> 11.5-12.0 us against the chunked
     // form; with one workgroup per CU, M = 12-16, it loses: 16.6-17.7 against 13.7-14.5 us).
     const bool bigx = !pairs && xbytes > 46 * 1024 && xbytes <= 80 * 1024;
+    const int per_wave = (s.nfrag + 7) / 8;
+    int stream_index = 0;
+    const StreamKernel stream_kernel = w8 ? stream_kernel_for<1>(per_wave, &stream_index) : stream_kernel_for<0>(per_wave, &stream_index);
     if (bigx) {
-        static std::atomic<uint64_t> attr_done[8];
-        const StreamKernel kernels[8] = {skinny_stream_kernel<0, 1, true>, skinny_stream_kernel<0, 1, false>,
-                                         skinny_stream_kernel<1, 1, true>, skinny_stream_kernel<1, 1, false>,
-                                         skinny_stream_kernel<0, 1, false, 10>, skinny_stream_kernel<0, 1, false, 8>,
-                                         skinny_stream_kernel<1, 1, false, 10>, skinny_stream_kernel<1, 1, false, 8>};
-        for (int i = 0; i < 8; i++) {
-            const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kernels[i]), 80 * 1024, attr_done[i]);
-            if (rc) return rc;
-        }
+        static std::atomic<uint64_t> attr_done[2][STREAM_KERNELS];
+        const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(stream_kernel), 80 * 1024, attr_done[w8 ? 1 : 0][stream_index]);
+        if (rc) return rc;
     }
     if (kpad == K && (xbytes <= 46 * 1024 || bigx) && s.x_vec_ok) {
         // the activations fit in LDS: streaming variant
         if (pairs && (panels & 1)) return set_error(MMX_E_INVALID, "SILU_GATE needs an even number of 32-column panels");
         note_kernel(pairs ? (w8 ? "skinny_stream_w8_gateup" : "skinny_stream_bf16_gateup") : (w8 ? "skinny_stream_w8" : "skinny_stream_bf16"));
-        const int per_wave = (s.nfrag + 7) / 8;
         // Half-panel workgroups pay off for up to 4 rows of x (cheap enough to stage per workgroup) if each still has enough
         // weights to stream (measured at M = 1: bf16 units of 80 KiB gain 8 %, of 64 KiB lose to the fixed cost of a
         // workgroup; int8 units of 172 KiB gain 16 %, of 128 KiB lose 1 %, of 64 KiB 20 %) and the list is short enough for balance to matter: at most two rounds of resident
@@ -1285,10 +1289,12 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
             hipLaunchKernelGGL((skinny_half_kernel<W8, NP, true, 16 / NP>), dim3(2 * (GRID)), dim3(256), xbytes, st, s, zero_off); \
         else if (halves) /* the rolling window holds fewer registers where two accumulator pairs need them */      \
             hipLaunchKernelGGL((half_window_kernel<W8, NP>(s.nfrag)), dim3(2 * (GRID)), dim3(256), xbytes, st, s, zero_off); \
+        else if (NP == 1)                                                                                            \
+            hipLaunchKernelGGL(stream_kernel, dim3(GRID), dim3(512), stream_lds_bytes(xbytes, 1), st, s, zero_off);       \
         else if (per_wave <= 16 / NP)                                                                                \
             hipLaunchKernelGGL((skinny_stream_kernel<W8, NP, true>), dim3(GRID), dim3(512), stream_lds_bytes(xbytes, NP), st, s, zero_off); \
         else                                                                                                         \
-            hipLaunchKernelGGL((stream_window_kernel<W8, NP>(per_wave)), dim3(GRID), dim3(512), stream_lds_bytes(xbytes, NP), st, s, zero_off); \
+            hipLaunchKernelGGL((skinny_stream_kernel<W8, NP, false>), dim3(GRID), dim3(512), stream_lds_bytes(xbytes, NP), st, s, zero_off); \
     } while (0)
         if (halves) note_kernel(pairs ? "skinny_half_bf16_gateup" : (w8 ? "skinny_half_w8" : "skinny_half_bf16"));
         // One row of x over int8 weights: a lane can own a column and half of a fragment's k (v_dot2_f32_bf16, one
@@ -1301,8 +1307,8 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         const bool valu = w8 && M == 1 && !pairs && !halves && !bigx && vforce != 0 && (vforce == 1 || panels <= num_cus());
         if (valu) {
             note_kernel("skinny_stream_w8_valu");
-            if (per_wave <= 16) hipLaunchKernelGGL((skinny_stream_kernel<4, 1, true>), dim3(panels), dim3(512), stream_lds_bytes(xbytes, 1), st, s, zero_off);
-            else hipLaunchKernelGGL((skinny_stream_kernel<4, 1, false>), dim3(panels), dim3(512), stream_lds_bytes(xbytes, 1), st, s, zero_off);
+            int unused;
+            hipLaunchKernelGGL(stream_kernel_for<4>(per_wave, &unused), dim3(panels), dim3(512), stream_lds_bytes(xbytes, 1), st, s, zero_off);
         } else if (pairs && w8) {
             if (per_wave <= 8) hipLaunchKernelGGL((skinny_stream_kernel<1, 2, true>), dim3(panels / 2), dim3(512), stream_lds_bytes(xbytes, 2), st, s, zero_off);
             else hipLaunchKernelGGL((skinny_stream_kernel<1, 2, false>), dim3(panels / 2), dim3(512), stream_lds_bytes(xbytes, 2), st, s, zero_off);
