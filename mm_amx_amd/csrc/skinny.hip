@@ -1170,7 +1170,11 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
                     hipLaunchKernelGGL((skinny_stream_kernel<2, 2, true>), dim3(panels / 2), dim3(512), stream_lds_bytes(xb, 2), st, s, zoff);
                 else
                     hipLaunchKernelGGL((skinny_stream_kernel<2, 2, false>), dim3(panels / 2), dim3(512), stream_lds_bytes(xb, 2), st, s, zoff);
-            } else if ((s.nfrag + 7) / 8 <= 8)
+            } else if ((s.nfrag + 7) / 8 <= 4)  // (register sets sized to the share of K, as for the other weight types)
+                hipLaunchKernelGGL((skinny_stream_kernel<2, 1, true, 4>), dim3(panels), dim3(512), stream_lds_bytes(xb, 1), st, s, zoff);
+            else if ((s.nfrag + 7) / 8 <= 6)
+                hipLaunchKernelGGL((skinny_stream_kernel<2, 1, true, 6>), dim3(panels), dim3(512), stream_lds_bytes(xb, 1), st, s, zoff);
+            else if ((s.nfrag + 7) / 8 <= 8)
                 hipLaunchKernelGGL((skinny_stream_kernel<2, 1, true>), dim3(panels), dim3(512), stream_lds_bytes(xb, 1), st, s, zoff);
             else
                 hipLaunchKernelGGL((skinny_stream_kernel<2, 1, false>), dim3(panels), dim3(512), stream_lds_bytes(xb, 1), st, s, zoff);

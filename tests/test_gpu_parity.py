@@ -981,7 +981,7 @@ def test_int4_quantise_non_finite_weights(po):
 
 
 @pytest.mark.parametrize("shape", [(1, 256, 64), (3, 320, 100), (16, 337, 96), (32, 2560, 192), (2, 4096, 352), (4, 8192, 64),
-                                   (8, 4096, 352), (20, 1024, 100), (16, 11008, 64)])
+                                   (8, 4096, 352), (20, 1024, 100), (16, 11008, 64), (2, 2560, 96)])
 def test_int4_decode_shapes(po, shape):
     M, K, N = shape
     rng = np.random.default_rng(sum(shape))
