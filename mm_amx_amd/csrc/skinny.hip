@@ -715,10 +715,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 // Cross-wave reduction per panel through red[8 waves][16][2][MR] (MR = 16 or 32 rows), behind the regions.
 template <bool W8, int U>  // U: fragments per panel and wave (K = 8 waves x U fragments)
 __global__ __launch_bounds__(512) void skinny_resident_kernel(const SkinnyArgs s, int region, int red_off, int mr_log2) {
-    // Fragments (KiB) a wave keeps in flight.  More is worse: a wave is held at a request until the CU accepts it
+    // Fragments (KiB) a wave keeps in flight.  More is worse at K = 4096: a wave is held at a request until the CU accepts it
     // (4096 x 11008 int8 at M = 16: 13.0 us with 4, 13.1 with 8, 14.1 with 16; 3: 13.3, 2: 14.3; a deeper window for the
     // workgroups with two panels only: 6: 13.0, 8: 13.1, 12: 13.6).
-    constexpr int D = 4;
+    constexpr int D = U >= 32 ? 8 : 4;  // (a long K with one workgroup per CU: 8192 x 8192 at M = 1 15.1 -> 14.1 us with 8)
     constexpr int XB = W8 ? 64 : 32;    // bytes of a row of x that one fragment covers
     extern __shared__ __attribute__((aligned(1024))) char xs[];
     float* const red = reinterpret_cast<float*>(xs + red_off);
@@ -1242,7 +1242,11 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         const bool shape_ok = kpad == K && s.x_vec_ok && !pairs && k_ok && panels > 0 &&
                               panels <= 2 * num_cus() && lds <= 160 * 1024;
         const bool one_each = panels <= num_cus();
-        const bool by_rule = (xbytes > 80 * 1024 && (w8 || one_each)) || (w8 && one_each && decode_valu() == -1 && decode_halves() == -1);
+        // (two panels on some CUs: ahead of the chunked form while a good part of the CUs has one, 344 or 432 panels on 256
+        // CUs; with two on every CU, 8192 x 16384 at M = 8, the chunked form's two workgroups per CU win, 24.5 against 26.0 us)
+        const bool some_two = !one_each && panels * 4 <= 7 * num_cus();
+        const bool by_rule = (xbytes > 80 * 1024 && (one_each || (w8 && some_two))) ||
+                             (w8 && one_each && decode_valu() == -1 && decode_halves() == -1);
         if (shape_ok && rforce != 0 && (rforce == 1 || by_rule)) {
             typedef void (*ResidentKernel)(const SkinnyArgs, int, int, int);
             static std::atomic<uint64_t> attr_done[6];
