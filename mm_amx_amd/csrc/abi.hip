@@ -356,7 +356,7 @@ int mmx_set_tile(const char* shape) {
     if (!shape || !*shape) { g_forced = {0, 0}; return MMX_OK; }
     int bm = 0, bn = 0;
     if (sscanf(shape, "%dx%d", &bm, &bn) != 2) return set_error(MMX_E_INVALID, "mmx_set_tile: cannot parse '%s'", shape);
-    if (!((bm == 256 && (bn == 256 || bn == 192)) || (bm == 128 && (bn == 256 || bn == 192 || bn == 128 || bn == 64))))
+    if (!((bm == 256 && (bn == 256 || bn == 192)) || (bm == 128 && (bn == 256 || bn == 192 || bn == 128 || bn == 64)) || (bm == 64 && bn == 128)))
         return set_error(MMX_E_INVALID, "mmx_set_tile: no kernel for %dx%d", bm, bn);
     g_forced = {bm, bn};
     return MMX_OK;

@@ -197,7 +197,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4,
     // int8 weights under bf16 A: every wave converts the fragments it multiplies, so the waves sit side by side
     // (four columns of waves in the 256-column tiles; a wave keeps two panels, which the gate/up store needs):
     // a fragment is then converted by NW/4 waves instead of NW/2
-    constexpr int WGN = (W8 && BN == 256) ? 4 : (BN >= 128 ? 2 : 1), WGM = NW / WGN;
+    constexpr int WGN = (W8 && (BN == 256 || BM == 64)) ? 4 : (BN >= 128 ? 2 : 1), WGM = NW / WGN;
     constexpr int WM = BM / WGM, WN = BN / WGN;
     constexpr int MI = WM / 32, NJ = WN / 32;
     constexpr int A_BYTES = BM * 128, B_BYTES = BN / 32 * BP_IT, STAGE = A_BYTES + B_BYTES;
@@ -1002,7 +1002,7 @@ struct Plan {
 // A K split is considered where the slices of all tiles are resident at once.
 static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, bool wide_only, int mode, const SplitRequest& rq) {
     static const struct { int bm, bn; float eff; } cand[] = {
-        {256, 256, 0.92f}, {256, 192, 0.90f}, {128, 256, 0.86f}, {128, 192, 0.84f}, {128, 128, 0.80f}, {128, 64, 0.70f}};
+        {256, 256, 0.92f}, {256, 192, 0.90f}, {128, 256, 0.86f}, {128, 192, 0.84f}, {128, 128, 0.80f}, {128, 64, 0.70f}, {64, 128, 0.70f}};
     const TileCfg f = forced_tile();
     const int cus = num_cus();
     // measured: a CU takes 36.6 bytes per clock from L2 with all CUs pulling; parking a 64 KiB partial tile and counting
@@ -1014,8 +1014,9 @@ static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, bool w
         if (f.bm && (f.bm != c.bm || f.bn != c.bn)) continue;
         if (need_pairs && (c.bn % 128) != 0) continue;
         if (wide_only && c.bn == 64) continue;                      // (no 64-column tile for int8 weights under bf16 A)
+        if ((!wide_only || need_pairs) && c.bm == 64) continue;     // (the 64-row tile: for int8 weights under bf16 A, no gate/up pairs)
         if (mode == 3 && !(c.bm == 128 && c.bn == 128)) continue;   // the masked path exists for one tile shape
-        if (mode != 2 && c.bn == 64) continue;                      // the 64-wide tile exists for the ring pipeline only
+        if (mode != 2 && (c.bn == 64 || c.bm == 64)) continue;      // the 64-wide and 64-row tiles exist for the ring pipeline only
         const int tiles = ((M + c.bm - 1) / c.bm) * ((Ncols + c.bn - 1) / c.bn);
         for (int S = 1; S <= KSPLIT_MAX; S++) {
             if (rq.k_splits > 0 && S != rq.k_splits) continue;
@@ -1029,7 +1030,8 @@ static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, bool w
             const int kit = S > 1 ? slice_kiters(nk, S) : nk;
             // int8 weights under bf16 A: every wave converts its own fragments, 12 vector instructions per MFMA operand,
             // which a block of only two row-blocks per wave cannot hide behind its MFMAs (measured issue efficiencies)
-            const float eff = !wide_only ? c.eff : (c.bm == 256 ? 0.85f : (c.bn == 256 ? 0.62f : (c.bn == 192 ? 0.60f : 0.50f)));
+            // (64 rows: one row-block pair per converted fragment; measured 980 cycles per k-iteration)
+            const float eff = !wide_only ? c.eff : (c.bm == 256 ? 0.85f : (c.bm == 64 ? 0.26f : (c.bn == 256 ? 0.62f : (c.bn == 192 ? 0.60f : 0.50f))));
             const float mfma = (float)(c.bm * c.bn / 32) / eff, bytes = (float)((c.bm + c.bn) * 128) / l1_bytes_per_clk;
             const float loop = (float)kit * (mfma > bytes ? mfma : bytes);
             const float epi = (float)(c.bm * c.bn / 256) * 100.0f;  // between a plain store (45) and a GELU (170): the plan must
@@ -1102,6 +1104,10 @@ static int launch_tiles(const GemmArgs& g, TileCfg t, int mode, int grid, hipStr
     if (t.bm == 128 && t.bn == 192) return MMX_LAUNCH_MODES(TIn, 128, 192, TOut);
     if constexpr (!Mfma<TIn>::W8) {
         if (t.bm == 128 && t.bn == 64 && mode == 2 && g.ksplit == 1) return MMX_LAUNCH(TIn, 128, 64, 2, TOut, 1);  // ring pipeline only
+    }
+    if constexpr (Mfma<TIn>::W8) {
+        if (t.bm == 64 && t.bn == 128 && mode == 2)  // ring pipeline only
+            return g.ksplit > 1 ? MMX_LAUNCH(TIn, 64, 128, 2, TOut, KSPLIT_MAX) : MMX_LAUNCH(TIn, 64, 128, 2, TOut, 1);
     }
     return set_error(MMX_E_UNSUPPORTED, "no MFMA tile kernel for %dx%d", t.bm, t.bn);
 }
