@@ -194,8 +194,8 @@ int mmx_mlp_splitk(const void* x, int64_t ldx_bytes, const void* w_gate_up, cons
                    void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- introspection / tuning (no reference counterpart) --------------------------------------- */
-/* Force the MFMA tile shape ("256x256", "256x192", "128x256", "128x192", "128x128", "128x64", "64x128" (int8-compressed
- * weights under bf16 activations with aligned operands only; otherwise 128x128 is used), "" = automatic)
+/* Force the MFMA tile shape ("256x256", "256x192", "128x256", "128x192", "128x128", "128x64", "64x128" (aligned
+ * operands and no SILU_GATE only; otherwise 128x128 is used), "" = automatic)
  * for the calling thread's later calls. */
 int mmx_set_tile(const char* shape);
 /* Name of the kernel variant the last mmx_gemm call of this thread launched. */

@@ -1002,7 +1002,8 @@ struct Plan {
 // A K split is considered where the slices of all tiles are resident at once.
 static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, bool wide_only, int mode, const SplitRequest& rq) {
     static const struct { int bm, bn; float eff; } cand[] = {
-        {256, 256, 0.92f}, {256, 192, 0.90f}, {128, 256, 0.86f}, {128, 192, 0.84f}, {128, 128, 0.80f}, {128, 64, 0.70f}, {64, 128, 0.70f}};
+        {256, 256, 0.92f}, {256, 192, 0.90f}, {128, 256, 0.86f}, {128, 192, 0.84f}, {128, 128, 0.80f}, {128, 64, 0.70f},
+        {64, 128, 0.27f}};  // (64 rows: two MFMAs per k-step and wave leave the loads nothing to hide behind: 940 cycles per k-iteration)
     const TileCfg f = forced_tile();
     const int cus = num_cus();
     // measured: a CU takes 36.6 bytes per clock from L2 with all CUs pulling; parking a 64 KiB partial tile and counting
@@ -1014,7 +1015,7 @@ static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, bool w
         if (f.bm && (f.bm != c.bm || f.bn != c.bn)) continue;
         if (need_pairs && (c.bn % 128) != 0) continue;
         if (wide_only && c.bn == 64) continue;                      // (no 64-column tile for int8 weights under bf16 A)
-        if ((!wide_only || need_pairs) && c.bm == 64) continue;     // (the 64-row tile: for int8 weights under bf16 A, no gate/up pairs)
+        if (need_pairs && c.bm == 64) continue;                     // (the 64-row tile stores no gate/up pairs)
         if (mode == 3 && !(c.bm == 128 && c.bn == 128)) continue;   // the masked path exists for one tile shape
         if (mode != 2 && (c.bn == 64 || c.bm == 64)) continue;      // the 64-wide and 64-row tiles exist for the ring pipeline only
         const int tiles = ((M + c.bm - 1) / c.bm) * ((Ncols + c.bn - 1) / c.bn);
@@ -1105,7 +1106,7 @@ static int launch_tiles(const GemmArgs& g, TileCfg t, int mode, int grid, hipStr
     if constexpr (!Mfma<TIn>::W8) {
         if (t.bm == 128 && t.bn == 64 && mode == 2 && g.ksplit == 1) return MMX_LAUNCH(TIn, 128, 64, 2, TOut, 1);  // ring pipeline only
     }
-    if constexpr (Mfma<TIn>::W8) {
+    {
         if (t.bm == 64 && t.bn == 128 && mode == 2)  // ring pipeline only
             return g.ksplit > 1 ? MMX_LAUNCH(TIn, 64, 128, 2, TOut, KSPLIT_MAX) : MMX_LAUNCH(TIn, 64, 128, 2, TOut, 1);
     }

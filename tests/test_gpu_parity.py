@@ -83,7 +83,7 @@ def test_bf16_exact_inputs_are_bit_exact(po):
     assert np.array_equal(host_bits(C), po.gemm_bf16(A, B))
 
 
-@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x192", "128x128", "128x64"])
+@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x192", "128x128", "128x64", "64x128"])
 @pytest.mark.parametrize("mode", [0, 2])
 def test_bf16_bias_gelu_every_kernel_variant(po, tile, mode):
     M, K, N = 600, 512, 832
@@ -92,8 +92,8 @@ def test_bf16_bias_gelu_every_kernel_variant(po, tile, mode):
     bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
     acc_ref = po.gemm_bf16(A, B)
     ref = po.pp(acc_ref, po.PP_BIAS | po.PP_GELU, po.BF16, bias=bias)
-    if tile == "128x64" and mode != 2:
-        pytest.skip("the 64-wide tile exists for the ring pipeline only")
+    if tile in ("128x64", "64x128") and mode != 2:
+        pytest.skip("the 64-wide and 64-row tiles exist for the ring pipeline only")
     mx.set_tile(tile)
     mx.set_option("load_mode", mode)
     try:
@@ -180,7 +180,7 @@ def test_int8_accumulators_bit_exact(po, shape):
     assert np.array_equal(host_bits(C), po.gemm_i8(A, B))
 
 
-@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x192", "128x128", "128x64"])
+@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x192", "128x128", "128x64", "64x128"])
 @pytest.mark.parametrize("mode", [0, 2])
 def test_int8_requant_every_kernel_variant(po, tile, mode):
     M, K, N = 520, 1024, 704
@@ -191,8 +191,8 @@ def test_int8_requant_every_kernel_variant(po, tile, mode):
     bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
     steps = po.PP_DEQUANT | po.PP_BIAS | po.PP_QUANT
     ref = po.pp(po.gemm_i8(A, B), steps, po.I8, bias=bias, deq_per_oc=deq, q=20.0)
-    if tile == "128x64" and mode != 2:
-        pytest.skip("the 64-wide tile exists for the ring pipeline only")
+    if tile in ("128x64", "64x128") and mode != 2:
+        pytest.skip("the 64-wide and 64-row tiles exist for the ring pipeline only")
     mx.set_tile(tile)
     mx.set_option("load_mode", mode)
     try:
@@ -1171,7 +1171,7 @@ def ws():
     assert not w[:16 << 10].any().item(), "the arrival counters must be left at zero"
 
 
-@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x192", "128x128"])
+@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x192", "128x128", "64x128"])
 @pytest.mark.parametrize("S", [2, 3, 4])
 def test_ksplit_int8_bit_exact(po, ws, tile, S):
     """int32 partial sums add exactly in any order: raw sums and requantised outputs equal the oracle's bits."""
@@ -1200,7 +1200,7 @@ def test_ksplit_int8_bit_exact(po, ws, tile, S):
         mx.set_tile("")
 
 
-@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x192", "128x128"])
+@pytest.mark.parametrize("tile", ["256x256", "256x192", "128x256", "128x192", "128x128", "64x128"])
 @pytest.mark.parametrize("S", [2, 3, 4])
 def test_ksplit_bf16_fixed_order(po, ws, tile, S):
     """fp32 partial sums are added in slice order whatever slice arrives last: repeated launches give the same
