@@ -290,13 +290,14 @@ def test_decode_small_shapes(po, shape, w8, no_resident_form):
         ref = po.pp(acc_ref, po.PP_BIAS | po.PP_GELU, po.F32, bias=bias)
         packed = mx.repack_b(dev_bf16(W))
         y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
-        mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_BIAS | mx.PP_GELU, bias=dev(bias)))
+        # k_splits = 1: at 24-32 rows the stream's own workspace would bring in the 64-row tile with a K split
+        mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_BIAS | mx.PP_GELU, bias=dev(bias)), k_splits=1)
     assert "skinny" in mx.last_kernel()
     if K >= 4096:   # x in LDS: the streaming kernel or, for few rows of a long K, its half-panel form
         assert "skinny_stream" in mx.last_kernel() or "skinny_half" in mx.last_kernel(), mx.last_kernel()
     # raw accumulators through the same kernel, then the oracle's post-op on them must give y's bits
     acc_gpu = torch.zeros((M, N), dtype=torch.float32, device="cuda")
-    mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc_gpu, mx.PP_NONE), b_dtype=mx.I8 if w8 else None)
+    mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc_gpu, mx.PP_NONE), b_dtype=mx.I8 if w8 else None, k_splits=1)
     check_float_parity(host_bits(acc_gpu), acc_ref, f"decode accumulators {shape} w8={w8}")
     steps = (po.PP_DEQUANT if w8 else 0) | po.PP_BIAS | po.PP_GELU
     again = po.pp(host_bits(acc_gpu), steps, po.F32, bias=bias, deq_per_oc=scale if w8 else None)
@@ -1310,6 +1311,39 @@ def test_ksplit_requests_that_cannot_be_met(ws):
         mx.gemm(A, gu, 256, mx.Epilogue(h, mx.PP_SILU_GATE), k_splits=2, ws=ws)
     assert mx.gemm_workspace_bytes(mx.BF16, mx.BF16, 64, 1024, 256, k_splits=2) > 16 << 10
     assert mx.gemm_workspace_bytes(mx.BF16, mx.BF16, 64, 1024, 256, k_splits=1) == 0
+
+
+@pytest.mark.parametrize("shape", [(24, 8192, 512), (32, 4096, 1024), (17, 8192, 256), (32, 11008, 100)])
+def test_few_rows_take_the_split_tile_when_a_workspace_is_given(po, ws, shape):
+    """17-32 rows over bf16 weights with no more panels than CUs: with a workspace the 64-row tile with a K split
+    runs in place of the chunked decode kernel; with k_splits = 1, or below 24 rows over a short K, the decode kernel stays.
+    Both meet the oracle's accumulators within the bar, and the fused post-op is the oracle's on those accumulators."""
+    M, K, N = shape
+    rng = np.random.default_rng(7 * sum(shape))
+    A, B = rand_bf16(rng, (M, K), 1.0), rand_bf16(rng, (K, N), 0.05)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    acc_ref = po.gemm_bf16(A, B)
+    Ad, packed = dev_bf16(A), mx.repack_b(dev_bf16(B))
+    acc = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    mx.gemm(Ad, packed, N, mx.Epilogue(acc, mx.PP_NONE), ws=ws)
+    if K % 64 == 0:
+        assert "64x128" in mx.last_kernel() and "ksplit" in mx.last_kernel(), mx.last_kernel()
+    else:
+        assert mx.last_kernel().startswith("skinny_"), mx.last_kernel()
+    check_float_parity(host_bits(acc), acc_ref, f"few rows, split tile {shape}")
+    C = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    mx.gemm(Ad, packed, N, mx.Epilogue(C, mx.PP_BIAS | mx.PP_GELU, bias=dev(bias)), ws=ws)
+    assert np.array_equal(host_bits(C), po.pp(host_bits(acc), po.PP_BIAS | po.PP_GELU, po.BF16, bias=bias))
+    again = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    mx.gemm(Ad, packed, N, mx.Epilogue(again, mx.PP_NONE), ws=ws)
+    assert np.array_equal(host_bits(again), host_bits(acc))
+    plain = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    mx.gemm(Ad, packed, N, mx.Epilogue(plain, mx.PP_NONE), k_splits=1)
+    assert mx.last_kernel().startswith("skinny_"), mx.last_kernel()
+    check_float_parity(host_bits(plain), acc_ref, f"few rows, decode kernel {shape}")
+    if M > 17:
+        mx.gemm(Ad[:17, :4096], mx.repack_b(dev_bf16(B[:4096])), N, mx.Epilogue(plain[:17], mx.PP_NONE), ws=ws)
+        assert mx.last_kernel().startswith("skinny_"), mx.last_kernel()
 
 
 @pytest.mark.parametrize("M", [64, 300])
