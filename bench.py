@@ -35,7 +35,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 MEASURED_TRAFFIC = {
     "gemm_bf16_256x192_ring8w_out_bf16": {"bytes": (81702.5 * 2.000 + 27474.0 * 1.000) * 1024, "source": "mm_amx_amd/csrc/gemm_tile.hpp",
                                           "sha": "e4f113cc1ef35526"},
-    "skinny_stream_w8": {"bytes": (22154.3 * 2.000 + 39.7 * 1.000) * 1024, "source": "mm_amx_amd/csrc/skinny.hip", "sha": "6ee5505f6c43943b"},
+    "skinny_stream_w8": {"bytes": (22154.3 * 2.000 + 39.7 * 1.000) * 1024, "source": "mm_amx_amd/csrc/skinny.hip", "sha": "defcc5419ef21ea7"},
 }
 
 
@@ -432,6 +432,28 @@ def main():
             sweepn[str(Nn)] = ent
             del packs, Wn
         extra["decode_gemv_int8w_K4096_M1_sweep_N"] = sweepn
+
+        # Decode shapes with a panel for at most every second CU: the chunked kernel whole (k_splits = 1) and with K cut
+        # into slices over several workgroups (k_splits = 0 with a workspace), weights rotated over 540 MB
+        ksp = {}
+        for w8k, Mk, Kk, Nk in ((True, 16, 11008, 4096), (True, 32, 11008, 4096), (True, 32, 8192, 1024),
+                                (False, 16, 11008, 4096), (False, 32, 11008, 4096), (False, 32, 8192, 1024)):
+            nbk = Kk * Nk * (1 if w8k else 2)
+            if w8k:
+                Wk = mx.repack_b(torch.randint(-127, 128, (Kk, Nk), dtype=torch.int8, device="cuda"))
+            else:
+                Wk = mx.repack_b((torch.randn((Kk, Nk), dtype=torch.float32, device="cuda") * 0.02).to(torch.bfloat16))
+            packs = [Wk] + [Wk.clone() for _ in range(max(2, int(540e6 // nbk)) - 1)]
+            xk = torch.randn((Mk, Kk), dtype=torch.float32, device="cuda").to(torch.bfloat16)
+            epk = mx.Epilogue(torch.zeros((Mk, Nk), dtype=torch.bfloat16, device="cuda"), mx.PP_NONE)
+            kwk = {"b_dtype": mx.I8} if w8k else {}
+            entk = {}
+            for label, ks in (("whole", 1), ("split", 0)):
+                msk = avg_ms(xk, packs, Nk, epk, 200, k_splits=ks, **kwk)
+                entk[label] = {"us": round(msk * 1e3, 2), "kernel": mx.last_kernel(), "weight_GBps": round(nbk / msk / 1e6, 0)}
+            ksp[f"{'int8w' if w8k else 'bf16'}_M{Mk}_K{Kk}_N{Nk}"] = entk
+            del packs, Wk
+        extra["decode_k_split"] = ksp
 
         # Steady state of a chain of decode layers (the topology of main.cpp:660-711: A1 x B1 -> A2, A2 x B2 -> A1, ...,
         # one set of weights per layer): 12 pairs of [1,4096] x [4096,11008] and [1,11008] x [11008,4096] over int8

@@ -135,9 +135,7 @@ int mmx_dequant_packed(const void* packed_i8, int K, int N, void* packed_bf16, v
  * A is [M, K] row-major with row stride lda_bytes; Bpacked comes from mmx_repack_b for the
  * FULL [K, N]; n0 % 32 == 0, 0 <= n0 < n1 <= N.  M <= 32 takes the bandwidth-bound decode
  * kernel (the M<=16 paths of the reference and weight_compression/fc16m.cpp:451-502), larger
- * M the MFMA tile kernel.  (One exception, through mmx_gemm_splitk only: 17 <= M <= 32 over bf16 weights with a
- * workspace and k_splits != 1 takes a 64-row tile with a K split where that is the faster kernel: few output
- * columns, a long K.) */
+ * M the MFMA tile kernel. */
 int mmx_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* Bpacked, int M, int K,
              int N, int n0, int n1, const mmx_epilogue* ep, void* stream);
 
@@ -150,8 +148,11 @@ int mmx_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const v
  * adds them in slice order (so the result does not depend on the arrival order) and applies the post-op.  It
  * pays where a shape has fewer tiles than the GPU has CUs, or tiles bound by the bytes a CU can pull in.
  *   k_splits  0 = the library chooses (possibly no split), 1 = none, 2..4 = exactly that many slices
- *             (MMX_E_INVALID if K is too short or the workspace too small, MMX_E_UNSUPPORTED for M <= 32
- *             where the decode kernel runs, SILU_GATE, unaligned A or K * sizeof(T) not a multiple of 128).
+ *             (MMX_E_INVALID if K is too short or the workspace too small, MMX_E_UNSUPPORTED for M <= 32,
+ *             SILU_GATE, unaligned A or K * sizeof(T) not a multiple of 128).  The decode kernels (M <= 32)
+ *             take 0 or 1 only: with 0 and a workspace, bf16 activations over bf16 or int8 weights whose x does
+ *             not fit in LDS and whose column range has a 32-column panel for at most every second CU walk K in
+ *             2-4 slices of their own choosing, combined the same way (same layout of the workspace).
  *   workspace device memory, 256-byte aligned, mmx_gemm_workspace_bytes() or more (64 MiB + 16 KiB always
  *             suffices for k_splits = 0; with less, the choice is restricted to what fits).  Its first 16 KiB are
  *             arrival counters: zero them once after allocation; every call leaves them zero.  Calls that share
@@ -189,8 +190,8 @@ int mmx_mlp(const void* x, int64_t ldx_bytes, const void* w_gate_up, const void*
             void* y, int64_t ldy_bytes, int M, int K, int N, void* stream);
 
 /* The same with the down projection's K split over `down_k_splits` slices (0 = the library chooses, 2 = the
- * reference's do_splitK, tests/amx-mlp.cpp:768 and :560-593); workspace as for mmx_gemm_splitk.  M <= 16 (decode
- * kernels) and workspace = NULL run without slices; at 17 <= M <= 32 the library chooses unless down_k_splits = 1. */
+ * reference's do_splitK, tests/amx-mlp.cpp:768 and :560-593); workspace as for mmx_gemm_splitk.  workspace = NULL
+ * runs without slices; at M <= 32 (decode kernels) the library chooses unless down_k_splits = 1. */
 int mmx_mlp_splitk(const void* x, int64_t ldx_bytes, const void* w_gate_up, const void* w_down, void* h,
                    int64_t ldh_bytes, void* y, int64_t ldy_bytes, int M, int K, int N, int down_k_splits,
                    void* workspace, size_t workspace_bytes, void* stream);

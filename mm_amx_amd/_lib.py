@@ -382,7 +382,7 @@ def mlp(x, w_gate_up, w_down, N, h=None, y=None, down_k_splits=0, ws=None):
     if y is None:
         y = torch.empty((M, K), dtype=torch.bfloat16, device=x.device)
     _dev(h, "h"), _dev(y, "y")
-    ks, wsp, wsb = _split_args(x, down_k_splits, ws) if M > 16 else (1, None, 0)
+    ks, wsp, wsb = _split_args(x, down_k_splits, ws)
     _check(lib().mmx_mlp_splitk(x.data_ptr(), _row_stride_bytes(x), w_gate_up.data_ptr(), w_down.data_ptr(), h.data_ptr(),
                                 _row_stride_bytes(h), y.data_ptr(), _row_stride_bytes(y), M, K, N, ks, wsp, wsb, _stream()))
     return h, y

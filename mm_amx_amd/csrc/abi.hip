@@ -61,7 +61,7 @@ int ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& don
 }
 
 
-bool few_rows_prefer_tiles_bf16(const void* A, int64_t lda, int M, int K, int Ncols, uint32_t steps, const SplitRequest& rq);
+size_t skinny_workspace_bytes(int wk, int M, int K, int n0, int n1);
 int launch_gemm_tiles_bf16(const void* A, int64_t lda, const void* Bp, int M, int K, int N, int n0, int n1,
                            const Epilogue& ep, const SplitRequest& rq, hipStream_t st);
 int launch_gemm_tiles_i8(const void* A, int64_t lda, const void* Bp, int M, int K, int N, int n0, int n1,
@@ -71,7 +71,7 @@ int launch_gemm_tiles_w8(const void* A, int64_t lda, const void* Bp, int M, int 
 size_t plan_workspace_bytes(int elesz, bool w8, int M, int K, int Ncols, uint32_t steps, int k_splits);
 bool skinny_i8_eligible(const void* x, int64_t ldx, int M, int K);
 int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
-                  const Epilogue& ep, hipStream_t st);
+                  const Epilogue& ep, hipStream_t st, const SplitRequest* rq);
 int launch_repack(int elesz, const void* B, int64_t ldb, int K, int N, int transpose, void* out, hipStream_t st);
 int launch_repack_gate_up(const void* wg, const void* wu, int64_t ldw, int K, int N, void* out, hipStream_t st);
 int launch_quantize(const void* W, int64_t ldw, int rows, int cols, void* Wq, int64_t ldq, float* scales_out,
@@ -172,14 +172,13 @@ static int gemm_dispatch(int a_dtype, int b_dtype, const void* A, int64_t lda_by
     if (rc) return rc;
     if (rq.k_splits < 0) return set_error(MMX_E_INVALID, "mmx_gemm: k_splits = %d", rq.k_splits);
     if (rq.ws && (reinterpret_cast<uintptr_t>(rq.ws) & 255)) return set_error(MMX_E_INVALID, "mmx_gemm: the workspace must be 256-byte aligned");
-    // the decode kernels walk the whole of K in one workgroup per panel: they take no explicit K split
-    const bool few_rows_tiles = bf && few_rows_prefer_tiles_bf16(A, lda_bytes, M, K, n1 - n0, ep.steps, rq);
-    const bool decode = (M <= 32 && !i8 && !few_rows_tiles) || (i8 && skinny_i8_eligible(A, lda_bytes, M, K) && forced_tile().bm == 0);
-    if (decode && rq.k_splits > 1) return set_error(MMX_E_UNSUPPORTED, "mmx_gemm: the decode kernels (M <= 32) take no K split");
+    // the decode kernels choose their own K split (the chunked form, given a workspace); they take no count of slices
+    const bool decode = (M <= 32 && !i8) || (i8 && skinny_i8_eligible(A, lda_bytes, M, K) && forced_tile().bm == 0);
+    if (decode && rq.k_splits > 1) return set_error(MMX_E_UNSUPPORTED, "mmx_gemm: the decode kernels (M <= 32) take k_splits = 0 or 1, not a count of slices");
     if ((ep.steps & MMX_PP_SILU_GATE) && ((n1 - n0) % 64)) return set_error(MMX_E_INVALID, "mmx_gemm: SILU_GATE needs (n1 - n0) %% 64 == 0");
-    if (M <= 32 && !i8 && !few_rows_tiles) return launch_skinny(w4 ? 2 : (w8 ? 1 : 0), A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st);
+    if (M <= 32 && !i8) return launch_skinny(w4 ? 2 : (w8 ? 1 : 0), A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st, &rq);
     if (i8 && skinny_i8_eligible(A, lda_bytes, M, K) && forced_tile().bm == 0)
-        return launch_skinny(3, A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st);
+        return launch_skinny(3, A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, st, nullptr);
     if (w4) return set_error(MMX_E_UNSUPPORTED, "mmx_gemm: bf16 x int4-weight is a decode path (M <= 32)");
     if (w8) return launch_gemm_tiles_w8(A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, rq, st);
     return i8 ? launch_gemm_tiles_i8(A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, rq, st)
@@ -310,7 +309,9 @@ int mmx_gemm_splitk_static(int a_dtype, int b_dtype, const void* A, int64_t lda_
 size_t mmx_gemm_workspace_bytes(int a_dtype, int b_dtype, int M, int K, int N, int n0, int n1, uint32_t steps, int k_splits) {
     const bool bf = a_dtype == MMX_BF16 && b_dtype == MMX_BF16, i8 = a_dtype == MMX_I8 && b_dtype == MMX_I8;
     const bool w8 = a_dtype == MMX_BF16 && b_dtype == MMX_I8;
-    if ((!bf && !i8 && !w8) || M <= (bf ? 16 : 32) || K <= 0 || N <= 0 || n0 < 0 || n1 > N || n0 >= n1 || k_splits < 0) return 0;
+    if (M > 0 && M <= 32 && (bf || w8) && K > 0 && N > 0 && n0 >= 0 && n1 <= N && n0 < n1)
+        return k_splits == 0 && !(steps & MMX_PP_SILU_GATE) ? skinny_workspace_bytes(w8 ? 1 : 0, M, K, n0, n1) : 0;
+    if ((!bf && !i8 && !w8) || M <= 32 || K <= 0 || N <= 0 || n0 < 0 || n1 > N || n0 >= n1 || k_splits < 0) return 0;
     return plan_workspace_bytes(i8 ? 1 : 2, w8, M, K, n1 - n0, steps, k_splits);
 }
 
@@ -349,8 +350,8 @@ int mmx_mlp_splitk(const void* x, int64_t ldx_bytes, const void* w_gate_up, cons
     e2.ldc_bytes = ldy_bytes;
     // AMX_MLP::MLP::setup builds `down` with do_splitK (tests/amx-mlp.cpp:768): two halves of its K blocks, summed
     // and rounded to bf16 by the half that finishes last (:648-682).  The decode kernels (M <= 32) sum K inside one
-    // workgroup and take no slices; at 17-32 rows the library may still take a split tile of its own choosing.
-    if (M <= 16 || !workspace || (M <= 32 && down_k_splits == 1))
+    // workgroup per panel or in slices of their own choosing (never a given count).
+    if (!workspace || (M <= 32 && down_k_splits == 1))
         return mmx_gemm(MMX_BF16, MMX_BF16, h, ldh_bytes, w_down, M, N, K, 0, K, &e2, stream);
     if (M <= 32) down_k_splits = 0;
     return mmx_gemm_splitk(MMX_BF16, MMX_BF16, h, ldh_bytes, w_down, M, N, K, 0, K, &e2, down_k_splits, workspace, workspace_bytes, stream);

@@ -38,6 +38,11 @@ struct SkinnyArgs {
     int n0, n1;
     int x_vec_ok;
     Epilogue ep;
+    // K split of the chunked kernel (kslices > 1): slice blockIdx.y walks its share of the chunks, parks its sums in
+    // ws_part and counts itself in at ws_cnt[blockIdx.x]; the slice that arrives last adds them up and stores
+    char* ws_part;
+    uint32_t* ws_cnt;
+    int kslices;
 };
 
 __device__ __forceinline__ bf16x8 load_x8(const char* xrow, int k0, int K, bool live, bool vec_ok) {
@@ -117,10 +122,85 @@ __device__ __forceinline__ void skinny_prefetch(const SkinnyArgs& s, int panel_f
 }
 
 // cross-wave reduction of the partial 32x32 blocks + post-op + store (shared by the 8-wave decode kernels)
-template <int NP, bool ISUM = false>  // ISUM: the partial sums are int32 (int8 activations), stored as bits
+// ISUM: the partial sums are int32 (int8 activations), stored as bits.
+// SPLIT: the workgroup holds one of s.kslices slices of K.  It writes its sums to the workspace at device scope (sc1:
+// through to the level all XCDs share), waits until the stores have been acknowledged and counts itself in with a
+// device-scope atomicInc that wraps to zero on the last arrival (ready for the next launch).  The last to arrive adds
+// the slices' sums in slice order 0, 1, 2, ... - so the result does not depend on who came last - and goes on to the
+// post-op; the others are done.  Nobody waits for anybody.
+template <int NP, bool ISUM = false, bool SPLIT = false>
 __device__ __forceinline__ void skinny_finish(const SkinnyArgs& s, const float (&red)[8][NP][16][64], int panel_first, int tid,
-                                              const FinishOperands<NP>& o) {
+                                              const FinishOperands<NP>& o, int slice = 0) {
     const Epilogue& ep = s.ep;
+    float fsum[2][NP];
+    int isum2[2][NP];
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int idx = tid + 512 * t;
+        const int v = idx >> 6, ln = idx & 63;
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            if constexpr (ISUM) {
+                int acc = 0;
+#pragma unroll
+                for (int w8 = 0; w8 < 8; w8++) acc += reinterpret_cast<const int*>(&red[w8][p][v][ln])[0];
+                isum2[t][p] = acc;
+            } else {
+                float acc = 0.0f;
+#pragma unroll
+                for (int w8 = 0; w8 < 8; w8++) acc += red[w8][p][v][ln];
+                fsum[t][p] = acc;
+            }
+        }
+    }
+    if constexpr (SPLIT) {
+        const int S = s.kslices;
+        if (S > 1) {
+            constexpr int AUX_SC1 = 16;             // cache policy operand of the buffer instructions: device scope
+            constexpr int UNIT = 2 * NP * 512 * 4;  // bytes of one workgroup's sums
+            __amdgpu_buffer_rsrc_t parts =
+                __builtin_amdgcn_make_buffer_rsrc(s.ws_part + (int64_t)blockIdx.x * S * UNIT, 0, S * UNIT, 0x00020000);
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int p = 0; p < NP; p++) {
+                    uint32_t bits;
+                    if constexpr (ISUM) bits = (uint32_t)isum2[t][p];
+                    else bits = __builtin_bit_cast(uint32_t, fsum[t][p]);
+                    __builtin_amdgcn_raw_buffer_store_b32(bits, parts, slice * UNIT + ((t * NP + p) * 512 + tid) * 4, 0, AUX_SC1);
+                }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // every store of this wave has been acknowledged
+            __syncthreads();                                  // ... and every read of the reduction scratch is done
+            volatile uint32_t* flag = reinterpret_cast<volatile uint32_t*>(const_cast<float*>(&red[0][0][0][0]));
+            if (tid == 0) *flag = atomicInc(s.ws_cnt + blockIdx.x, (uint32_t)S - 1u);
+            __syncthreads();
+            if (*flag != (uint32_t)S - 1u) return;
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int p = 0; p < NP; p++) {
+                    float fa = 0.0f;
+                    int ia = 0;
+#pragma unroll
+                    for (int sl = 0; sl < 4; sl++) {
+                        if (sl < S) {
+                            uint32_t bits;
+                            if (sl == slice) {
+                                if constexpr (ISUM) bits = (uint32_t)isum2[t][p];
+                                else bits = __builtin_bit_cast(uint32_t, fsum[t][p]);
+                            } else {
+                                bits = __builtin_amdgcn_raw_buffer_load_b32(parts, sl * UNIT + ((t * NP + p) * 512 + tid) * 4, 0, AUX_SC1);
+                            }
+                            if constexpr (ISUM) ia = sl == 0 ? (int)bits : ia + (int)bits;
+                            else fa = sl == 0 ? __builtin_bit_cast(float, bits) : fa + __builtin_bit_cast(float, bits);
+                        }
+                    }
+                    if constexpr (ISUM) isum2[t][p] = ia;
+                    else fsum[t][p] = fa;
+                }
+        }
+    }
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         const int idx = tid + 512 * t;
@@ -133,16 +213,10 @@ __device__ __forceinline__ void skinny_finish(const SkinnyArgs& s, const float (
 #pragma unroll
         for (int p = 0; p < NP; p++) {
             if constexpr (ISUM) {
-                int acc = 0;
-#pragma unroll
-                for (int w8 = 0; w8 < 8; w8++) acc += reinterpret_cast<const int*>(&red[w8][p][v][ln])[0];
-                isum[p] = acc;
-                sum[p] = (float)acc;  // vcvtdq2ps, round to nearest even (include/kernels_amx.hpp:631-634)
+                isum[p] = isum2[t][p];
+                sum[p] = (float)isum2[t][p];  // vcvtdq2ps, round to nearest even (include/kernels_amx.hpp:631-634)
             } else {
-                float acc = 0.0f;
-#pragma unroll
-                for (int w8 = 0; w8 < 8; w8++) acc += red[w8][p][v][ln];
-                sum[p] = acc;
+                sum[p] = fsum[t][p];
             }
         }
         if (ISUM && ep.out_dtype == MMX_I32) {  // raw accumulators (steps == 0)
@@ -397,7 +471,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         for (int v = 0; v < 16; v++) acc[p][v] = 0;
 
     const int f_last = s.nfrag - 1;
-    const int nchunk = (s.nfrag + FC - 1) / FC;
+    // chunks [chunk0, nchunk) are this workgroup's: all of them, or slice blockIdx.y of kslices equal shares
+    const int nchunk_all = (s.nfrag + FC - 1) / FC;
+    const int slice = s.kslices > 1 ? (int)blockIdx.y : 0;
+    const int per_slice = (nchunk_all + s.kslices - 1) / s.kslices;
+    const int chunk0 = slice * per_slice;
+    const int nchunk = chunk0 + per_slice < nchunk_all ? chunk0 + per_slice : nchunk_all;
     const int row_bytes = s.K * (I8A ? 1 : 2);
     const char* wbase[NP];
 #pragma unroll
@@ -485,9 +564,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 
     skinny_static_for<0, W>([&](auto j_c) {
         constexpr int J = decltype(j_c)::value;
-        if (J < nchunk) MMX_LOAD(J, J);
+        if (chunk0 + J < nchunk) MMX_LOAD(chunk0 + J, J);
     });
-    for (int c0 = 0; c0 < nchunk; c0 += W) {
+    for (int c0 = chunk0; c0 < nchunk; c0 += W) {
         skinny_static_for<0, W>([&](auto j_c) {
             constexpr int J = decltype(j_c)::value;
             if (c0 + J < nchunk) {
@@ -508,7 +587,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             else red[wave][p][v][lane] = W4 ? acc[p][v] * 16.0f : acc[p][v];  // int4 operands were q / 16
         }
     __syncthreads();
-    skinny_finish<NP, I8A>(s, red, panel_first, tid, fin);
+    if constexpr (WIN != 0 && NP == 1) skinny_finish<NP, I8A, true>(s, red, panel_first, tid, fin, slice);  // (the forms launched with a K split)
+    else skinny_finish<NP, I8A>(s, red, panel_first, tid, fin);
 }
 
 // ---- streaming variant for the smallest M -----------------------------------------------------------
@@ -1059,6 +1139,34 @@ int decode_resident();
 // int8 x int8 at M <= 32 can use the decode kernels if x is 16-byte aligned and K fills whole 128-byte groups of
 // the packed weights: the streaming form if x fits in LDS, else the chunked one, which walks K in chunks of 256
 // dynamic LDS of skinny_stream_kernel: x + the zero row, reused afterwards as the reduction scratch (32 KiB per panel)
+// Workspace of a K split: arrival counters first (one per workgroup column, zero between launches), the slices' sums after
+// them - the layout the tile kernels use, so one workspace serves both.
+constexpr int SPLIT_MAX_PANELS = 4096;
+constexpr size_t SPLIT_COUNTER_BYTES = (size_t)SPLIT_MAX_PANELS * 4;
+
+// Slices of K for the chunked kernel: with a panel for at most every second CU the workgroups of a panel walk K in 2-4
+// slices, none empty and each at least four chunks long, and the last to arrive adds them up (int8 weights, weights
+// rotated over 540 MB: 11008 x 4096 at M = 16 / 32 20.4 / 25.1 -> 14.5 / 17.3 us, 8192 x 1024 15.5 / 19.0 -> 9.1 / 10.5;
+// bf16 weights: 11008 x 4096 at M = 16 / 32 26.7 / 34.7 -> 19.4 / 22.4, 8192 x 1024 19.7 / 25.4 -> 10.3 / 11.5).
+static int chunk_slices(bool w8, int M, int nfrag, int panels, size_t ws_bytes) {
+    if (panels <= 0 || panels * 2 > num_cus() || panels > SPLIT_MAX_PANELS) return 1;
+    const int fc = (!w8 && M <= 16) ? 16 : 8;  // fragments per chunk of the kernels launched for these shapes
+    const int nchunk = (nfrag + fc - 1) / fc;
+    int S = num_cus() / panels < 4 ? num_cus() / panels : 4;
+    while (S > 1 && ((nchunk + S - 1) / S < 4 || (S - 1) * ((nchunk + S - 1) / S) >= nchunk ||
+                     SPLIT_COUNTER_BYTES + (size_t)panels * S * 4096 > ws_bytes))
+        S--;
+    return S;
+}
+
+// Bytes of workspace a decode launch of this shape can use (0: it takes no K split)
+size_t skinny_workspace_bytes(int wk, int M, int K, int n0, int n1) {
+    const int nfrag = (K * (wk == 1 ? 1 : 2) + 127) / 128 * 128 / 32;
+    const int panels = ((n1 + 31) >> 5) - (n0 >> 5);
+    const int S = chunk_slices(wk == 1, M, nfrag, panels, ~(size_t)0);
+    return S > 1 ? SPLIT_COUNTER_BYTES + (size_t)panels * S * 4096 : 0;
+}
+
 static inline int stream_lds_bytes(int xbytes, int np) { return xbytes > 32768 * np ? xbytes : 32768 * np; }
 
 bool skinny_i8_eligible(const void* x, int64_t ldx, int M, int K) {
@@ -1124,7 +1232,7 @@ static StreamKernel stream_kernel_for(int per_wave, int* index) {
 
 // wk: weights are bf16 (0), int8 (1) or int4 (2); 3: int8 weights and int8 activations
 int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
-                  const Epilogue& ep, hipStream_t st) {
+                  const Epilogue& ep, hipStream_t st, const SplitRequest* rq) {
     const bool w8 = wk == 1;
     // the byte counts below are 32-bit: M <= 32 rows of at most 2^24 elements
     if (M > 32 || K > (1 << 24)) return set_error(MMX_E_UNSUPPORTED, "decode kernels take M <= 32 and K <= 2^24 (got M = %d, K = %d)", M, K);
@@ -1142,6 +1250,9 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
     s.n1 = n1;
     s.x_vec_ok = ((reinterpret_cast<uintptr_t>(x) & 15) == 0) && ((ldx & 15) == 0);
     s.ep = ep;
+    s.ws_part = nullptr;
+    s.ws_cnt = nullptr;
+    s.kslices = 1;
     const int panels = ((n1 + 31) >> 5) - (n0 >> 5);
     const bool pairs = (ep.steps & MMX_PP_SILU_GATE) != 0;
     if (wk == 3) {
@@ -1326,7 +1437,10 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
 #undef MMX_STREAM
         return check_hip(hipGetLastError(), "skinny_stream_kernel launch");
     }
-    if (kpad == K && s.x_vec_ok && !w8 && !pairs && M <= 8) {
+    // K split of the chunked kernel (a workspace at hand, the library left to choose)
+    const int ksl = (kpad == K && s.x_vec_ok && !pairs && wk <= 1 && rq && rq->ws && rq->k_splits == 0)
+                        ? chunk_slices(w8, M, s.nfrag, panels, rq->ws_bytes) : 1;
+    if (kpad == K && s.x_vec_ok && !w8 && !pairs && M <= 8 && ksl == 1) {
         // aligned, x too large for LDS, few rows, plain bf16 weights: every lane reads its own part of x
         // (measured: for int8 weights and for gate/up pairs the chunked kernel below is faster at these M too)
         note_kernel("skinny_direct_bf16");
@@ -1343,6 +1457,16 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         constexpr int lds_ = (2 * 8 * XD * 1024) > (8 * NP * 16 * 64 * 4) ? (2 * 8 * XD * 1024) : (8 * NP * 16 * 64 * 4); \
         hipLaunchKernelGGL((skinny_chunk_kernel<W8, NP, FPW, XD>), dim3(GRID), dim3(512), lds_, st, s);            \
     } while (0)
+        dim3 grid(panels);
+        if (ksl > 1) {
+            s.ws_cnt = reinterpret_cast<uint32_t*>(rq->ws);
+            s.ws_part = rq->ws + SPLIT_COUNTER_BYTES;
+            s.kslices = ksl;
+            grid = dim3(panels, ksl);
+            static const char* const names[2][3] = {{"skinny_chunk_bf16_ksplit2", "skinny_chunk_bf16_ksplit3", "skinny_chunk_bf16_ksplit4"},
+                                                    {"skinny_chunk_w8_ksplit2", "skinny_chunk_w8_ksplit3", "skinny_chunk_w8_ksplit4"}};
+            note_kernel(names[w8][ksl - 2]);
+        }
         // rows of x per buffer = 8 KiB * XD / (8 * FPW fragments * 64 or 32 bytes)
         if (pairs) {
             if (M <= 16) MMX_CHUNKED(false, 2, 2, 1, panels / 2);
@@ -1351,15 +1475,15 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
             // With at most one workgroup per CU, six chunks in flight instead of three (11008 x 4096 at M = 8 / 32: 22.0 / 27.4
             // -> 19.1 / 24.7 us; 4096 x 4096 at M = 16: 10.4 -> 9.5); with two per CU three are better (4096 x 11008 at
             // M = 16: 14.6 against 15.0), and nine no longer fit the registers.
-            if (panels <= num_cus() && M <= 16) hipLaunchKernelGGL((skinny_chunk_kernel<true, 1, 1, 1, 6>), dim3(panels), dim3(512), 32768, st, s);
-            else if (panels <= num_cus()) hipLaunchKernelGGL((skinny_chunk_kernel<true, 1, 1, 2, 6>), dim3(panels), dim3(512), 32768, st, s);
+            if (panels <= num_cus() && M <= 16) hipLaunchKernelGGL((skinny_chunk_kernel<true, 1, 1, 1, 6>), grid, dim3(512), 32768, st, s);
+            else if (panels <= num_cus()) hipLaunchKernelGGL((skinny_chunk_kernel<true, 1, 1, 2, 6>), grid, dim3(512), 32768, st, s);
             else if (M <= 16) MMX_CHUNKED(true, 1, 1, 1, panels);
             else MMX_CHUNKED(true, 1, 1, 2, panels);
         } else {
             // (six chunks in flight with at most one workgroup per CU, as above: 11008 x 4096 at M = 16 / 32 28.9 / 39.3 ->
             // 26.2 / 34.1 us, 4096 x 4096 at M = 32 16.4 -> 14.6)
-            if (panels <= num_cus() && M <= 16) hipLaunchKernelGGL((skinny_chunk_kernel<false, 1, 2, 1, 6>), dim3(panels), dim3(512), 32768, st, s);
-            else if (panels <= num_cus()) hipLaunchKernelGGL((skinny_chunk_kernel<false, 1, 1, 1, 6>), dim3(panels), dim3(512), 32768, st, s);
+            if (panels <= num_cus() && M <= 16) hipLaunchKernelGGL((skinny_chunk_kernel<false, 1, 2, 1, 6>), grid, dim3(512), 32768, st, s);
+            else if (panels <= num_cus()) hipLaunchKernelGGL((skinny_chunk_kernel<false, 1, 1, 1, 6>), grid, dim3(512), 32768, st, s);
             else if (M <= 16) MMX_CHUNKED(false, 1, 2, 1, panels);
             else MMX_CHUNKED(false, 1, 1, 1, panels);
         }

@@ -282,7 +282,7 @@ def test_decode_small_shapes(po, shape, w8, no_resident_form):
         packed = mx.repack_b(dev(W))
         y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
         mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_DEQUANT | mx.PP_BIAS | mx.PP_GELU, bias=dev(bias),
-                                                    deq_scale_per_oc=dev(scale)), b_dtype=mx.I8)
+                                                    deq_scale_per_oc=dev(scale)), b_dtype=mx.I8, k_splits=1)
     else:
         W = rand_bf16(rng, (K, N), 0.05)
         scale = None
@@ -290,7 +290,7 @@ def test_decode_small_shapes(po, shape, w8, no_resident_form):
         ref = po.pp(acc_ref, po.PP_BIAS | po.PP_GELU, po.F32, bias=bias)
         packed = mx.repack_b(dev_bf16(W))
         y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
-        # k_splits = 1: at 24-32 rows the stream's own workspace would bring in the 64-row tile with a K split
+        # k_splits = 1: with the stream's own workspace the chunked kernel would split K over several workgroups
         mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_BIAS | mx.PP_GELU, bias=dev(bias)), k_splits=1)
     assert "skinny" in mx.last_kernel()
     if K >= 4096:   # x in LDS: the streaming kernel or, for few rows of a long K, its half-panel form
@@ -476,11 +476,11 @@ def test_decode_chunked_few_panels(po, shape):
     _, acc_ref = po.gemv_w8(x, W, scale, want_acc=True)
     packed = mx.repack_b(dev(W))
     acc = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
-    mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc, mx.PP_NONE), b_dtype=mx.I8)
+    mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc, mx.PP_NONE), b_dtype=mx.I8, k_splits=1)
     assert mx.last_kernel() == "skinny_chunk_w8", mx.last_kernel()
     check_float_parity(host_bits(acc), acc_ref, f"chunked accumulators {shape}")
     y = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
-    mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_DEQUANT | mx.PP_BIAS, bias=dev(bias), deq_scale_per_oc=dev(scale)), b_dtype=mx.I8)
+    mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_DEQUANT | mx.PP_BIAS, bias=dev(bias), deq_scale_per_oc=dev(scale)), b_dtype=mx.I8, k_splits=1)
     assert mx.last_kernel() == "skinny_chunk_w8"
     assert np.array_equal(host_bits(y), po.pp(host_bits(acc), po.PP_DEQUANT | po.PP_BIAS, po.BF16, bias=bias, deq_per_oc=scale))
 
@@ -497,7 +497,7 @@ def test_decode_resident_rule(po):
         else:
             packed, kw = mx.repack_b(dev_bf16(rand_bf16(rng, (K, N), 0.05))), {}
         y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
-        mx.gemm(x, packed, N, mx.Epilogue(y, mx.PP_NONE), **kw)
+        mx.gemm(x, packed, N, mx.Epilogue(y, mx.PP_NONE), k_splits=1, **kw)
         return mx.last_kernel()
 
     assert kernel_for(True, 16, 4096, 11008) == "skinny_resident_w8"
@@ -1313,37 +1313,91 @@ def test_ksplit_requests_that_cannot_be_met(ws):
     assert mx.gemm_workspace_bytes(mx.BF16, mx.BF16, 64, 1024, 256, k_splits=1) == 0
 
 
-@pytest.mark.parametrize("shape", [(24, 8192, 512), (32, 4096, 1024), (17, 8192, 256), (32, 11008, 100)])
-def test_few_rows_take_the_split_tile_when_a_workspace_is_given(po, ws, shape):
-    """17-32 rows over bf16 weights with no more panels than CUs: with a workspace the 64-row tile with a K split
-    runs in place of the chunked decode kernel; with k_splits = 1, or below 24 rows over a short K, the decode kernel stays.
-    Both meet the oracle's accumulators within the bar, and the fused post-op is the oracle's on those accumulators."""
-    M, K, N = shape
-    rng = np.random.default_rng(7 * sum(shape))
-    A, B = rand_bf16(rng, (M, K), 1.0), rand_bf16(rng, (K, N), 0.05)
+# K split of the chunked decode kernel: few panels (at most one for every second CU), x too large for LDS, a workspace
+# and k_splits = 0.  2-4 slices, ragged N, a column range, a last slice shorter than the others, every store type.
+@pytest.mark.parametrize("case", [(True, 16, 8192, 1024), (True, 32, 11008, 1000), (True, 24, 4096, 4096), (True, 20, 5120, 1280),
+                                  (False, 16, 8192, 512), (False, 32, 11008, 200), (False, 24, 4096, 4096), (False, 12, 9216, 96),
+                                  (False, 32, 2560, 2560), (True, 17, 4352, 300)])
+def test_decode_k_split(po, ws, case):
+    w8, M, K, N = case
+    rng = np.random.default_rng(11 * (M + K + N) + int(w8))
+    x = rand_bf16(rng, (M, K), 1.0)
     bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
-    acc_ref = po.gemm_bf16(A, B)
-    Ad, packed = dev_bf16(A), mx.repack_b(dev_bf16(B))
-    acc = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
-    mx.gemm(Ad, packed, N, mx.Epilogue(acc, mx.PP_NONE), ws=ws)
-    if K % 64 == 0:
-        assert "64x128" in mx.last_kernel() and "ksplit" in mx.last_kernel(), mx.last_kernel()
+    qs = rng.uniform(10.0, 30.0, N).astype(np.float32)
+    if w8:
+        W = np.clip(np.rint(rng.standard_normal((K, N)) * 40), -127, 127).astype(np.int8)
+        scale = rng.uniform(1e-3, 5e-3, N).astype(np.float32)
+        _, acc_ref = po.gemv_w8(x, W, scale, want_acc=True)
+        packed, kw = mx.repack_b(dev(W)), {"b_dtype": mx.I8}
+        steps, pos = mx.PP_DEQUANT | mx.PP_BIAS | mx.PP_GELU, po.PP_DEQUANT | po.PP_BIAS | po.PP_GELU
+        opd, opo = {"bias": dev(bias), "deq_scale_per_oc": dev(scale)}, {"bias": bias, "deq_per_oc": scale}
     else:
-        assert mx.last_kernel().startswith("skinny_"), mx.last_kernel()
-    check_float_parity(host_bits(acc), acc_ref, f"few rows, split tile {shape}")
-    C = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
-    mx.gemm(Ad, packed, N, mx.Epilogue(C, mx.PP_BIAS | mx.PP_GELU, bias=dev(bias)), ws=ws)
-    assert np.array_equal(host_bits(C), po.pp(host_bits(acc), po.PP_BIAS | po.PP_GELU, po.BF16, bias=bias))
-    again = torch.zeros((M, N), dtype=torch.float32, device="cuda")
-    mx.gemm(Ad, packed, N, mx.Epilogue(again, mx.PP_NONE), ws=ws)
-    assert np.array_equal(host_bits(again), host_bits(acc))
+        W = rand_bf16(rng, (K, N), 0.05)
+        acc_ref = po.gemm_bf16(x, W)
+        packed, kw = mx.repack_b(dev_bf16(W)), {}
+        steps, pos = mx.PP_BIAS | mx.PP_GELU, po.PP_BIAS | po.PP_GELU
+        opd, opo = {"bias": dev(bias)}, {"bias": bias}
+    xd = dev_bf16(x)
+    want = "skinny_chunk_w8_ksplit" if w8 else "skinny_chunk_bf16_ksplit"
+    accs = []
+    for rep in range(3):
+        acc = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        mx.gemm(xd, packed, N, mx.Epilogue(acc, mx.PP_NONE), ws=ws, **kw)
+        assert mx.last_kernel().startswith(want), mx.last_kernel()
+        accs.append(host_bits(acc))
+    assert np.array_equal(accs[0], accs[1]) and np.array_equal(accs[0], accs[2])   # slices are added in slice order
+    check_float_parity(accs[0], acc_ref, f"decode K split accumulators {case}")
+    # the fused stores are the oracle's post-op on the GPU's own sums
+    y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    mx.gemm(xd, packed, N, mx.Epilogue(y, steps, **opd), ws=ws, **kw)
+    assert mx.last_kernel().startswith(want)
+    assert np.array_equal(host_bits(y), po.pp(accs[0], pos, po.F32, **opo))
+    yb = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    mx.gemm(xd, packed, N, mx.Epilogue(yb, steps, **opd), ws=ws, **kw)
+    assert np.array_equal(host_bits(yb), po.pp(accs[0], pos, po.BF16, **opo))
+    y8 = torch.zeros((M, N), dtype=torch.int8, device="cuda")
+    mx.gemm(xd, packed, N, mx.Epilogue(y8, steps | mx.PP_QUANT, q_scale_per_oc=dev(qs), **opd), ws=ws, **kw)
+    assert np.array_equal(host_bits(y8), po.pp(accs[0], pos | po.PP_QUANT, po.I8, q_per_oc=qs, **opo))
+    # a column range: the rest of C is left alone
+    if N >= 200:
+        n0, n1 = 32, N - 5
+        part = torch.full((M, N), -3.0, dtype=torch.float32, device="cuda")
+        mx.gemm(xd, packed, N, mx.Epilogue(part, mx.PP_NONE), n0=n0, n1=n1, ws=ws, **kw)
+        assert mx.last_kernel().startswith(want)
+        got = host_bits(part)
+        assert np.array_equal(got[:, n0:n1], accs[0][:, n0:n1])
+        assert np.all(got[:, :n0] == -3.0) and np.all(got[:, n1:] == -3.0)
+    # k_splits = 1: the unsplit kernel, within the same bar
     plain = torch.zeros((M, N), dtype=torch.float32, device="cuda")
-    mx.gemm(Ad, packed, N, mx.Epilogue(plain, mx.PP_NONE), k_splits=1)
-    assert mx.last_kernel().startswith("skinny_"), mx.last_kernel()
-    check_float_parity(host_bits(plain), acc_ref, f"few rows, decode kernel {shape}")
-    if M > 17:
-        mx.gemm(Ad[:17, :4096], mx.repack_b(dev_bf16(B[:4096])), N, mx.Epilogue(plain[:17], mx.PP_NONE), ws=ws)
-        assert mx.last_kernel().startswith("skinny_"), mx.last_kernel()
+    mx.gemm(xd, packed, N, mx.Epilogue(plain, mx.PP_NONE), k_splits=1, ws=ws, **kw)
+    assert "ksplit" not in mx.last_kernel() and mx.last_kernel().startswith("skinny_"), mx.last_kernel()
+    check_float_parity(host_bits(plain), acc_ref, f"decode, no split {case}")
+
+
+def test_decode_k_split_rule(po, ws):
+    """The split is taken only with a workspace, k_splits = 0, panels for at most half of the CUs and slices of at least
+    four chunks; a workspace too small for the slices' sums restricts it; the size query reports what a shape can use."""
+    rng = np.random.default_rng(5)
+
+    def kernel_for(M, K, N, **kw):
+        x = dev_bf16(rand_bf16(rng, (M, K), 1.0))
+        packed = mx.repack_b(dev(rng.integers(-127, 128, (K, N), dtype=np.int8)))
+        y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        mx.gemm(x, packed, N, mx.Epilogue(y, mx.PP_NONE), b_dtype=mx.I8, **kw)
+        return mx.last_kernel()
+
+    assert kernel_for(32, 8192, 1024, ws=ws) == "skinny_chunk_w8_ksplit4"
+    assert kernel_for(32, 8192, 4096, ws=ws) == "skinny_chunk_w8_ksplit2"
+    assert kernel_for(32, 8192, 4128, ws=ws) == "skinny_chunk_w8"              # 129 panels: more than half of the CUs
+    assert kernel_for(32, 1536, 1024, ws=ws) == "skinny_chunk_w8"              # 6 chunks: too short to split
+    assert kernel_for(32, 8192, 1024, ws=ws, k_splits=1) == "skinny_chunk_w8"
+    assert kernel_for(32, 8192, 1024, ws=ws[:(16 << 10) + 32 * 2 * 4096]) == "skinny_chunk_w8_ksplit2"
+    assert kernel_for(32, 8192, 1024, ws=ws[:(16 << 10) + 4096]) == "skinny_chunk_w8"
+    with pytest.raises(mx.MmxError, match="decode kernels"):
+        kernel_for(32, 8192, 1024, ws=ws, k_splits=2)
+    assert mx.gemm_workspace_bytes(mx.BF16, mx.I8, 32, 8192, 1024) == (16 << 10) + 32 * 4 * 4096
+    assert mx.gemm_workspace_bytes(mx.BF16, mx.I8, 32, 8192, 1024, k_splits=1) == 0
+    assert mx.gemm_workspace_bytes(mx.BF16, mx.I8, 32, 8192, 8192) == 0
 
 
 @pytest.mark.parametrize("M", [64, 300])
