@@ -1145,17 +1145,22 @@ constexpr int SPLIT_MAX_PANELS = 4096;
 constexpr size_t SPLIT_COUNTER_BYTES = (size_t)SPLIT_MAX_PANELS * 4;
 
 // Slices of K for the chunked kernel: with a panel for at most every second CU the workgroups of a panel walk K in 2-4
-// slices, none empty and each at least four chunks long, and the last to arrive adds them up (int8 weights, weights
-// rotated over 540 MB: 11008 x 4096 at M = 16 / 32 20.4 / 25.1 -> 14.5 / 17.3 us, 8192 x 1024 15.5 / 19.0 -> 9.1 / 10.5;
-// bf16 weights: 11008 x 4096 at M = 16 / 32 26.7 / 34.7 -> 19.4 / 22.4, 8192 x 1024 19.7 / 25.4 -> 10.3 / 11.5).
+// slices (as many as give every CU one workgroup; more - 6, 8 - measured slower), none empty and each at least four
+// chunks long, and the last to arrive adds them up (int8 weights, weights rotated over 540 MB: 11008 x 4096 at
+// M = 16 / 32 20.4 / 25.1 -> 14.5 / 17.3 us, 8192 x 1024 15.5 / 19.0 -> 9.1 / 10.5; bf16 weights: 11008 x 4096 at
+// M = 16 / 32 26.7 / 34.7 -> 19.4 / 22.4, 8192 x 1024 19.7 / 25.4 -> 10.3 / 11.5).  With a panel for up to two thirds of the
+// CUs, three slices of at least ten chunks fill the two workgroups a CU holds (11008 x 5120, int8 M = 16 / 32 20.9 / 25.8
+// -> 17.1 / 21.7, bf16 27.6 / 35.7 -> 24.2 / 26.7); shorter slices and more panels measured level or behind.
 static int chunk_slices(bool w8, int M, int nfrag, int panels, size_t ws_bytes) {
-    if (panels <= 0 || panels * 2 > num_cus() || panels > SPLIT_MAX_PANELS) return 1;
+    if (panels <= 0 || panels * 3 > 2 * num_cus() || panels > SPLIT_MAX_PANELS) return 1;
     const int fc = (!w8 && M <= 16) ? 16 : 8;  // fragments per chunk of the kernels launched for these shapes
     const int nchunk = (nfrag + fc - 1) / fc;
-    int S = num_cus() / panels < 4 ? num_cus() / panels : 4;
-    while (S > 1 && ((nchunk + S - 1) / S < 4 || (S - 1) * ((nchunk + S - 1) / S) >= nchunk ||
+    const bool wide = panels * 2 > num_cus();
+    int S = wide ? 3 : (num_cus() / panels < 4 ? num_cus() / panels : 4);
+    const int shortest = wide ? 10 : 4;
+    while (S > 1 && ((nchunk + S - 1) / S < shortest || (S - 1) * ((nchunk + S - 1) / S) >= nchunk ||
                      SPLIT_COUNTER_BYTES + (size_t)panels * S * 4096 > ws_bytes))
-        S--;
+        S = wide ? 1 : S - 1;
     return S;
 }
 
@@ -1463,9 +1468,9 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
             s.ws_part = rq->ws + SPLIT_COUNTER_BYTES;
             s.kslices = ksl;
             grid = dim3(panels, ksl);
-            static const char* const names[2][3] = {{"skinny_chunk_bf16_ksplit2", "skinny_chunk_bf16_ksplit3", "skinny_chunk_bf16_ksplit4"},
-                                                    {"skinny_chunk_w8_ksplit2", "skinny_chunk_w8_ksplit3", "skinny_chunk_w8_ksplit4"}};
-            note_kernel(names[w8][ksl - 2]);
+            char name_[40];
+            snprintf(name_, sizeof name_, "skinny_chunk_%s_ksplit%d", w8 ? "w8" : "bf16", ksl);
+            note_kernel(name_);
         }
         // rows of x per buffer = 8 KiB * XD / (8 * FPW fragments * 64 or 32 bytes)
         if (pairs) {

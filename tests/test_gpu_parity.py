@@ -1313,11 +1313,12 @@ def test_ksplit_requests_that_cannot_be_met(ws):
     assert mx.gemm_workspace_bytes(mx.BF16, mx.BF16, 64, 1024, 256, k_splits=1) == 0
 
 
-# K split of the chunked decode kernel: few panels (at most one for every second CU), x too large for LDS, a workspace
+# K split of the chunked decode kernel: few panels (at most one for two of every three CUs), x too large for LDS, a workspace
 # and k_splits = 0.  2-4 slices, ragged N, a column range, a last slice shorter than the others, every store type.
 @pytest.mark.parametrize("case", [(True, 16, 8192, 1024), (True, 32, 11008, 1000), (True, 24, 4096, 4096), (True, 20, 5120, 1280),
                                   (False, 16, 8192, 512), (False, 32, 11008, 200), (False, 24, 4096, 4096), (False, 12, 9216, 96),
-                                  (False, 32, 2560, 2560), (True, 17, 4352, 300)])
+                                  (False, 32, 2560, 2560), (True, 17, 4352, 300),
+                                  (True, 24, 8192, 4160), (False, 32, 4096, 5120)])   # (three slices, two workgroups per CU)
 def test_decode_k_split(po, ws, case):
     w8, M, K, N = case
     rng = np.random.default_rng(11 * (M + K + N) + int(w8))
@@ -1376,7 +1377,7 @@ def test_decode_k_split(po, ws, case):
 
 def test_decode_k_split_rule(po, ws):
     """The split is taken only with a workspace, k_splits = 0, panels for at most half of the CUs and slices of at least
-    four chunks; a workspace too small for the slices' sums restricts it; the size query reports what a shape can use."""
+    four chunks (or for at most two thirds of them and three slices of at least ten); a workspace too small for the slices' sums restricts it; the size query reports what a shape can use."""
     rng = np.random.default_rng(5)
 
     def kernel_for(M, K, N, **kw):
@@ -1388,7 +1389,9 @@ def test_decode_k_split_rule(po, ws):
 
     assert kernel_for(32, 8192, 1024, ws=ws) == "skinny_chunk_w8_ksplit4"
     assert kernel_for(32, 8192, 4096, ws=ws) == "skinny_chunk_w8_ksplit2"
-    assert kernel_for(32, 8192, 4128, ws=ws) == "skinny_chunk_w8"              # 129 panels: more than half of the CUs
+    assert kernel_for(32, 8192, 4128, ws=ws) == "skinny_chunk_w8_ksplit3"      # 129 panels: more than half of the CUs
+    assert kernel_for(32, 4096, 4128, ws=ws) == "skinny_chunk_w8"              # ... and slices shorter than ten chunks
+    assert kernel_for(32, 8192, 5504, ws=ws) == "skinny_chunk_w8"              # 172 panels: more than two thirds
     assert kernel_for(32, 1536, 1024, ws=ws) == "skinny_chunk_w8"              # 6 chunks: too short to split
     assert kernel_for(32, 8192, 1024, ws=ws, k_splits=1) == "skinny_chunk_w8"
     assert kernel_for(32, 8192, 1024, ws=ws[:(16 << 10) + 32 * 2 * 4096]) == "skinny_chunk_w8_ksplit2"
