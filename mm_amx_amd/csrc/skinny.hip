@@ -1472,6 +1472,19 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
             snprintf(name_, sizeof name_, "skinny_chunk_%s_ksplit%d", w8 ? "w8" : "bf16", ksl);
             note_kernel(name_);
         }
+        // More than one panel per CU but fewer than two, 17-32 rows: a workgroup takes two neighbouring panels and stages x
+        // once for both (at these M a chunk of x is 1-2 times the bytes of a panel's chunk of weights, and with one panel per
+        // workgroup every workgroup pulls all of x through its CU).  4096 x 11008: int8 weights M = 24 / 32 18.2 / 19.3 ->
+        // 16.7 / 17.4 us, bf16 22.6 / 24.6 -> 22.1 / 22.9; 4096 x 13824: 19.5 -> 18.2 and 25.4 -> 24.3 at M = 32.  With exactly
+        // one panel per CU or fewer it leaves CUs idle (4096 x 8192: 12.8 -> 16.7), with two or more per CU and at M <= 16
+        // it measured level or behind; so did a K split on top of it.
+        if (!pairs && wk <= 1 && M > 16 && panels > num_cus() && panels < 2 * num_cus()) {
+            note_kernel(w8 ? "skinny_chunk_w8_2p" : "skinny_chunk_bf16_2p");
+            const dim3 g2((panels + 1) / 2);  // (an odd last panel: the second one of the last workgroup stores nothing)
+            if (w8) hipLaunchKernelGGL((skinny_chunk_kernel<true, 2, 1, 2>), g2, dim3(512), 65536, st, s);
+            else hipLaunchKernelGGL((skinny_chunk_kernel<false, 2, 1, 1>), g2, dim3(512), 65536, st, s);
+            return check_hip(hipGetLastError(), "skinny_chunk_kernel launch");
+        }
         // rows of x per buffer = 8 KiB * XD / (8 * FPW fragments * 64 or 32 bytes)
         if (pairs) {
             if (M <= 16) MMX_CHUNKED(false, 2, 2, 1, panels / 2);

@@ -1375,6 +1375,57 @@ def test_decode_k_split(po, ws, case):
     check_float_parity(host_bits(plain), acc_ref, f"decode, no split {case}")
 
 
+# More than one 32-column panel per CU but fewer than two, 17-32 rows: a workgroup of the chunked kernel takes two
+# neighbouring panels and stages x once for both.  An odd number of panels (the last workgroup's second panel stores
+# nothing), a ragged N, a column range, every post-op operand.
+@pytest.mark.parametrize("case", [(True, 24, 4096, 8352), (False, 32, 2560, 11008), (True, 17, 5120, 8315), (False, 20, 4096, 8352)])
+def test_decode_two_panels_per_workgroup(po, case):
+    w8, M, K, N = case
+    rng = np.random.default_rng(19 * (M + K + N) + int(w8))
+    x = rand_bf16(rng, (M, K), 1.0)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    qs = rng.uniform(10.0, 30.0, N).astype(np.float32)
+    if w8:
+        W = np.clip(np.rint(rng.standard_normal((K, N)) * 40), -127, 127).astype(np.int8)
+        scale = rng.uniform(1e-3, 5e-3, N).astype(np.float32)
+        _, acc_ref = po.gemv_w8(x, W, scale, want_acc=True)
+        packed, kw = mx.repack_b(dev(W)), {"b_dtype": mx.I8}
+        steps, pos = mx.PP_DEQUANT | mx.PP_BIAS | mx.PP_GELU, po.PP_DEQUANT | po.PP_BIAS | po.PP_GELU
+        opd, opo = {"bias": dev(bias), "deq_scale_per_oc": dev(scale)}, {"bias": bias, "deq_per_oc": scale}
+    else:
+        W = rand_bf16(rng, (K, N), 0.05)
+        acc_ref = po.gemm_bf16(x, W)
+        packed, kw = mx.repack_b(dev_bf16(W)), {}
+        steps, pos = mx.PP_BIAS | mx.PP_GELU, po.PP_BIAS | po.PP_GELU
+        opd, opo = {"bias": dev(bias)}, {"bias": bias}
+    xd = dev_bf16(x)
+    want = "skinny_chunk_w8_2p" if w8 else "skinny_chunk_bf16_2p"
+    acc = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    mx.gemm(xd, packed, N, mx.Epilogue(acc, mx.PP_NONE), **kw)
+    assert mx.last_kernel() == want, mx.last_kernel()
+    acc_gpu = host_bits(acc)
+    check_float_parity(acc_gpu, acc_ref, f"two panels per workgroup, accumulators {case}")
+    y8 = torch.zeros((M, N), dtype=torch.int8, device="cuda")
+    mx.gemm(xd, packed, N, mx.Epilogue(y8, steps | mx.PP_QUANT, q_scale_per_oc=dev(qs), **opd), **kw)
+    assert mx.last_kernel() == want
+    assert np.array_equal(host_bits(y8), po.pp(acc_gpu, pos | po.PP_QUANT, po.I8, q_per_oc=qs, **opo))
+    # a column range that starts at an odd panel and ends inside one: the rest of C is left alone
+    n0, n1 = 32, N - 37
+    part = torch.full((M, N), -3.0, dtype=torch.bfloat16, device="cuda")
+    mx.gemm(xd, packed, N, mx.Epilogue(part, steps, **opd), n0=n0, n1=n1, **kw)
+    assert mx.last_kernel() == want
+    got = host_bits(part)
+    assert np.array_equal(got[:, n0:n1], po.pp(acc_gpu, pos, po.BF16, **opo)[:, n0:n1])
+    minus3 = host_bits(torch.full((1,), -3.0, dtype=torch.bfloat16, device="cuda"))[0]
+    assert np.all(got[:, :n0] == minus3) and np.all(got[:, n1:] == minus3)
+    # the same sums as the one-panel form: each wave adds the same products in the same order
+    if N <= 8352:
+        one = torch.zeros((M, 8160), dtype=torch.float32, device="cuda")     # 255 panels: one per workgroup
+        mx.gemm(xd, packed, N, mx.Epilogue(one, mx.PP_NONE), n0=0, n1=8160, k_splits=1, **kw)
+        assert mx.last_kernel() in ("skinny_chunk_w8", "skinny_chunk_bf16"), mx.last_kernel()
+        assert np.array_equal(host_bits(one), acc_gpu[:, :8160])
+
+
 def test_decode_k_split_rule(po, ws):
     """The split is taken only with a workspace, k_splits = 0, panels for at most half of the CUs and slices of at least
     four chunks (or for at most two thirds of them and three slices of at least ten); a workspace too small for the slices' sums restricts it; the size query reports what a shape can use."""
