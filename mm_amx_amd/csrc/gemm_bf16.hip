@@ -28,7 +28,7 @@ size_t plan_workspace_bytes(int elesz, bool w8, int M, int K, int Ncols, uint32_
     if (kbytes % 128) return 0;
     const SplitRequest rq = {k_splits, reinterpret_cast<char*>(256), ~(size_t)0};
     if (steps & MMX_PP_SILU_GATE) return 0;
-    const Plan p = choose_plan(M, Ncols, (int)(kbytes / 128), false, w8, 2, rq);
+    const Plan p = choose_plan(M, Ncols, (int)(kbytes / 128), false, w8, 2, rq, elesz == 1);
     if (p.S <= 1) return 0;
     const size_t tiles = (size_t)((M + p.t.bm - 1) / p.t.bm) * ((Ncols + p.t.bn - 1) / p.t.bn);
     return WS_COUNTER_BYTES + tiles * p.S * p.t.bm * p.t.bn * 4;
