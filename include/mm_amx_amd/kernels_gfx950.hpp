@@ -346,7 +346,8 @@ struct Matmul {
         require(ppkernel.out_rows() >= M && ppkernel.out_cols() >= n1, "Matmul: C is smaller than M x n1");
         if (!constB || !internalB) internalB = repackB_1x2(matB, transposeB, stream);
         const mmx_epilogue e = ppkernel.descriptor();
-        const Workspace ws = (k_splits == 1 || M <= 32) ? Workspace() : workspace_for(stream);
+        // (decode launches, M <= 32, choose their own slices: they take the workspace with k_splits = 0 only)
+        const Workspace ws = (k_splits == 1 || (M <= 32 && k_splits != 0)) ? Workspace() : workspace_for(stream);
         check(mmx_gemm_splitk(dtype_of<TA>::value, dtype_of<TB>::value, matA.data, matA.stride, internalB.data, M, K, N, n0, n1,
                               &e, ws.data ? k_splits : 1, ws.data, ws.bytes, stream),
               "Matmul");
@@ -366,6 +367,7 @@ struct Matmul<bfloat16, int8_t, float> {
     constexpr static int kStep = 32;
     float quant_scale_B = 0.0f;
     float dequant_scale_B = 0.0f;
+    int k_splits = 0;  // as in the primary template
 
     Matmul(bool constB = false, bool transposeB = false) : constB(constB), transposeB(transposeB) {}
 
@@ -397,7 +399,9 @@ struct Matmul<bfloat16, int8_t, float> {
         }
         ppkernel.set_deq_scale(dequant_scale_B);
         const mmx_epilogue e = ppkernel.descriptor();
-        check(mmx_gemm(MMX_BF16, MMX_I8, matA.data, matA.stride, internalBI8.data, M, K, N, n0, n1, &e, stream),
+        const Workspace ws = (k_splits == 1 || (M <= 32 && k_splits != 0)) ? Workspace() : workspace_for(stream);
+        check(mmx_gemm_splitk(MMX_BF16, MMX_I8, matA.data, matA.stride, internalBI8.data, M, K, N, n0, n1, &e,
+                              ws.data ? k_splits : 1, ws.data, ws.bytes, stream),
               "Matmul<bf16,int8>");
     }
 };
@@ -528,7 +532,7 @@ struct MLP {
         const int M = x.dims[0];
         require(x.dims[1] == m_K && y.dims[0] == M && y.dims[1] == m_K, "run: x and y must be [M, K]");
         setM(M);
-        const Workspace ws = (down_k_splits == 1 || M <= 32) ? Workspace() : workspace_for(stream);
+        const Workspace ws = down_k_splits == 1 ? Workspace() : workspace_for(stream);  // (M <= 32: the library chooses)
         check(mmx_mlp_splitk(x.data, x.stride, gate_up.data, down.data, actUp.data, actUp.stride, y.data, y.stride, M, m_K, m_N,
                              ws.data ? down_k_splits : 1, ws.data, ws.bytes, stream),
               "MLP::run");

@@ -199,6 +199,8 @@ static void test_matmul_weight_int8(int M, int K, int N) {
     B.upload(hB.data());
     Matmul<bfloat16, int8_t> mm(true, false);
     mm(A, B, PP::BiasGeluStore<float, PP::DEQUANT>(C));
+    if (M <= 32 && M > 16 && K >= 8192 && N <= 4096)
+        EXPECT(std::string(mmx_last_kernel()).find("skinny_chunk_w8_ksplit") == 0, "ran %s, not the decode K split", mmx_last_kernel());
     check_hip(hipDeviceSynchronize(), "sync");
     std::vector<float> got(static_cast<size_t>(M) * N);
     C.download(got.data());
@@ -310,7 +312,7 @@ static void test_mlp(int M, int K, int N, int down_k_splits = 0) {
     mlp.down_k_splits = down_k_splits;
     mlp.setup(wg, wu, wd);
     mlp.run(x, y);
-    if (down_k_splits > 1)
+    if (down_k_splits > 1 || (M <= 32 && M > 8 && N >= 8192))  // (few panels of a long K at decode sizes: the library's own split)
         EXPECT(std::string(mmx_last_kernel()).find("ksplit") != std::string::npos, "down projection ran %s, not a K split", mmx_last_kernel());
     check_hip(hipDeviceSynchronize(), "sync");
     std::vector<bfloat16> gh(static_cast<size_t>(M) * N), gy(static_cast<size_t>(M) * K);
@@ -412,6 +414,7 @@ int main() {
         test_matmul_weight_int8(2, 2560, 192);  // fc16m.cpp:749
         test_matmul_weight_int8(160, 512, 256);   // large M: int8 fragments converted between LDS and the MFMA operand
         test_matmul_weight_int8(300, 200, 96);    // ... with a K tail (masked loads)
+        test_matmul_weight_int8(24, 8192, 256);   // decode with few panels: K walked in slices through the stream's workspace
         test_matmul_weight_int4(1, 4096, 352);
         test_matmul_weight_int4(7, 300, 77);
         test_matvec(901, 80);  // main.cpp:884
@@ -420,6 +423,7 @@ int main() {
         test_linear_nxn(512, 128, 4096);  // torch-ext/test.py:37
         test_mlp(1, 512, 1024);
         test_mlp(96, 512, 1024);
+        test_mlp(24, 512, 8192);    // decode: the down projection (K = 8192, 16 panels) takes its own K split
         test_mlp(96, 512, 1024, 2);  // the reference's do_splitK for the down projection (tests/amx-mlp.cpp:768)
         test_matmul_i8_requant(160, 2048, 320);  // long enough K for the two-way K split
         test_two_threads_first_call();
