@@ -1166,9 +1166,9 @@ static int chunk_slices(bool w8, int M, int nfrag, int panels, size_t ws_bytes) 
 
 // Bytes of workspace a decode launch of this shape can use (0: it takes no K split)
 size_t skinny_workspace_bytes(int wk, int M, int K, int n0, int n1) {
-    const int nfrag = (K * (wk == 1 ? 1 : 2) + 127) / 128 * 128 / 32;
+    const int nfrag = (K * ((wk == 1 || wk == 3) ? 1 : 2) + 127) / 128 * 128 / 32;
     const int panels = ((n1 + 31) >> 5) - (n0 >> 5);
-    const int S = chunk_slices(wk == 1, M, nfrag, panels, ~(size_t)0);
+    const int S = chunk_slices(wk != 0, M, nfrag, panels, ~(size_t)0);
     return S > 1 ? SPLIT_COUNTER_BYTES + (size_t)panels * S * 4096 : 0;
 }
 
@@ -1265,6 +1265,18 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         // kernel otherwise
         const int zoff = (M * K + 1023) & ~1023;
         if (zoff + K > 46 * 1024) {  // x does not fit in LDS: through LDS chunk by chunk (32 rows x 256 bytes per buffer)
+            // (few panels, a workspace at hand: K in slices as for bf16 activations; int32 sums, the same bits in any order)
+            const int ksl3 = (rq && rq->ws && rq->k_splits == 0) ? chunk_slices(true, M, s.nfrag, panels, rq->ws_bytes) : 1;
+            if (ksl3 > 1) {
+                s.ws_cnt = reinterpret_cast<uint32_t*>(rq->ws);
+                s.ws_part = rq->ws + SPLIT_COUNTER_BYTES;
+                s.kslices = ksl3;
+                char name_[40];
+                snprintf(name_, sizeof name_, "skinny_chunk_i8_ksplit%d", ksl3);
+                note_kernel(name_);
+                hipLaunchKernelGGL((skinny_chunk_kernel<3, 1, 1, 1, 6>), dim3(panels, ksl3), dim3(512), 8 * 1 * 16 * 64 * 4, st, s);
+                return check_hip(hipGetLastError(), "skinny_chunk_kernel launch");
+            }
             note_kernel("skinny_chunk_i8");
             hipLaunchKernelGGL((skinny_chunk_kernel<3, 1, 1, 1>), dim3(panels), dim3(512), 8 * 1 * 16 * 64 * 4, st, s);
             return check_hip(hipGetLastError(), "skinny_chunk_kernel launch");

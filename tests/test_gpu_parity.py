@@ -1426,6 +1426,39 @@ def test_decode_two_panels_per_workgroup(po, case):
         assert np.array_equal(host_bits(one), acc_gpu[:, :8160])
 
 
+@pytest.mark.parametrize("shape", [(24, 8192, 512), (32, 11008, 1000), (9, 16384, 96), (32, 11008, 4160)])
+def test_int8_decode_k_split(po, ws, shape):
+    """int8 activations on int8 weights, x too large for LDS, few panels: the chunked kernel's K split.  int32 sums are
+    the oracle's bit for bit whatever the slices and their arrival order; every post-op step on top."""
+    M, K, N = shape
+    rng = np.random.default_rng(23 * sum(shape))
+    A = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    B = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    deq = (np.float32(0.02) * rng.uniform(1e-3, 1e-2, N).astype(np.float32)).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    qoc = rng.uniform(5, 40, N).astype(np.float32)
+    acc_ref = po.gemm_i8(A, B)
+    Ad, packed = dev(A), mx.repack_b(dev(B))
+    for rep in range(2):
+        C = torch.full((M, N), -7, dtype=torch.int32, device="cuda")
+        mx.gemm(Ad, packed, N, mx.Epilogue(C, mx.PP_NONE), ws=ws)
+        assert mx.last_kernel().startswith("skinny_chunk_i8_ksplit"), mx.last_kernel()
+        assert np.array_equal(host_bits(C), acc_ref)
+    out8 = torch.zeros((M, N), dtype=torch.int8, device="cuda")
+    mx.gemm(Ad, packed, N, mx.Epilogue(out8, 15, bias=dev(bias), deq_scale_per_oc=dev(deq), q_scale_per_oc=dev(qoc)), ws=ws)
+    assert mx.last_kernel().startswith("skinny_chunk_i8_ksplit")
+    assert np.array_equal(host_bits(out8), po.pp(acc_ref, 15, po.I8, bias=bias, deq_per_oc=deq, q_per_oc=qoc))
+    n0, n1 = 32, N - 3
+    part = torch.full((M, N), -7, dtype=torch.int32, device="cuda")
+    mx.gemm(Ad, packed, N, mx.Epilogue(part, mx.PP_NONE), n0=n0, n1=n1, ws=ws)
+    got = host_bits(part)
+    assert np.array_equal(got[:, n0:n1], acc_ref[:, n0:n1]) and np.all(got[:, :n0] == -7) and np.all(got[:, n1:] == -7)
+    whole = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    mx.gemm(Ad, packed, N, mx.Epilogue(whole, mx.PP_NONE), k_splits=1, ws=ws)
+    assert mx.last_kernel() == "skinny_chunk_i8", mx.last_kernel()
+    assert np.array_equal(host_bits(whole), acc_ref)
+
+
 def test_decode_k_split_rule(po, ws):
     """The split is taken only with a workspace, k_splits = 0, panels for at most half of the CUs and slices of at least
     four chunks (or for at most two thirds of them and three slices of at least ten); a workspace too small for the slices' sums restricts it; the size query reports what a shape can use."""
