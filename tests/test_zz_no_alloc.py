@@ -67,6 +67,11 @@ def test_static_workspace_entry_point_matches_the_workspace_one(po):
     k5 = _bf16_case(po, 64, 4096, 512, 5, 0, ws)
     k6 = _bf16_case(po, 8, 1024, 256, 6, 0, ws)
     assert "ksplit" in k5 and "skinny" in k6, (k5, k6)
+    # decode shapes with few panels of a long K: the chunked kernel's own K split parks its sums in the same array
+    k7 = _bf16_case(po, 24, 8192, 512, 7, 0, ws)
+    k8 = _int8_case(po, 24, 8192, 512, 8, 0, ws)
+    k9 = _bf16_case(po, 12, 4096, 96, 9, 0, ws)       # ... and a smaller one after them
+    assert k7.startswith("skinny_chunk_bf16_ksplit") and k8.startswith("skinny_chunk_i8_ksplit") and "skinny" in k9, (k7, k8, k9)
     torch.cuda.synchronize()
     assert not ws[:16 << 10].any().item()
 
