@@ -1122,6 +1122,40 @@ def test_ksplit_replays_from_a_hip_graph(po, ws, S):
         mx.set_tile("")
 
 
+def test_decode_k_split_replays_from_a_hip_graph(po, ws):
+    """The decode kernels' K split under graph replay: as for the tiles, the counters wrap to zero with the last arrival,
+    so a captured launch replays with nothing cleared in between; every replay gives the eager bits."""
+    M, K, N = 24, 8192, 512
+    rng = np.random.default_rng(77)
+    W = np.clip(np.rint(rng.standard_normal((K, N)) * 40), -127, 127).astype(np.int8)
+    scale = rng.uniform(1e-3, 5e-3, N).astype(np.float32)
+    packed, sd = mx.repack_b(dev(W)), dev(scale)
+    x = dev_bf16(rand_bf16(rng, (M, K), 1.0)).clone()
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    ep = mx.Epilogue(y, mx.PP_DEQUANT, deq_scale_per_oc=sd)
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        mx.gemm(x, packed, N, ep, b_dtype=mx.I8, ws=ws)   # warm-up on the capture stream
+        side.synchronize()
+        with torch.cuda.graph(g, stream=side):
+            mx.gemm(x, packed, N, ep, b_dtype=mx.I8, ws=ws)
+    assert mx.last_kernel() == "skinny_chunk_w8_ksplit4", mx.last_kernel()
+    torch.cuda.synchronize()
+    for rep in range(4):
+        x.copy_(dev_bf16(rand_bf16(rng, (M, K), 1.0)))
+        y.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        got = host_bits(y).copy()
+        assert not ws[:16 << 10].any().item(), "counters not back at zero after a replay"
+        y2 = torch.zeros_like(y)
+        mx.gemm(x, packed, N, mx.Epilogue(y2, mx.PP_DEQUANT, deq_scale_per_oc=sd), b_dtype=mx.I8, ws=ws)   # eager, same workspace
+        torch.cuda.synchronize()
+        assert np.array_equal(got, host_bits(y2)), rep
+
+
 # ---- int8 activations at M <= 32: the streaming decode form (int32 sums, order-free) --------------------------
 @pytest.mark.parametrize("shape", [(1, 128, 64), (5, 1024, 100), (32, 1152, 192), (4, 4096, 352), (9, 4096, 33),
                                    (2, 8192, 96), (16, 4096, 352), (32, 2560, 100), (12, 11008, 64), (32, 4224, 96)])
