@@ -150,7 +150,7 @@ int mmx_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const v
  *   k_splits  0 = the library chooses (possibly no split), 1 = none, 2..4 = exactly that many slices
  *             (MMX_E_INVALID if K is too short or the workspace too small, MMX_E_UNSUPPORTED for M <= 32,
  *             SILU_GATE, unaligned A or K * sizeof(T) not a multiple of 128).  The decode kernels (M <= 32)
- *             take 0 or 1 only: with 0 and a workspace, launches over bf16 or int8 weights (not int4) whose x does
+ *             take 0 or 1 only: with 0 and a workspace, launches over bf16, int8 or int4 weights whose x does
  *             not fit in LDS and whose column range has 32-column panels for at most two thirds of the CUs walk K in
  *             2-4 slices of their own choosing, combined the same way (same layout of the workspace).
  *   workspace device memory, 256-byte aligned, mmx_gemm_workspace_bytes() or more (64 MiB + 16 KiB always

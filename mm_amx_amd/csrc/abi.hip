@@ -309,8 +309,9 @@ int mmx_gemm_splitk_static(int a_dtype, int b_dtype, const void* A, int64_t lda_
 size_t mmx_gemm_workspace_bytes(int a_dtype, int b_dtype, int M, int K, int N, int n0, int n1, uint32_t steps, int k_splits) {
     const bool bf = a_dtype == MMX_BF16 && b_dtype == MMX_BF16, i8 = a_dtype == MMX_I8 && b_dtype == MMX_I8;
     const bool w8 = a_dtype == MMX_BF16 && b_dtype == MMX_I8;
-    if (M > 0 && M <= 32 && (bf || w8 || i8) && K > 0 && N > 0 && n0 >= 0 && n1 <= N && n0 < n1)
-        return k_splits == 0 && !(steps & MMX_PP_SILU_GATE) ? skinny_workspace_bytes(i8 ? 3 : (w8 ? 1 : 0), M, K, n0, n1) : 0;
+    const bool w4 = a_dtype == MMX_BF16 && b_dtype == MMX_I4;
+    if (M > 0 && M <= 32 && (bf || w8 || i8 || w4) && K > 0 && N > 0 && n0 >= 0 && n1 <= N && n0 < n1)
+        return k_splits == 0 && !(steps & MMX_PP_SILU_GATE) ? skinny_workspace_bytes(i8 ? 3 : (w4 ? 2 : (w8 ? 1 : 0)), M, K, n0, n1) : 0;
     if ((!bf && !i8 && !w8) || M <= 32 || K <= 0 || N <= 0 || n0 < 0 || n1 > N || n0 >= n1 || k_splits < 0) return 0;
     return plan_workspace_bytes(i8 ? 1 : 2, w8, M, K, n1 - n0, steps, k_splits);
 }

@@ -1166,7 +1166,7 @@ static int chunk_slices(bool w8, int M, int nfrag, int panels, size_t ws_bytes) 
 
 // Bytes of workspace a decode launch of this shape can use (0: it takes no K split)
 size_t skinny_workspace_bytes(int wk, int M, int K, int n0, int n1) {
-    const int nfrag = (K * ((wk == 1 || wk == 3) ? 1 : 2) + 127) / 128 * 128 / 32;
+    const int nfrag = wk == 2 ? (K + 255) / 256 * 4 : (K * ((wk == 1 || wk == 3) ? 1 : 2) + 127) / 128 * 128 / 32;
     const int panels = ((n1 + 31) >> 5) - (n0 >> 5);
     const int S = chunk_slices(wk != 0, M, nfrag, panels, ~(size_t)0);
     return S > 1 ? SPLIT_COUNTER_BYTES + (size_t)panels * S * 4096 : 0;
@@ -1315,6 +1315,18 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         }
         if (s.nfrag * 64 == K && s.x_vec_ok) {
             // x too large for LDS: through LDS chunk by chunk (two buffers of 16 or 32 rows x 1 KiB)
+            const int ksl4 = (rq && rq->ws && rq->k_splits == 0) ? chunk_slices(true, M, s.nfrag, panels, rq->ws_bytes) : 1;
+            if (ksl4 > 1) {  // few panels, a workspace at hand: K in slices as for the other weight types
+                s.ws_cnt = reinterpret_cast<uint32_t*>(rq->ws);
+                s.ws_part = rq->ws + SPLIT_COUNTER_BYTES;
+                s.kslices = ksl4;
+                char name_[40];
+                snprintf(name_, sizeof name_, "skinny_chunk_w4_ksplit%d", ksl4);
+                note_kernel(name_);
+                if (M <= 16) hipLaunchKernelGGL((skinny_chunk_kernel<2, 1, 1, 2, 3>), dim3(panels, ksl4), dim3(512), 2 * 8 * 2 * 1024, st, s);
+                else hipLaunchKernelGGL((skinny_chunk_kernel<2, 1, 1, 4, 2>), dim3(panels, ksl4), dim3(512), 2 * 8 * 4 * 1024, st, s);
+                return check_hip(hipGetLastError(), "skinny_chunk_kernel launch");
+            }
             note_kernel("skinny_chunk_w4");
             if (M <= 16) hipLaunchKernelGGL((skinny_chunk_kernel<2, 1, 1, 2>), dim3(panels), dim3(512), 2 * 8 * 2 * 1024, st, s);
             else hipLaunchKernelGGL((skinny_chunk_kernel<2, 1, 1, 4>), dim3(panels), dim3(512), 2 * 8 * 4 * 1024, st, s);

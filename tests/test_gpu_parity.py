@@ -1010,6 +1010,34 @@ def test_int4_decode_shapes(po, shape):
     assert np.linalg.norm(host_bits(y) - ref) <= 1e-3 * np.linalg.norm(ref)
 
 
+@pytest.mark.parametrize("shape", [(24, 8192, 512), (8, 11008, 1000), (17, 16384, 4128)])
+def test_int4_decode_k_split(po, ws, shape):
+    """int4 weights, x too large for LDS, few panels: the chunked kernel's K split (two to four slices, and three with
+    panels for more than half of the CUs); the same bits on every run, the oracle's accumulators within the bar."""
+    M, K, N = shape
+    rng = np.random.default_rng(29 * sum(shape))
+    x = rand_bf16(rng, (M, K), 1.0)
+    W = rand_bf16(rng, (K, N), 0.05)
+    q, deq = po.quantize_int4(W)
+    _, acc_ref = po.gemv_w8(x, q, deq, want_acc=True)
+    packed, deq_gpu = mx.quantize_pack_int4(dev_bf16(W))
+    accs = []
+    for rep in range(3):
+        acc = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc, mx.PP_NONE), b_dtype=mx.I4, ws=ws)
+        assert mx.last_kernel().startswith("skinny_chunk_w4_ksplit"), mx.last_kernel()
+        accs.append(host_bits(acc))
+    assert np.array_equal(accs[0], accs[1]) and np.array_equal(accs[0], accs[2])
+    check_float_parity(accs[0], acc_ref, f"int4 decode K split accumulators {shape}")
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_DEQUANT, deq_scale_per_oc=deq_gpu), b_dtype=mx.I4, ws=ws)
+    assert np.array_equal(host_bits(y), po.pp(accs[0], po.PP_DEQUANT, po.BF16, deq_per_oc=deq))
+    whole = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(whole, mx.PP_NONE), b_dtype=mx.I4, k_splits=1, ws=ws)
+    assert mx.last_kernel() == "skinny_chunk_w4", mx.last_kernel()
+    check_float_parity(host_bits(whole), acc_ref, f"int4 decode, no split {shape}")
+
+
 @pytest.mark.parametrize("M", [1, 4])
 def test_int4_gemv_full_size(po, M):
     w = wl.decode_gemv_w8(M=M)      # x of the int8 case; the weights come from a bf16 matrix here
