@@ -35,7 +35,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 MEASURED_TRAFFIC = {
     "gemm_bf16_256x192_ring8w_out_bf16": {"bytes": (81702.5 * 2.000 + 27474.0 * 1.000) * 1024, "source": "mm_amx_amd/csrc/gemm_tile.hpp",
                                           "sha": "6f92c557e1ef21c0"},
-    "skinny_stream_w8": {"bytes": (22154.3 * 2.000 + 39.7 * 1.000) * 1024, "source": "mm_amx_amd/csrc/skinny.hip", "sha": "75501ed1cda66016"},
+    "skinny_stream_w8": {"bytes": (22154.3 * 2.000 + 39.7 * 1.000) * 1024, "source": "mm_amx_amd/csrc/skinny.hip", "sha": "c4f3a25ae1d3b1c9"},
 }
 
 
