@@ -220,6 +220,24 @@ def test_tuning_knobs_are_per_thread(lib):
     assert b"17x3" not in lib.mmx_last_error()  # this thread's error string is its own
 
 
+def test_workspace_query_covers_the_decode_kernels_k_split():
+    """mmx_gemm_workspace_bytes (a host-side computation; 256 CUs assumed before mmx_init has seen a device): decode shapes
+    with panels for at most two thirds of the CUs report the counters plus one 4 KiB block of sums per panel and slice,
+    every operand type; more panels, k_splits = 1 and SILU_GATE report none."""
+    import mm_amx_amd as mx
+    counters = 16 << 10
+    assert mx.gemm_workspace_bytes(mx.BF16, mx.I8, 32, 8192, 1024) == counters + 32 * 4 * 4096          # 32 panels, 4 slices
+    assert mx.gemm_workspace_bytes(mx.BF16, mx.BF16, 16, 11008, 4096) == counters + 128 * 2 * 4096      # 128 panels, 2 slices
+    assert mx.gemm_workspace_bytes(mx.BF16, mx.I4, 16, 8192, 1024) == counters + 32 * 4 * 4096
+    assert mx.gemm_workspace_bytes(mx.I8, mx.I8, 32, 8192, 1024) == counters + 32 * 4 * 4096
+    assert mx.gemm_workspace_bytes(mx.BF16, mx.I8, 32, 8192, 4160) == counters + 130 * 3 * 4096         # 130 panels, 3 slices
+    assert mx.gemm_workspace_bytes(mx.BF16, mx.I8, 32, 4096, 4160) == 0                                 # ... too short for three
+    assert mx.gemm_workspace_bytes(mx.BF16, mx.I8, 32, 8192, 8192) == 0
+    assert mx.gemm_workspace_bytes(mx.BF16, mx.I8, 32, 8192, 1024, k_splits=1) == 0
+    assert mx.gemm_workspace_bytes(mx.BF16, mx.BF16, 32, 8192, 1024, steps=mx.PP_SILU_GATE) == 0
+    assert mx.gemm_workspace_bytes(mx.BF16, mx.BF16, 64, 4096, 512) > counters                          # the tile kernels' plan
+
+
 def test_bench_traffic_figures_belong_to_the_current_kernel_sources():
     """bench.py reports a measured HBM traffic only for the kernel source it was measured on (keyed by a hash of the
     file): after a change of such a file the figure has to be measured again, or the bench reports null."""
