@@ -20,7 +20,6 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_INT8_TOPS = 5000.0     # MI355X dense int8 MFMA
@@ -90,7 +89,7 @@ def main():
 
     import mm_amx_amd as mx
     from mm_amx_amd import workloads as wl
-    from gpu_util import dev, dev_bf16
+    dev, dev_bf16 = wl.to_device, wl.to_device_bf16
 
     torch.cuda.set_device(0)
     mx.init(0)
@@ -150,10 +149,7 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "llama7b_ffn_up_bf16_bias_gelu", "M": M, "K": K, "N": N, "kernel": kernel_name,
                    "inputs": "A~N(0,1) bf16, B~N(0,0.02) bf16 repacked once, bias~N(0,0.1) fp32, all resident in HBM",
-                   "parity": "vs the CPU oracle at this size: relative Frobenius <= 1e-3; 99.87 % of all elements within 1 bf16 ulp "
-                             "(the stated bar is 99.9 %: met where the pre-activation is > -3.5, 99.99 %; below it GELU's bracket cancels and "
-                             "one fp32 ulp of summation order moves a bf16 ulp); the fused epilogue equals the oracle's bit for bit on the "
-                             "GPU's own accumulators (tests/test_gpu_parity.py::test_ffn_up_bias_gelu_full_size)"},
+                   "parity": "not checked in this run (--no-cpu); tests/test_gpu_parity.py::test_ffn_up_bias_gelu_full_size checks this shape"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                      "traffic": measured_traffic(kernel_name),
@@ -199,6 +195,24 @@ def main():
         def run_ref():
             acc = po.gemm_bf16(w["A"], w["B"], nthreads=cores)
             po.pp(acc, po.PP_BIAS | po.PP_GELU, po.BF16, bias=w["bias"])
+        # parity of what the timed launches wrote, against the oracle on the first rows of the same inputs (untimed;
+        # the oracle is the checker here, nothing of it is measured): relative Frobenius error and the share of elements
+        # within one bf16 ulp, over all elements and where GELU is well conditioned (pre-activation above -3.5)
+        rows = 64
+        acc_ref = po.gemm_bf16(np.ascontiguousarray(w["A"][:rows]), w["B"], nthreads=cores)
+        want = po.bf16_to_f32(po.pp(acc_ref, po.PP_BIAS | po.PP_GELU, po.BF16, bias=w["bias"])).astype(np.float64)
+        got = C[:rows].float().cpu().numpy().astype(np.float64)
+        ulp = np.exp2(np.floor(np.log2(np.maximum(np.abs(want), 2.0 ** -126))) - 7)
+        within = np.abs(got - want) <= ulp
+        well = (acc_ref + w["bias"][None, :]) > -3.5
+        out["config"]["parity"] = {
+            "against": f"CPU oracle, rows 0..{rows - 1} of the timed output ({rows * N} elements)",
+            "rel_frobenius": float(f"{np.linalg.norm(got - want) / np.linalg.norm(want):.3e}"),
+            "within_1_bf16_ulp_all": round(float(within.mean()), 6),
+            "within_1_bf16_ulp_preact_above_-3.5": round(float(within[well].mean()), 6),
+            "bar": "rel_frobenius <= 1e-3 and 99.9 % within 1 bf16 ulp where GELU is well conditioned; below -3.5 one fp32 ulp of "
+                   "summation order moves the reference polynomial by more than a bf16 ulp (tests/test_oracle_math.py shows the "
+                   "reference's arithmetic against an fp64 sum short of 99.9 % over all elements as well)"}
         reps, el = time_cpu(run_ref, args.cpu_seconds)
         out["cpu_baseline"] = {
             "value": round(flops * reps / el / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
@@ -235,16 +249,20 @@ def main():
             "port": {"value": round(opsi * reps / el / 1e12, 4), "unit": "TOP/s", "cores": cores, "sample": f"{reps} x the full workload in {el:.1f} s"},
             "onednn": gpu_note(onednn_i8)}
 
-        # config 4: decode GEMV over int8 weights, M=1, rotating over 8 weight copies (360 MB: nothing stays in a cache)
+        # config 4: decode GEMV over int8 weights, M=1, rotating over 8 weight copies (360 MB: nothing stays in a cache).
+        # The port is the reference's own form (weight_compression/fc16m.cpp:451-502, 620-663): weights packed once in
+        # repackB_1xL order, then every call streams the int8 bytes and converts them in registers, N split over the threads
         wgc = wl.decode_gemv_w8(M=1)
-        Wcopies = [wgc["W"].copy() for _ in range(8)]
+        packed0 = po.pack_1x2_s8(wgc["W"])
+        Wcopies = [packed0.copy() for _ in range(8)]
         turn = [0]
 
         def run_gemv():
-            po.gemv_w8(wgc["x"], Wcopies[turn[0] % 8], wgc["scale"], nthreads=cores)
+            po.gemv_w8_stream(wgc["x"], Wcopies[turn[0] % 8], wgc["scale"], wgc["N"], nthreads=cores)
             turn[0] += 1
         reps, el = time_cpu(run_gemv, b3)
         wbytes = float(wgc["K"]) * wgc["N"]
+        Wcopies = [wgc["W"].copy() for _ in range(8)]
 
         def onednn_gemv():
             xt = torch.from_numpy(wgc["x"].view(np.int16).copy()).view(torch.bfloat16)
@@ -259,7 +277,8 @@ def main():
                     "sample": f"{r} x torch.matmul(x bf16 [1,4096], W bf16 [4096,11008]) over 8 rotated copies in {e:.1f} s (bf16 weights: 2 bytes each)"}
         cpu_other["decode_gemv_int8w_K4096_N11008_M1"] = {
             "port": {"value": round(wbytes * reps / el / 1e9, 2), "unit": "GB/s", "cores": cores,
-                     "sample": f"{reps} x the full GEMV over 8 rotated weight copies in {el:.1f} s (the restatement converts the weights to bf16 on every call)"},
+                     "sample": f"{reps} x the full GEMV over 8 rotated copies of the packed int8 weights in {el:.1f} s (weights streamed once "
+                               "and converted in registers, as matmul16m_Wint8B does)"},
             "onednn": gpu_note(onednn_gemv)}
         del Wcopies
 
@@ -603,6 +622,23 @@ def main():
         del gu, dn
         extra["llama7b_mlp_stages"] = stages
 
+        # The reference's end-to-end demo at its size (torch-ext/test.py:176-218): a stack of 32 Llama-7B MLPs (RMSNorm +
+        # fused MLP, every layer its own 270 MB of weights: 8.7 GB packed + the same again for torch's layers), per-layer
+        # time through torch's bf16 linear layers and through this library; at M=1 also replayed from a HIP graph,
+        # which shows what the Python/ctypes host layer costs per layer
+        del op
+        from mm_amx_amd import mlp_llama
+        demo = {}
+        for Md, rounds in ((256, 10), (1, 20)):
+            r = mlp_llama.perf_llama7b_MLP(M=Md, num_layers=32, rounds=rounds, verbose=False, graph=True)
+            demo[str(Md)] = {k: ({kk: (round(vv, 1) if isinstance(vv, float) else vv) for kk, vv in v.items()} if isinstance(v, dict)
+                                 else float(f"{v:.3e}")) for k, v in r.items()}
+            host = r["mm_amx_amd"]["per_layer_us"] - r["mm_amx_amd_graph"]["per_layer_us"]
+            demo[str(Md)]["host_side_us_per_layer"] = round(host, 1)
+            demo[str(Md)]["host_side_share"] = round(host / r["mm_amx_amd"]["per_layer_us"], 3)
+            torch.cuda.empty_cache()
+        extra["llama7b_mlp_stack_32_layers"] = demo
+
         # q against a cache of keys (the mat-vec of test_qk.cpp): 2^21 tokens x head size 128, bf16, 537 MB
         # (more than the 256 MB last-level cache holds)
         T, D = 1 << 21, 128
@@ -624,33 +660,61 @@ def main():
                                                  "frac_of_hbm_peak": round(T * D * 2 / ms / 1e6 / PEAK_HBM_GBS, 4)}
         del keys, sc
 
-        # What a kernel that only streams the same number of bytes takes, launch after launch: the mat-vec kernel
-        # over key caches of the size of the decode weights (45 / 90 / 180 MB, rotated over 541 MB), replayed
-        # from a HIP graph so that no host time is in the figure.  The decode kernels are judged against this.
-        floor = {}
-        for label, Tf in (("45MB", 176128), ("90MB", 352256), ("180MB", 704512)):
-            ks = [torch.randn((Tf, D), dtype=torch.float32, device="cuda").to(torch.bfloat16) for _ in range(12 * 176128 // Tf)]
-            scf = torch.empty(Tf, dtype=torch.float32, device="cuda")
-            nl = len(ks) * 10
+        # What a kernel that only streams the same number of bytes takes, launch after launch, replayed from a HIP graph
+        # so that no host time is in the figure, buffers rotated over 541 MB+ (more than the last-level cache holds).
+        # The decode kernels are judged against the best of these:
+        #   matvec:      the mat-vec kernel over key caches of the size of the decode weights (many short workgroups)
+        #   persistent:  a resident grid of 256 / 512 workgroups, each wave a rolling window of 8 / 16 / 32 KiB of loads
+        #   device_copy: the runtime's own device-to-device copy of as many bytes (reads AND writes them)
+        def graph_us(launch, nl):
             for i in range(nl):
-                mv(ks[i % len(ks)], q, scf)
+                launch(i)
             torch.cuda.synchronize()
             gr, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
             with torch.cuda.stream(side):
                 with torch.cuda.graph(gr, stream=side):
                     for i in range(nl):
-                        mv(ks[i % len(ks)], q, scf)
+                        launch(i)
             torch.cuda.synchronize()
             gr.replay()
             torch.cuda.synchronize()
-            a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a0.record()
-            gr.replay()
-            a1.record()
-            torch.cuda.synchronize()
-            us = a0.elapsed_time(a1) / nl * 1e3
-            floor[label] = {"us": round(us, 2), "GBps": round(Tf * D * 2 / us / 1e3, 0)}
-            del gr, ks, scf
+            ts = []
+            for _ in range(5):
+                a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a0.record()
+                gr.replay()
+                a1.record()
+                torch.cuda.synchronize()
+                ts.append(a0.elapsed_time(a1) / nl * 1e3)
+            del gr
+            return sorted(ts)[2]
+
+        floor = {}
+        sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+        for label, mult in (("45MB", 1), ("90MB", 2), ("180MB", 4)):
+            Tf = 176128 * mult
+            nbytes = Tf * D * 2                      # 45 088 768 bytes = 4096 x 11008 = 5504 x 8 KiB
+            ncopy = 12 // mult
+            ks = [torch.randn((Tf, D), dtype=torch.float32, device="cuda").to(torch.bfloat16) for _ in range(ncopy)]
+            flat = [k.view(torch.uint8).view(-1) for k in ks]
+            scf = torch.empty(Tf, dtype=torch.float32, device="cuda")
+            ent = {}
+            us = graph_us(lambda i: mv(ks[i % ncopy], q, scf), ncopy * 10)
+            ent["matvec"] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3)}
+            for grid in (256, 512):
+                # equal shares of whole 8 KiB per workgroup: the figure is over the bytes actually read
+                share = nbytes // grid // 8192 * 8192
+                for kib in (8, 16, 32):
+                    us = graph_us(lambda i: mx.probe_read(flat[i % ncopy][:share * grid], grid, kib, sink), ncopy * 10)
+                    ent[f"persistent_{grid}wg_{kib}KiB"] = {"us": round(us, 2), "bytes": share * grid, "GBps": round(share * grid / us / 1e3),
+                                                            "us_scaled_to_all_bytes": round(us * nbytes / (share * grid), 2)}
+            dst = torch.empty_like(flat[0])
+            us = graph_us(lambda i: dst.copy_(flat[i % ncopy]), ncopy * 10)
+            ent["device_copy"] = {"us": round(us, 2), "GBps_read_plus_written": round(2 * nbytes / us / 1e3)}
+            best = min(v.get("us_scaled_to_all_bytes", v["us"]) for k, v in ent.items() if k != "device_copy")
+            ent["best_read_only_us"] = best
+            floor[label] = ent
+            del ks, flat, scf, dst
         extra["streaming_read_floor"] = floor
 
         # The vendor library on the same shapes, same box (torch.matmul / torch._int_mm -> hipBLASLt; the bare product,

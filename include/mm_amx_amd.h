@@ -107,6 +107,15 @@ int mmx_repack_gate_up(const void* w_gate, const void* w_up, int64_t ldw_bytes, 
 int mmx_quantize_weights(const void* W, int64_t ldw_bytes, int rows, int cols, void* Wq, int64_t ldq_bytes,
                          float* scales_out, uint32_t* absmax_scratch, void* stream);
 
+/* The quantising half of repackB_1xL<int8_t, L> (weight_compression/fc16m.cpp:61-99), the way fc16m makes its int8
+ * weights (:123, :630-649 with quantize_i8_scale, :51): q = trunc(bf16_rne(float(w) * scale)) per element - the
+ * product is rounded to bf16 first (ov::bfloat16::operator*, include/bf16.hpp:181-183), then converted toward zero
+ * (:80-81).  Where the reference's conversion is undefined the result is defined here: values beyond int8's range
+ * saturate, NaN gives 0.  W is [rows, cols] bf16, Wq [rows, cols] int8; the tile order of that function is
+ * replaced by mmx_repack_b on Wq, and the kernels' per-tensor dequant scale is 1 / scale (:280). */
+int mmx_quantize_weights_scaled(const void* W, int64_t ldw_bytes, int rows, int cols, float scale, void* Wq,
+                                int64_t ldq_bytes, void* stream);
+
 /* int4 weight compression.  The reference only times a stand-in that copies bytes
  * (weight_compression/wcompress.hpp:90-134, README.md:216-244: "we haven't found efficient instructions to
  * implement a fully-functional dequant() for INT4"); this is the real thing for the decode path.  Per output
@@ -220,21 +229,6 @@ const char* mmx_last_kernel(void);
  * over int8 weights, wherever no workgroup gets a second panel (and only while decode_halves and decode_valu are
  * left at -1); 0 never; 1 wherever the shape allows (same bits as the streaming kernel). */
 int mmx_set_option(const char* name, int value);  /* like mmx_set_tile: affects the calling thread's later calls only */
-/* HIP-event timing of `iters` back-to-back launches of the given gemm on `stream`, launch i
- * using the packed weights Bpacked_rot[i % n_rot] (rotate over several copies so that a
- * bandwidth-bound shape is not served from cache); returns the average milliseconds per launch
- * in *ms_out.  Other arguments as for mmx_gemm_splitk.  Blocks until the last launch has finished. */
-int mmx_time_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* const* Bpacked_rot, int n_rot,
-                  int M, int K, int N, int n0, int n1, const mmx_epilogue* ep, int k_splits, void* workspace,
-                  size_t workspace_bytes, void* stream, int iters, float* ms_out);
-
-/* What an issue-bound loop of independent 32x32 MFMAs (dtype MMX_BF16 or MMX_I8) reaches on this device
- * right now, with all-zero operands (random_operands = 0) or with random ones (bf16: N(0,1) x N(0,0.02);
- * int8: uniform): *rate_out in Tflop/s or Top/s, *mhz_out the shader clock during the loop.  The clock of
- * this part under matrix load depends on the operand data; benchmarks report this next to a GEMM's rate.
- * scratch: 16 KiB of device memory.  Blocks until the loop has finished; not thread-safe. */
-int mmx_probe_mfma(int dtype, int random_operands, int iters, void* scratch, void* stream, float* rate_out, float* mhz_out);
-
 #ifdef __cplusplus
 }
 #endif

@@ -296,21 +296,53 @@ struct Workspace {
     void* data = nullptr;
     size_t bytes = 0;
 };
-inline Workspace workspace_for(hipStream_t stream) {
-    static std::mutex mu;
-    static std::map<std::pair<int, hipStream_t>, std::shared_ptr<void>> all;
-    constexpr size_t kBytes = (size_t(64) << 20) + (size_t(16) << 10);
+// `need`: what mmx_gemm_workspace_bytes says the call can use; 0 = the call would not split, nothing is allocated.
+// A stream that is being captured into a graph gets no NEW buffer (an allocation and a memset there would be captured
+// or would invalidate the capture): the call then runs without a K split, whose sums may differ in their last bits
+// from the split form an eager call of the same shape takes.  Buffers live until release_workspaces() or the end of
+// the process (they are deliberately not freed from a static destructor, which may run after the HIP runtime's own).
+inline std::map<std::pair<int, hipStream_t>, Workspace>& workspace_slots() {
+    static auto* all = new std::map<std::pair<int, hipStream_t>, Workspace>();
+    return *all;
+}
+inline std::mutex& workspace_mutex() {
+    static auto* mu = new std::mutex();
+    return *mu;
+}
+// `forced`: the caller named a count of slices: the library then gets a workspace in any case and reports what does not fit.
+inline Workspace workspace_for(hipStream_t stream, size_t need, bool forced = false) {
+    if (need == 0 && !forced) return Workspace();
+    if (need == 0) need = 1;
     int dev = 0;
     check_hip(hipGetDevice(&dev), "workspace_for: hipGetDevice");
-    std::lock_guard<std::mutex> lock(mu);
-    std::shared_ptr<void>& slot = all[std::make_pair(dev, stream)];
-    if (!slot) {
+    std::lock_guard<std::mutex> lock(workspace_mutex());
+    Workspace& slot = workspace_slots()[std::make_pair(dev, stream)];
+    if (slot.bytes < need) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &cap) != hipSuccess) {
+            (void)hipGetLastError();  // (the legacy default stream cannot be queried while another stream captures)
+            cap = hipStreamCaptureStatusActive;
+        }
+        if (cap != hipStreamCaptureStatusNone) return slot.bytes ? slot : Workspace();
+        constexpr size_t kAlways = (size_t(64) << 20) + (size_t(16) << 10);  // serves every shape with k_splits = 0
+        const size_t bytes = need > kAlways ? need : kAlways;
         void* p = nullptr;
-        check_hip(hipMalloc(&p, kBytes), "workspace_for: hipMalloc");
-        check_hip(hipMemset(p, 0, kBytes), "workspace_for: hipMemset");  // the arrival counters start at zero
-        slot = std::shared_ptr<void>(p, [](void* q) { (void)hipFree(q); });
+        check_hip(hipMalloc(&p, bytes), "workspace_for: hipMalloc");
+        check_hip(hipMemset(p, 0, bytes), "workspace_for: hipMemset");  // the arrival counters start at zero
+        if (slot.data) {
+            check_hip(hipStreamSynchronize(stream), "workspace_for: hipStreamSynchronize");  // launches may still use the old one
+            (void)hipFree(slot.data);
+        }
+        slot = Workspace{p, bytes};
     }
-    return Workspace{slot.get(), kBytes};
+    return slot;
+}
+// Frees every workspace (call with no launch in flight, e.g. after hipDeviceSynchronize).
+inline void release_workspaces() {
+    std::lock_guard<std::mutex> lock(workspace_mutex());
+    for (auto& kv : workspace_slots())
+        if (kv.second.data) (void)hipFree(kv.second.data);
+    workspace_slots().clear();
 }
 
 // ---- Matmul<TA,TB,TC> (include/kernels_amx.hpp:1045-1315) ---------------------------------------
@@ -347,7 +379,11 @@ struct Matmul {
         if (!constB || !internalB) internalB = repackB_1x2(matB, transposeB, stream);
         const mmx_epilogue e = ppkernel.descriptor();
         // (decode launches, M <= 32, choose their own slices: they take the workspace with k_splits = 0 only)
-        const Workspace ws = (k_splits == 1 || (M <= 32 && k_splits != 0)) ? Workspace() : workspace_for(stream);
+        const Workspace ws = (k_splits == 1 || (M <= 32 && k_splits != 0))
+                                 ? Workspace()
+                                 : workspace_for(stream, mmx_gemm_workspace_bytes(dtype_of<TA>::value, dtype_of<TB>::value, M, K, N, n0, n1,
+                                                                                  e.steps, k_splits),
+                                                 k_splits > 1);
         check(mmx_gemm_splitk(dtype_of<TA>::value, dtype_of<TB>::value, matA.data, matA.stride, internalB.data, M, K, N, n0, n1,
                               &e, ws.data ? k_splits : 1, ws.data, ws.bytes, stream),
               "Matmul");
@@ -399,7 +435,9 @@ struct Matmul<bfloat16, int8_t, float> {
         }
         ppkernel.set_deq_scale(dequant_scale_B);
         const mmx_epilogue e = ppkernel.descriptor();
-        const Workspace ws = (k_splits == 1 || (M <= 32 && k_splits != 0)) ? Workspace() : workspace_for(stream);
+        const Workspace ws = (k_splits == 1 || (M <= 32 && k_splits != 0))
+                                 ? Workspace()
+                                 : workspace_for(stream, mmx_gemm_workspace_bytes(MMX_BF16, MMX_I8, M, K, N, n0, n1, e.steps, k_splits), k_splits > 1);
         check(mmx_gemm_splitk(MMX_BF16, MMX_I8, matA.data, matA.stride, internalBI8.data, M, K, N, n0, n1, &e,
                               ws.data ? k_splits : 1, ws.data, ws.bytes, stream),
               "Matmul<bf16,int8>");
@@ -532,7 +570,11 @@ struct MLP {
         const int M = x.dims[0];
         require(x.dims[1] == m_K && y.dims[0] == M && y.dims[1] == m_K, "run: x and y must be [M, K]");
         setM(M);
-        const Workspace ws = down_k_splits == 1 ? Workspace() : workspace_for(stream);  // (M <= 32: the library chooses)
+        // the down projection is the GEMM [M, N] x [N, K] (M <= 32: the library chooses its own slices)
+        const Workspace ws = down_k_splits == 1 ? Workspace()
+                                                : workspace_for(stream, mmx_gemm_workspace_bytes(MMX_BF16, MMX_BF16, M, m_N, m_K, 0, m_K, MMX_PP_NONE,
+                                                                                                 M <= 32 ? 0 : down_k_splits),
+                                                                M > 32 && down_k_splits > 1);
         check(mmx_mlp_splitk(x.data, x.stride, gate_up.data, down.data, actUp.data, actUp.stride, y.data, y.stride, M, m_K, m_N,
                              ws.data ? down_k_splits : 1, ws.data, ws.bytes, stream),
               "MLP::run");

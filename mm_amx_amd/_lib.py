@@ -16,9 +16,11 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.environ.get("MMX_LIB_PATH") or os.path.join(_HERE, "libmm_amx_amd.so")
 
 EXPORTS = ["mmx_last_error", "mmx_init", "mmx_packed_b_bytes", "mmx_repack_b", "mmx_repack_gate_up",
-           "mmx_quantize_weights", "mmx_quantize_pack_int4", "mmx_dequant_packed", "mmx_gemm", "mmx_gemm_splitk",
+           "mmx_quantize_weights", "mmx_quantize_weights_scaled", "mmx_quantize_pack_int4", "mmx_dequant_packed", "mmx_gemm", "mmx_gemm_splitk",
            "mmx_gemm_splitk_static", "mmx_gemm_workspace_bytes", "mmx_matvec", "mmx_mlp", "mmx_mlp_splitk", "mmx_set_tile",
-           "mmx_set_option", "mmx_last_kernel", "mmx_time_gemm", "mmx_probe_mfma"]
+           "mmx_set_option", "mmx_last_kernel"]
+# measurement aids (include/mm_amx_amd_bench.h)
+BENCH_EXPORTS = ["mmx_time_gemm", "mmx_probe_mfma", "mmx_probe_read"]
 
 # a workspace of this size serves every shape when the library chooses the K split itself (include/mm_amx_amd.h)
 WORKSPACE_BYTES = (64 << 20) + (16 << 10)
@@ -59,6 +61,8 @@ def lib():
         l.mmx_repack_gate_up.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
         l.mmx_quantize_weights.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p,
                                            C.c_void_p, C.c_void_p]
+        l.mmx_quantize_weights_scaled.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_int64,
+                                                  C.c_void_p]
         l.mmx_quantize_pack_int4.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
                                              C.c_void_p]
         l.mmx_dequant_packed.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
@@ -82,6 +86,7 @@ def lib():
                                     C.c_void_p, C.c_int, C.POINTER(C.c_float)]
         l.mmx_probe_mfma.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.POINTER(C.c_float),
                                      C.POINTER(C.c_float)]
+        l.mmx_probe_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
         _lib = l
     return _lib
 
@@ -188,6 +193,18 @@ def quantize_weights(W):
     return Wq, scales
 
 
+def quantize_weights_scaled(W, scale):
+    """q = trunc(bf16_rne(w * scale)) per element, int8: how repackB_1xL<int8_t> (weight_compression/fc16m.cpp:80-81)
+    makes fc16m's int8 weights; the matching per-tensor dequant scale is 1 / scale."""
+    _dev(W, "W")
+    if W.dtype != torch.bfloat16 or W.dim() != 2:
+        raise MmxError("W must be a 2-D bf16 tensor")
+    Wq = torch.empty(W.shape, dtype=torch.int8, device=W.device)
+    _check(lib().mmx_quantize_weights_scaled(W.data_ptr(), _row_stride_bytes(W), W.shape[0], W.shape[1], float(scale),
+                                             Wq.data_ptr(), _row_stride_bytes(Wq), _stream()))
+    return Wq
+
+
 def quantize_pack_int4(W, transpose=False):
     """Per-output-channel symmetric int4 compression of a bf16 matrix W [K,N] (or [N,K] with transpose), packed for
     gemm(..., b_dtype=I4) with M <= 32; returns (packed uint8, deq_scales fp32 [N])."""
@@ -208,23 +225,33 @@ def dequant_packed(packed_i8, K, N):
     return out
 
 
-_workspaces = {}
+_workspaces = {}          # (device, raw stream handle) -> uint8 tensor; insertion order = age
+_MAX_WORKSPACES = 8       # stream handles are reused after a stream is destroyed: the cache is bounded
 
 
 def workspace(device=None, nbytes=WORKSPACE_BYTES):
     """The K-split workspace of the current stream on `device` (zeroed once, when it is created).  Calls
     on one stream are ordered, so one workspace per stream is enough; returns None while the stream is
-    being captured into a graph and has no workspace yet (an allocation there would be captured too)."""
+    being captured into a graph and has no workspace of that size yet (an allocation there would be captured
+    too).  At most _MAX_WORKSPACES are kept (the oldest is dropped); release_workspaces() drops them all."""
     dev_index = torch.cuda.current_device() if device is None else (device.index or 0)
     key = (dev_index, torch.cuda.current_stream(dev_index).cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         if torch.cuda.is_current_stream_capturing():
             return None
-        ws = torch.zeros(nbytes, dtype=torch.uint8, device=f"cuda:{dev_index}")
+        ws = torch.zeros(max(nbytes, WORKSPACE_BYTES), dtype=torch.uint8, device=f"cuda:{dev_index}")
         torch.cuda.current_stream(dev_index).synchronize()
+        _workspaces.pop(key, None)
         _workspaces[key] = ws
+        while len(_workspaces) > _MAX_WORKSPACES:
+            _workspaces.pop(next(iter(_workspaces)))
     return ws
+
+
+def release_workspaces():
+    """Drops every cached K-split workspace (the memory returns to torch's allocator once no launch uses it)."""
+    _workspaces.clear()
 
 
 def _is_2d(t, what):
@@ -268,12 +295,17 @@ def _packed_bytes_host(dtype, K, N):
     return ((N + 31) // 32) * 32 * ((K * es + 127) // 128 * 128)
 
 
-def _split_args(A, k_splits, ws):
-    """(k_splits, workspace pointer, bytes): without an explicit workspace the stream's own one is used."""
+def _split_args(A, k_splits, ws, need):
+    """(k_splits, workspace pointer, bytes).  Without an explicit workspace the stream's own one is used, and it is
+    only created when the library says the call can use one (`need` = mmx_gemm_workspace_bytes of the call, a
+    callable): a shape that never splits allocates nothing."""
     if k_splits == 1 and ws is None:
         return 1, None, 0
     if ws is None:
-        ws = workspace(A.device)
+        nbytes = need()
+        if nbytes == 0 and k_splits == 0:
+            return 1, None, 0
+        ws = workspace(A.device, max(nbytes, 1))  # (an explicit count that does not fit: the library says why)
     if ws is None:
         if k_splits > 1:
             raise MmxError("a K split needs a workspace, and none can be allocated while the stream is being captured")
@@ -286,13 +318,16 @@ def _split_args(A, k_splits, ws):
 def gemm(A, Bpacked, N, ep, b_dtype=None, n0=0, n1=None, k_splits=0, ws=None):
     """C[:, n0:n1] = PP(A · B[:, n0:n1]); A [M,K] bf16/int8, Bpacked from repack_b of the full [K,N].
     k_splits: 0 = the library decides whether to split K over several workgroups per tile, 1 = never,
-    2..4 = exactly that many slices; ws = the workspace for the partial sums (default: the stream's own)."""
+    2..4 = exactly that many slices; ws = the workspace for the partial sums (default: the stream's own, created at
+    the first call that can use one).  A first call of a shape made while the stream is being captured into a graph
+    finds no workspace and runs unsplit: its sums can differ in the last bits from an eager call of the same shape,
+    which splits.  Call the shape once eagerly before capturing (or pass ws) to have both take the same form."""
     n1 = N if n1 is None else n1
     b_dt = (dtype_code(A) if isinstance(A, torch.Tensor) else None) if b_dtype is None else b_dtype
     M, K, a_dt = _check_gemm_args(A, Bpacked, N, ep, b_dt, n0, n1)
     _dev(A, "A"), _dev(Bpacked, "Bpacked")
     s = ep.struct()
-    ks, wsp, wsb = _split_args(A, k_splits, ws)
+    ks, wsp, wsb = _split_args(A, k_splits, ws, lambda: gemm_workspace_bytes(a_dt, b_dt, M, K, N, ep.steps, k_splits, n0, n1))
     _check(lib().mmx_gemm_splitk(a_dt, b_dt, A.data_ptr(), _row_stride_bytes(A), Bpacked.data_ptr(), M, K, N, n0, n1,
                                  C.byref(s), ks, wsp, wsb, _stream()))
 
@@ -323,7 +358,7 @@ def time_gemm(A, Bpacked_list, N, ep, iters, b_dtype=None, n0=0, n1=None, k_spli
     s = ep.struct()
     arr = (C.c_void_p * len(Bpacked_list))(*[b.data_ptr() for b in Bpacked_list])
     ms = C.c_float(0)
-    ks, wsp, wsb = _split_args(A, k_splits, ws)
+    ks, wsp, wsb = _split_args(A, k_splits, ws, lambda: gemm_workspace_bytes(a_dt, b_dt, M, K, N, ep.steps, k_splits, n0, n1))
     _check(lib().mmx_time_gemm(a_dt, b_dt, A.data_ptr(), _row_stride_bytes(A), arr, len(Bpacked_list), M, K, N, n0,
                                n1, C.byref(s), ks, wsp, wsb, _stream(), iters, C.byref(ms)))
     return ms.value
@@ -336,6 +371,11 @@ def probe_mfma(dtype, random_operands, iters=20000):
     _check(lib().mmx_probe_mfma(dtype, int(bool(random_operands)), iters, scratch.data_ptr(), _stream(), C.byref(rate),
                                 C.byref(mhz)))
     return rate.value, mhz.value
+
+
+def probe_read(buf, workgroups, kib_in_flight, sink):
+    """One launch of the read-only kernel over the uint8 tensor `buf` (asynchronous; see mm_amx_amd_bench.h)."""
+    _check(lib().mmx_probe_read(buf.data_ptr(), buf.numel(), int(workgroups), int(kib_in_flight), sink.data_ptr(), _stream()))
 
 
 def matvec(A, b, out=None):
@@ -382,7 +422,9 @@ def mlp(x, w_gate_up, w_down, N, h=None, y=None, down_k_splits=0, ws=None):
     if y is None:
         y = torch.empty((M, K), dtype=torch.bfloat16, device=x.device)
     _dev(h, "h"), _dev(y, "y")
-    ks, wsp, wsb = _split_args(x, down_k_splits, ws)
+    # the down projection is the GEMM [M, N] x [N, K]; decode shapes (M <= 32) choose their own slices
+    ks, wsp, wsb = _split_args(x, down_k_splits, ws,
+                               lambda: gemm_workspace_bytes(BF16, BF16, M, N, K, PP_NONE, 0 if M <= 32 else down_k_splits))
     _check(lib().mmx_mlp_splitk(x.data_ptr(), _row_stride_bytes(x), w_gate_up.data_ptr(), w_down.data_ptr(), h.data_ptr(),
                                 _row_stride_bytes(h), y.data_ptr(), _row_stride_bytes(y), M, K, N, ks, wsp, wsb, _stream()))
     return h, y

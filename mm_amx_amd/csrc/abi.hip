@@ -6,6 +6,7 @@
 #include <mutex>
 
 #include "common.hpp"
+#include "../../include/mm_amx_amd_bench.h"
 
 namespace mmx {
 
@@ -76,10 +77,12 @@ int launch_repack(int elesz, const void* B, int64_t ldb, int K, int N, int trans
 int launch_repack_gate_up(const void* wg, const void* wu, int64_t ldw, int K, int N, void* out, hipStream_t st);
 int launch_quantize(const void* W, int64_t ldw, int rows, int cols, void* Wq, int64_t ldq, float* scales_out,
                     uint32_t* scratch, hipStream_t st);
+int launch_quantize_scale_trunc(const void* W, int64_t ldw, int rows, int cols, float scale, void* Wq, int64_t ldq, hipStream_t st);
 int launch_dequant_packed(const void* in, int K, int N, void* out, hipStream_t st);
 int probe_mfma(bool i8, int random_operands, int iters, void* scratch, hipStream_t st, float* rate_out, float* mhz_out);
 int launch_quantize_pack_int4(const void* W, int64_t ldw, int K, int N, int transpose, void* packed, float* deq_out,
                               hipStream_t st);
+int probe_read(const void* buf, size_t bytes, int workgroups, int kib_in_flight, void* sink, hipStream_t st);
 int launch_matvec(bool i8, const void* A, int64_t lda, const void* b, void* c, int M, int K, hipStream_t st);
 
 struct TileCfg {
@@ -92,12 +95,14 @@ static thread_local int g_decode_halves = -1;
 static thread_local int g_decode_valu = -1;
 static thread_local int g_decode_resident = -1;
 static thread_local int g_waves = 8;
+static thread_local int g_a_kblocked = 0;
 TileCfg forced_tile() { return g_forced; }
 int load_mode() { return g_load_mode; }
 int decode_halves() { return g_decode_halves; }
 int decode_valu() { return g_decode_valu; }
 int decode_resident() { return g_decode_resident; }
 int wave_count() { return g_waves; }
+int a_kblocked() { return g_a_kblocked; }
 
 static int elesz_of(int dtype) { return dtype == MMX_BF16 ? 2 : dtype == MMX_I8 ? 1 : 0; }
 
@@ -258,6 +263,16 @@ int mmx_quantize_weights(const void* W, int64_t ldw_bytes, int rows, int cols, v
     return launch_quantize(W, ldw_bytes, rows, cols, Wq, ldq_bytes, scales_out, absmax_scratch, static_cast<hipStream_t>(stream));
 }
 
+int mmx_quantize_weights_scaled(const void* W, int64_t ldw_bytes, int rows, int cols, float scale, void* Wq, int64_t ldq_bytes,
+                                void* stream) {
+    if (!W || !Wq) return set_error(MMX_E_INVALID, "mmx_quantize_weights_scaled: NULL pointer");
+    if (rows <= 0 || cols <= 0 || ldw_bytes < (int64_t)cols * 2 || ldq_bytes < cols)
+        return set_error(MMX_E_INVALID, "mmx_quantize_weights_scaled: bad shape or stride");
+    if ((ldw_bytes & 1) || (reinterpret_cast<uintptr_t>(W) & 1))
+        return set_error(MMX_E_INVALID, "mmx_quantize_weights_scaled: W is not aligned to its element size");
+    return launch_quantize_scale_trunc(W, ldw_bytes, rows, cols, scale, Wq, ldq_bytes, static_cast<hipStream_t>(stream));
+}
+
 int mmx_quantize_pack_int4(const void* W, int64_t ldw_bytes, int K, int N, int transpose, void* packed, float* deq_scales_out,
                            void* stream) {
     if (!W || !packed || !deq_scales_out) return set_error(MMX_E_INVALID, "mmx_quantize_pack_int4: NULL pointer");
@@ -389,6 +404,11 @@ int mmx_set_option(const char* name, int value) {
         g_decode_resident = value;
         return MMX_OK;
     }
+    if (name && !strcmp(name, "a_kblocked")) {
+        if (value != 0 && value != 1) return set_error(MMX_E_INVALID, "mmx_set_option: a_kblocked is 0 or 1");
+        g_a_kblocked = value;
+        return MMX_OK;
+    }
     if (name && !strcmp(name, "waves")) {
         if (value != 4 && value != 8) return set_error(MMX_E_INVALID, "mmx_set_option: waves is 4 or 8");
         g_waves = value;
@@ -401,6 +421,12 @@ int mmx_probe_mfma(int dtype, int random_operands, int iters, void* scratch, voi
     if ((dtype != MMX_BF16 && dtype != MMX_I8) || iters <= 0 || !scratch || !rate_out || !mhz_out)
         return set_error(MMX_E_INVALID, "mmx_probe_mfma: bad argument");
     return probe_mfma(dtype == MMX_I8, random_operands, iters, scratch, static_cast<hipStream_t>(stream), rate_out, mhz_out);
+}
+
+int mmx_probe_read(const void* buf, size_t bytes, int workgroups, int kib_in_flight, void* sink, void* stream) {
+    if (!buf || !sink || workgroups <= 0 || workgroups > 65536 || (reinterpret_cast<uintptr_t>(buf) & 15))
+        return set_error(MMX_E_INVALID, "mmx_probe_read: bad argument");
+    return probe_read(buf, bytes, workgroups, kib_in_flight, sink, static_cast<hipStream_t>(stream));
 }
 
 int mmx_time_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* const* Bpacked_rot, int n_rot, int M,

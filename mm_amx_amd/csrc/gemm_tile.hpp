@@ -95,6 +95,7 @@ struct Mfma<int8_t> {
 struct GemmArgs {
     const char* A;
     int64_t lda;           // bytes
+    int64_t a_kstride;     // bytes from one 128-byte k-iteration of a row of A to the next (128: rows are contiguous)
     const char* Bp;        // packed weights
     int64_t panel_stride;  // bytes per 32-column panel = nk * 4096
     int M;
@@ -108,6 +109,7 @@ struct GemmArgs {
     int kq;        // k-iterations per slice
     char* ws_part;     // partial accumulators of the K slices: [tile][slice][BM*BN] 4-byte words
     uint32_t* ws_cnt;  // one arrival counter per tile, zero between launches
+    uint64_t* stamps;  // instrumented build only: 64 bytes per workgroup for its phase stamps, or null
     Epilogue ep;
 };
 
@@ -165,12 +167,13 @@ struct Ring {
 // SMAX: the largest number of K slices per tile this instantiation can combine (1: no K split; the
 // code of the split is then absent and the kernel is the plain one).
 // Development aid, compiled in with -DMMX_STAMPS only: workgroup L records the shader clock at a few points of
-// its life in the 64 bytes at ws_part + 96 MiB + 64 L (the caller provides that much workspace).
+// its life in the 64 bytes at ws_part + 96 MiB + 64 L; the host passes that address (GemmArgs::stamps) only when the
+// caller's workspace reaches that far, so an ordinary workspace is never written outside.
 #ifdef MMX_STAMPS
 #define MMX_STAMP(i)                                                                                                   \
     do {                                                                                                               \
-        if (threadIdx.x == 0 && g.ws_part) {                                                                           \
-            uint64_t* st_ = reinterpret_cast<uint64_t*>(g.ws_part + ((size_t)96 << 20)) + 8 * (size_t)L;              \
+        if (threadIdx.x == 0 && g.stamps) {                                                                            \
+            uint64_t* st_ = g.stamps + 8 * (size_t)L;                                                                  \
             st_[i] = (i) == 0 || (i) == 7 ? __builtin_amdgcn_s_memrealtime() : __builtin_readcyclecounter();          \
         }                                                                                                              \
     } while (0)
@@ -223,7 +226,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4,
         kt0 = slice * g.kq;
         nk = g.nk - kt0 < g.kq ? g.nk - kt0 : g.kq;
     }
-    const char* const a_base = g.A + (int64_t)kt0 * 128;
+    const char* const a_base = g.A + (int64_t)kt0 * g.a_kstride;
     const int tn = tile / g.tiles_m, tm = tile % g.tiles_m;
     MMX_STAMP(0);
     MMX_STAMP(1);
@@ -454,7 +457,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4,
             } else if constexpr (PART == 2) {
                 int st = (w + 1) >> 1;
                 st = st < last_st ? st : last_st;
-                n.srcA = a_base + (int64_t)st * 128;
+                n.srcA = a_base + (int64_t)st * g.a_kstride;
                 asm volatile("" : "+s"(n.srcA));
             } else {
                 // A operand of k-step s (0..3 within the stage): position (2 s + g32) ^ ((row >> 1) & 7) of the row
@@ -553,7 +556,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4,
                 kp.m0B = lds_wave + B0 + W * BH;
                 kp.m0A = lds_wave + (((W + 1) >> 1) % RA) * A_ST + HALF * (BM / 2) * 128;
                 kp.srcB = b_base + (int64_t)hs * BP_HS;
-                kp.srcA = a_base + (int64_t)st * 128;
+                kp.srcA = a_base + (int64_t)st * g.a_kstride;
                 static_for<0, (W < R - 1 ? NL : H)>([&](auto q_c) { dma(q_c, integral_constant<int, HALF>{}, kp); });
             });
         }
@@ -976,6 +979,7 @@ struct TileCfg {
 TileCfg forced_tile();
 int load_mode();
 int wave_count();
+int a_kblocked();
 int ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done_on_device);
 
 // Where the partial sums of a K split live: the first WS_COUNTER_BYTES hold one arrival counter per tile
@@ -1124,6 +1128,7 @@ static inline int prepare_gemm(GemmArgs& g, TileCfg& t, int& mode, int elesz, co
                                int M, int K, int N, int n0, int n1, const Epilogue& ep, const SplitRequest& rq, bool w8 = false) {
     g.A = static_cast<const char*>(A);
     g.lda = lda;
+    g.a_kstride = 128;
     g.Bp = static_cast<const char*>(Bp);
     g.M = M;
     g.kbytes = K * elesz;
@@ -1159,10 +1164,19 @@ static inline int prepare_gemm(GemmArgs& g, TileCfg& t, int& mode, int elesz, co
     g.kq = plan.S > 1 ? slice_kiters(g.nk, plan.S) : g.nk;
     g.ws_cnt = reinterpret_cast<uint32_t*>(use.ws);
     g.ws_part = use.ws ? use.ws + WS_COUNTER_BYTES : nullptr;
+    g.stamps = nullptr;
+    if (a_kblocked() && mode == 2) {  // A as [K * elesz / 128][M][128 bytes]: a load instruction's 8 rows x 128 bytes are contiguous
+        g.lda = 128;
+        g.a_kstride = (int64_t)M * 128;
+    }
     g.tiles_m = (M + t.bm - 1) / t.bm;
     const int tiles_n = (n1 - n0 + t.bn - 1) / t.bn;
     g.total_tiles = g.tiles_m * tiles_n * g.ksplit;
     g.tiles_per_xcd = (g.total_tiles + 7) / 8;
+#ifdef MMX_STAMPS
+    if (use.ws && use.ws_bytes >= WS_COUNTER_BYTES + ((size_t)96 << 20) + (size_t)64 * g.tiles_per_xcd * 8)
+        g.stamps = reinterpret_cast<uint64_t*>(g.ws_part + ((size_t)96 << 20));
+#endif
     return g.tiles_per_xcd * 8;
 }
 

@@ -85,6 +85,34 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(uint64_t* stamps, int ra
     }
 }
 
+
+// A grid of resident workgroups that only reads: workgroup g walks the g-th of gridDim.x equal shares of the buffer,
+// its eight waves side by side (wave w takes the 1 KiB pieces w, w + 8, ... of the share), each wave with U pieces
+// in flight as a rolling window: piece i + U is requested as soon as piece i has been consumed (one XOR per dword).
+template <int U>
+__global__ __launch_bounds__(512) void read_stream_kernel(const char* buf, int pieces_per_wave, uint32_t* sink, uint32_t unlikely) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+    const char* p = buf + ((size_t)blockIdx.x * pieces_per_wave * 8 + wave) * 1024 + lane * 16;
+    u32x4 w[U];
+    uint32_t x = 0;
+    const int last = pieces_per_wave - 1;
+#pragma unroll
+    for (int u = 0; u < U; u++) w[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + (size_t)(u < last ? u : last) * 8192));
+    for (int i0 = 0; i0 < pieces_per_wave; i0 += U) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            x ^= w[u][0] ^ w[u][1] ^ w[u][2] ^ w[u][3];
+            int nx = i0 + U + u;  // past the end: the last piece once more (it stays in the window, unused)
+            nx = nx < last ? nx : last;
+            w[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + (size_t)nx * 8192));
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) x ^= w[u][0] & 1u;  // (the trailing requests must be waited for before the wave ends)
+    if (x == unlikely) *sink = x;  // keeps the loads alive; one lane in 2^32 writes 4 harmless bytes
+}
+
 }  // namespace
 
 // scratch: 1024 waves x 16 bytes on the device.  Synchronises the stream (it reads the stamps back).
@@ -115,6 +143,22 @@ int probe_mfma(bool i8, int random_operands, int iters, void* scratch, hipStream
     *rate_out = (float)(ops / us / 1e6);  // Tflop/s or Top/s
     *mhz_out = (float)(cyc / us);
     return MMX_OK;
+}
+
+int probe_read(const void* buf, size_t bytes, int workgroups, int kib_in_flight, void* sink, hipStream_t st) {
+    const size_t per_wg = bytes / (size_t)workgroups;
+    if (per_wg * workgroups != bytes || per_wg % 8192 || per_wg == 0 || per_wg / 8192 > (size_t)1 << 20)
+        return set_error(MMX_E_INVALID, "mmx_probe_read: %zu bytes do not divide into %d shares of whole 8 KiB", bytes, workgroups);
+    const int ppw = (int)(per_wg / 8192);
+    const char* b = static_cast<const char*>(buf);
+    uint32_t* s = static_cast<uint32_t*>(sink);
+    switch (kib_in_flight) {
+    case 8: hipLaunchKernelGGL(read_stream_kernel<8>, dim3(workgroups), dim3(512), 0, st, b, ppw, s, 0x9e3779b9u); break;
+    case 16: hipLaunchKernelGGL(read_stream_kernel<16>, dim3(workgroups), dim3(512), 0, st, b, ppw, s, 0x9e3779b9u); break;
+    case 32: hipLaunchKernelGGL(read_stream_kernel<32>, dim3(workgroups), dim3(512), 0, st, b, ppw, s, 0x9e3779b9u); break;
+    default: return set_error(MMX_E_INVALID, "mmx_probe_read: kib_in_flight is 8, 16 or 32");
+    }
+    return check_hip(hipGetLastError(), "read_stream_kernel launch");
 }
 
 }  // namespace mmx

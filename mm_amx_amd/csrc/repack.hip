@@ -137,6 +137,33 @@ int launch_quantize(const void* W, int64_t ldw, int rows, int cols, void* Wq, in
     return check_hip(hipGetLastError(), "quantize kernels launch");
 }
 
+// q = trunc(bf16_rne(float(w) * scale)): the element conversion of repackB_1xL<int8_t, L>
+// (weight_compression/fc16m.cpp:80-81, "*dst++ = src0[n] * scale" with src0 an ov::bfloat16* and dst an int8_t*: the
+// product is a bfloat16 again, include/bf16.hpp:181-183, and its conversion to int8_t goes through float and
+// truncates toward zero).  Values the language leaves undefined are defined here: beyond int8's range saturates,
+// NaN gives 0.
+__global__ void quantize_scale_trunc_kernel(const char* __restrict__ W, int64_t ldw, int rows, int cols, float scale,
+                                            char* __restrict__ Wq, int64_t ldq) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < (int64_t)rows * cols;
+         i += (int64_t)gridDim.x * blockDim.x) {
+        const int r = (int)(i / cols), c = (int)(i % cols);
+        const float w = from_bf16(*reinterpret_cast<const uint16_t*>(W + (int64_t)r * ldw + (int64_t)c * 2));
+        const float t = from_bf16(to_bf16(w * scale));
+        int q = 0;
+        if (t == t) q = t >= 127.0f ? 127 : (t <= -128.0f ? -128 : (int)t);  // float -> int: toward zero
+        Wq[(int64_t)r * ldq + c] = (char)q;
+    }
+}
+
+int launch_quantize_scale_trunc(const void* W, int64_t ldw, int rows, int cols, float scale, void* Wq, int64_t ldq, hipStream_t st) {
+    const int64_t n = (int64_t)rows * cols;
+    int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(quantize_scale_trunc_kernel, dim3(blocks), dim3(256), 0, st, static_cast<const char*>(W), ldw, rows, cols,
+                       scale, static_cast<char*>(Wq), ldq);
+    return check_hip(hipGetLastError(), "quantize_scale_trunc_kernel launch");
+}
+
 // ---- packed int8 -> packed bf16 (exact) -------------------------------------------------------------
 // int8 slot (panel, f, lane): 16 consecutive k of column n -> bf16 fragments 2f and 2f+1 ... the
 // 16 k's starting at 32f + 16g split into two runs of 8: run h goes to bf16 fragment 2f+g,

@@ -43,7 +43,20 @@ struct SkinnyArgs {
     char* ws_part;
     uint32_t* ws_cnt;
     int kslices;
+    uint64_t* stamps;  // instrumented build only (-DMMX_STAMPS): 64 bytes per workgroup for its phase stamps, or null
 };
+
+// Development aid, compiled in with -DMMX_STAMPS only: thread 0 of workgroup blockIdx.x records the wall clock (100 MHz,
+// slots 0 and 7) or the shader clock (the others) at a few points of the workgroup's life.
+#ifdef MMX_STAMPS
+#define SKINNY_STAMP(i)                                                                                                 \
+    do {                                                                                                                \
+        if (threadIdx.x == 0 && s.stamps)                                                                               \
+            s.stamps[8 * (size_t)blockIdx.x + (i)] = (i) == 0 || (i) == 7 ? __builtin_amdgcn_s_memrealtime() : __builtin_readcyclecounter(); \
+    } while (0)
+#else
+#define SKINNY_STAMP(i) do {} while (0)
+#endif
 
 __device__ __forceinline__ bf16x8 load_x8(const char* xrow, int k0, int K, bool live, bool vec_ok) {
     bf16x8 v;
@@ -630,6 +643,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const int panel_end = (s.n1 + 31) >> 5;
     const int row_bytes = s.K * (I8A ? 1 : 2);
     const int real_bytes = s.M * row_bytes;
+    SKINNY_STAMP(0);
+    SKINNY_STAMP(1);
 
     // x -> LDS, 1 KiB per wave per instruction; the lanes past the end of x re-read its last 16 bytes
     // into the gap in front of the zero row (zero_off is the next multiple of 1 KiB)
@@ -732,6 +747,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" : : "n"(U0 * NP) : "memory");
         __builtin_amdgcn_sched_barrier(0);
+        SKINNY_STAMP(2);
 #pragma unroll
         for (int u = U0; u < U; u++) MMX_REQUEST(0, u);
     }
@@ -752,7 +768,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #undef MMX_REQUEST
 #undef MMX_MULTIPLY
 
+    SKINNY_STAMP(3);
     __syncthreads();  // every wave has read its last x: the buffer becomes the reduction scratch
+    SKINNY_STAMP(4);
     if constexpr (VALU) {
         // lane (column l32, k half g32): add the other half's sum, then put the column's value where the
         // matrix-core form would hold it (output row 0 of a 32x32 block), so that the post-op below is shared
@@ -770,6 +788,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     }
     __syncthreads();
     skinny_finish<NP, I8A>(s, red, panel_first, tid, fin);
+    SKINNY_STAMP(5);
+    SKINNY_STAMP(7);
 }
 
 // ---- resident-x variant: more rows than two workgroups per CU can hold a copy of ----------------------
@@ -1258,7 +1278,12 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
     s.ws_part = nullptr;
     s.ws_cnt = nullptr;
     s.kslices = 1;
+    s.stamps = nullptr;
     const int panels = ((n1 + 31) >> 5) - (n0 >> 5);
+#ifdef MMX_STAMPS
+    if (rq && rq->ws && rq->ws_bytes >= SPLIT_COUNTER_BYTES + ((size_t)96 << 20) + (size_t)64 * 2 * panels)
+        s.stamps = reinterpret_cast<uint64_t*>(rq->ws + SPLIT_COUNTER_BYTES + ((size_t)96 << 20));
+#endif
     const bool pairs = (ep.steps & MMX_PP_SILU_GATE) != 0;
     if (wk == 3) {
         // int8 activations x int8 weights (int32 sums): the caller has checked skinny_i8_eligible and uses the tile

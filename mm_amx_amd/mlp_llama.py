@@ -58,7 +58,7 @@ class LlamaMLP(torch.nn.Module):
         return F.linear(F.silu(F.linear(x, self.w_gate)) * F.linear(x, self.w_up), self.w_down)
 
 
-def perf_llama7b_MLP(M=256, num_layers=32, rounds=10, hidden_size=4096, intermediate_size=11008, verbose=True):
+def perf_llama7b_MLP(M=256, num_layers=32, rounds=10, hidden_size=4096, intermediate_size=11008, verbose=True, graph=False):
     layers = []
     for i in range(num_layers):
         layers += [LlamaRMSNorm(), LlamaMLP(hidden_size, intermediate_size, seed=i)]
@@ -84,6 +84,31 @@ def perf_llama7b_MLP(M=256, num_layers=32, rounds=10, hidden_size=4096, intermed
             if verbose:
                 print(f"{name:>11}: per-layer dt {dt * 1e6:9.1f} us   GFlops {out[name]['GFlops']:10.0f}   "
                       f"GB/s {out[name]['GBps']:8.0f}")
+        if graph:
+            # the same stack through this library replayed from a HIP graph: what is left when the host side of every
+            # call (Python, ctypes marshalling, launch) is taken out of the per-layer figure
+            side = torch.cuda.Stream()
+            with torch.cuda.stream(side):
+                net(x)  # (an eager pass on this stream first: the K-split workspace of a stream is made outside a capture)
+                torch.cuda.synchronize()
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr, stream=side):
+                    yg = net(x)
+            torch.cuda.synchronize()
+            gr.replay()
+            torch.cuda.synchronize()
+            t0 = time.time()
+            for _ in range(rounds):
+                gr.replay()
+            torch.cuda.synchronize()
+            dt = (time.time() - t0) / rounds / num_layers
+            out["mm_amx_amd_graph"] = {"per_layer_us": dt * 1e6, "GFlops": mlps[0].flops(M) * 1e-9 / dt,
+                                       "GBps": mlps[0].numel(M) * 2 * 1e-9 / dt,
+                                       "same_bits_as_eager": bool(torch.equal(yg.float(), out["y_mm_amx_amd"]))}
+            if verbose:
+                print(f"{'graph':>11}: per-layer dt {dt * 1e6:9.1f} us   GFlops {out['mm_amx_amd_graph']['GFlops']:10.0f}   "
+                      f"GB/s {out['mm_amx_amd_graph']['GBps']:8.0f}")
+            del gr
     y0, y1 = out.pop("y_torch"), out.pop("y_mm_amx_amd")
     out["rel_err"] = (torch.linalg.norm(y1 - y0) / torch.linalg.norm(y0)).item()
     # one layer on the same input: the stack has no residual connections, so rounding differences of
@@ -106,6 +131,7 @@ if __name__ == "__main__":
     ap.add_argument("--M", type=int, default=256)
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--rounds", type=int, default=10)
+    ap.add_argument("--graph", action="store_true", help="also replay the stack from a HIP graph")
     a = ap.parse_args()
     ops.L.init(0)
-    perf_llama7b_MLP(a.M, a.layers, a.rounds)
+    perf_llama7b_MLP(a.M, a.layers, a.rounds, graph=a.graph)

@@ -17,6 +17,18 @@ def bf16_bits_to_f32(b):
     return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
 
 
+def to_device(a, device="cuda"):
+    """numpy array -> torch tensor on the GPU, same bytes."""
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def to_device_bf16(bits, device="cuda"):
+    """uint16 bf16 bit patterns (numpy) -> torch.bfloat16 on the GPU, same bytes."""
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).to(device).view(torch.bfloat16)
+
+
 def _normal_bf16(rng, shape, std):
     return f32_to_bf16_bits((rng.standard_normal(shape, dtype=np.float32) * np.float32(std)))
 

@@ -187,6 +187,44 @@ float orc_quantize_weights(const uint16_t* W, int64_t ldw, int rows, int cols, i
     return dq;
 }
 
+/* ------------------------------------------------------------------------------------ */
+/* The quantising half of repackB_1xL<int8_t, L> (weight_compression/fc16m.cpp:61-99): every element goes through
+ *     *dst++ = src0[n] * scale;                                  (:80-81)
+ * with src0 an ov::bfloat16* and dst an int8_t*.  ov::bfloat16::operator*(float) (include/bf16.hpp:181-183) returns
+ * a bfloat16 built from the fp32 product, i.e. rounded to nearest even (include/bf16.hpp:14, :95-107), and the
+ * assignment to int8_t converts that bfloat16 through operator float() (:70-76) with the language's float -> integer
+ * conversion: truncation toward zero.  So q = trunc(bf16_rne(float(w) * scale)).  The language leaves a value
+ * outside [-128, 127] (and NaN) undefined; here it saturates (NaN -> 0), and fc16m's own use (fill_rnd weights
+ * times quantize_i8_scale = 2, :51, :123) never gets there. */
+int8_t orc_bf16_scale_trunc_s8(uint16_t w, float scale) {
+    const float prod = orc_bf16_to_f32(w) * scale;
+    const float r = orc_bf16_to_f32(orc_f32_to_bf16(prod));
+    if (r != r) return 0;
+    if (r >= 127.0f) return 127;
+    if (r <= -128.0f) return -128;
+    return (int8_t)(int)r;  /* C conversion: toward zero */
+}
+
+void orc_quantize_scale_trunc(const uint16_t* W, int64_t ldw, int rows, int cols, float scale, int8_t* Wq, int64_t ldq) {
+    for (int r = 0; r < rows; r++)
+        for (int c = 0; c < cols; c++) Wq[(size_t)r * ldq + c] = orc_bf16_scale_trunc_s8(W[(size_t)r * ldw + c], scale);
+}
+
+/* repackB_1xL<int8_t, L> whole (weight_compression/fc16m.cpp:61-99): B [K, N] bf16 (K % 32 == 0, N % (16 L) == 0)
+ * -> K*N int8 in the function's own order: column groups of 16 L in computation order, K in blocks of 32, L tiles
+ * per block; a tile is 16 pairs of k, each pair 16 columns x (k, k + 1) interleaved (:76-86). */
+void orc_repack_1xL_s8(const uint16_t* B, int64_t ldb, int K, int N, int L, float scale, int8_t* out) {
+    int8_t* dst = out;
+    for (int n0 = 0; n0 < N; n0 += L * 16)
+        for (int k0 = 0; k0 < K; k0 += 32)
+            for (int l = 0; l < L; l++)
+                for (int k = 0; k < 32; k += 2)
+                    for (int n = 0; n < 16; n++) {
+                        *dst++ = orc_bf16_scale_trunc_s8(B[(size_t)(k0 + k) * ldb + n0 + l * 16 + n], scale);
+                        *dst++ = orc_bf16_scale_trunc_s8(B[(size_t)(k0 + k + 1) * ldb + n0 + l * 16 + n], scale);
+                    }
+}
+
 /* int4 weight compression.  The reference has no algorithm to restate here: weight_compression/wcompress.hpp:90-134
  * and README.md:216-244 only time a stand-in that copies bytes ("we haven't found efficient instructions to
  * implement a fully-functional dequant() for INT4").  This is the definition the device code is held to:

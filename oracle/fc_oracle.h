@@ -25,6 +25,13 @@
  *                                    counterpart); checked to be a bijection + zero pad
  *   orc_quantize_weights   pinned  — against the compiled reference Matmul<bf16,int8>
  *   orc_gemv_w8            pinned  — through orc_gemm_bf16 on exactly converted weights
+ *   orc_bf16_scale_trunc_s8, orc_quantize_scale_trunc, orc_repack_1xL_s8
+ *                          pinned  — the element expression of repackB_1xL<int8_t, L> (fc16m.cpp:80-81) is compiled
+ *                                    from the reference's own bfloat16 class (include/bf16.hpp) in the reference
+ *                                    shim and compared on all 65536 bf16 inputs x several scales (values inside
+ *                                    int8's range: beyond it the reference's conversion is undefined); the tile
+ *                                    order by its index formula on matrices whose entries encode their position.
+ *                                    fc16m.cpp itself needs xbyak (through test_bw.hpp) and cannot be compiled here.
  *   orc_quantize_int4,     spec    — PARITY UNPINNED against the reference, which has no int4 algorithm (it
  *   orc_pack_int4                    only times a byte-copying stand-in): these define what the device code
  *                                    must produce; checked by what the mathematics fixes (|w - q deq| <=
@@ -89,6 +96,10 @@ void orc_gemm_bf16_f64(const uint16_t* A, int64_t lda, const uint16_t* B, int64_
 void orc_gemm_i8(const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb, int transB,
                  int32_t* C, int64_t ldc, int M, int K, int N, int nthreads);
 
+/* the same without the AVX-512BW path (scalar-order check of the fast one) */
+void orc_gemm_i8_generic(const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb, int transB,
+                         int32_t* C, int64_t ldc, int M, int K, int N);
+
 /* ---- epilogue -------------------------------------------------------------------- */
 float orc_gelu(float x);
 void orc_gelu_n(const float* src, float* dst, size_t n);
@@ -120,6 +131,11 @@ float orc_quantize_weights(const uint16_t* W, int64_t ldw, int rows, int cols,
 /* y[M,N] (bf16) = bf16( (x[M,K] bf16 · float(Wq[K,N] int8)) * scale[n] ), fp32 AMX-order
  * accumulation.  Wq is [K,N] (transW=0) or [N,K] (transW=1).  If acc_out != NULL the raw
  * fp32 accumulators are also returned. */
+/* repackB_1xL<int8_t, L> (weight_compression/fc16m.cpp:61-99): q = trunc(bf16_rne(float(w) * scale)) */
+int8_t orc_bf16_scale_trunc_s8(uint16_t w, float scale);
+void orc_quantize_scale_trunc(const uint16_t* W, int64_t ldw, int rows, int cols, float scale, int8_t* Wq, int64_t ldq);
+void orc_repack_1xL_s8(const uint16_t* B, int64_t ldb, int K, int N, int L, float scale, int8_t* out);
+
 /* int4 weight compression (definition of this project; the reference only times a stand-in,
  * weight_compression/wcompress.hpp:90-134) and its packed layout */
 void orc_quantize_int4(const uint16_t* W, int64_t ldw, int K, int N, int transpose, int8_t* q, float* deq);
@@ -129,6 +145,14 @@ void orc_pack_int4(const int8_t* q, int K, int N, uint8_t* out);
 void orc_gemv_w8(const uint16_t* x, int64_t ldx, const int8_t* Wq, int64_t ldw, int transW,
                  const float* scale, uint16_t* y, int64_t ldy, float* acc_out, int M, int K, int N,
                  int nthreads);
+
+/* The same result (bit for bit) computed as the reference computes it: weights packed once in the order of
+ * repackB_1xL<int8_t,2> (orc_pack_1x2_s8: K*N bytes), then streamed and converted in registers, N split over threads
+ * in 32-column groups (weight_compression/fc16m.cpp:61-99, 451-502, 620-663).  K % 32 == 0, N % 32 == 0, M <= 16;
+ * returns -1 for shapes it does not take.  This is the form whose time means something. */
+void orc_pack_1x2_s8(const int8_t* W, int64_t ldw, int K, int N, int8_t* out);
+int orc_gemv_w8_stream(const uint16_t* x, int64_t ldx, const int8_t* Wpacked, const float* scale, uint16_t* y,
+                       int64_t ldy, int M, int K, int N, int nthreads);
 
 /* ---- matrix x vector ------------------------------------------------------------- */
 /* c[M] = A[M,K]·b[K]; bf16 in AMX order (MatmulVector), fp32 out */

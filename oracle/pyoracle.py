@@ -100,6 +100,14 @@ def gemm_i8(A, B, transB=False, nthreads=0):
     return Cm
 
 
+def gemm_i8_generic(A, B, transB=False):
+    M, K = A.shape
+    N = B.shape[0] if transB else B.shape[1]
+    Cm = np.empty((M, N), np.int32)
+    lib().orc_gemm_i8_generic(_p(A), C.c_int64(_ld(A)), _p(B), C.c_int64(_ld(B)), int(transB), _p(Cm), C.c_int64(N), M, K, N)
+    return Cm
+
+
 def gelu(x):
     x = _c(x, np.float32)
     out = np.empty_like(x)
@@ -158,6 +166,25 @@ def quantize_weights(W):
     return Wq, float(dq), float(qs.value)
 
 
+def quantize_scale_trunc(W, scale):
+    """W bf16 bits [rows, cols] -> int8, q = trunc(bf16_rne(w * scale)): repackB_1xL<int8_t> (fc16m.cpp:80-81)."""
+    W = _c(W, np.uint16)
+    Wq = np.empty(W.shape, np.int8)
+    lib().orc_quantize_scale_trunc(_p(W), C.c_int64(W.shape[1]), W.shape[0], W.shape[1], C.c_float(scale), _p(Wq),
+                                   C.c_int64(W.shape[1]))
+    return Wq
+
+
+def repack_1xL_s8(B, L, scale):
+    """B bf16 bits [K, N] -> K*N int8 in the order of repackB_1xL<int8_t, L> (fc16m.cpp:61-99)."""
+    B = _c(B, np.uint16)
+    K, N = B.shape
+    assert K % 32 == 0 and N % (16 * L) == 0
+    out = np.empty(K * N, np.int8)
+    lib().orc_repack_1xL_s8(_p(B), C.c_int64(N), K, N, L, C.c_float(scale), _p(out))
+    return out
+
+
 def quantize_int4(W, transpose=False):
     """W bf16 bits [K,N] (or [N,K] with transpose) -> (q int8 [K,N] in [-7,7], deq fp32 [N])"""
     W = _c(W, np.uint16)
@@ -186,6 +213,28 @@ def gemv_w8(x, Wq, scale, transW=False, nthreads=0, want_acc=False):
     lib().orc_gemv_w8(_p(x), C.c_int64(_ld(x)), _p(Wq), C.c_int64(_ld(Wq)), int(transW), _p(scale), _p(y),
                       C.c_int64(N), _p(acc), M, K, N, nthreads)
     return (y, acc) if want_acc else y
+
+
+def pack_1x2_s8(Wq):
+    """int8 [K, N] -> the stream order of repackB_1xL<int8_t,2> (weight_compression/fc16m.cpp:61-99), K*N bytes."""
+    Wq = _c(Wq, np.int8)
+    K, N = Wq.shape
+    assert K % 32 == 0 and N % 32 == 0
+    out = np.empty(K * N, np.int8)
+    lib().orc_pack_1x2_s8(_p(Wq), C.c_int64(N), K, N, _p(out))
+    return out
+
+
+def gemv_w8_stream(x, Wpacked, scale, N, nthreads=0):
+    """gemv_w8 computed as the reference computes it: packed int8 weights (pack_1x2_s8) read once and converted in
+    registers.  Same bits as gemv_w8; this is the form whose time means something."""
+    M, K = x.shape
+    y = np.empty((M, N), np.uint16)
+    scale = _c(scale, np.float32)
+    rc = lib().orc_gemv_w8_stream(_p(x), C.c_int64(_ld(x)), _p(Wpacked), _p(scale), _p(y), C.c_int64(N), M, K, N, nthreads)
+    if rc != 0:
+        raise ValueError("gemv_w8_stream takes K % 32 == 0, N % 32 == 0 and M <= 16")
+    return y
 
 
 def matvec_bf16(A, b, order="amx"):

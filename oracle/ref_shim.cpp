@@ -241,4 +241,12 @@ long long ref_rcp14_check_all(float (*fn)(float), unsigned* first_bad) {
     return bad;
 }
 
+/* The element expression of repackB_1xL<int8_t, L> (weight_compression/fc16m.cpp:80-81: "*dst++ = src0[n] * scale"
+ * with src0 an ov::bfloat16* and dst an int8_t*), evaluated by the reference's own bfloat16 class.  The function
+ * around it cannot be compiled here (its file needs xbyak); this is the part of it that has arithmetic. */
+void ref_bf16_scale_to_s8(const uint16_t* src, float scale, int8_t* dst, size_t n) {
+    const bfloat16* s = reinterpret_cast<const bfloat16*>(src);
+    for (size_t i = 0; i < n; i++) dst[i] = s[i] * scale;
+}
+
 } // extern "C"

@@ -9,6 +9,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB = os.path.join(ROOT, "mm_amx_amd", "libmm_amx_amd.so")
 HEADER = os.path.join(ROOT, "include", "mm_amx_amd.h")
+BENCH_HEADER = os.path.join(ROOT, "include", "mm_amx_amd_bench.h")
 
 
 @pytest.fixture(scope="module")
@@ -18,8 +19,8 @@ def lib():
     return C.CDLL(LIB)
 
 
-def declared_functions():
-    text = open(HEADER).read()
+def declared_functions(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(mmx_[a-z0-9_]+)\s*\(", text)))
 
@@ -31,13 +32,21 @@ def test_header_declares_the_path():
 
 
 def test_every_declared_symbol_is_exported(lib):
-    for name in declared_functions():
-        assert hasattr(lib, name), f"{name} declared in mm_amx_amd.h but not exported"
+    for header in (HEADER, BENCH_HEADER):
+        for name in declared_functions(header):
+            assert hasattr(lib, name), f"{name} declared in {os.path.basename(header)} but not exported"
 
 
 def test_python_binding_lists_the_same_exports():
     import mm_amx_amd._lib as L
     assert sorted(L.EXPORTS) == declared_functions()
+    assert sorted(L.BENCH_EXPORTS) == declared_functions(BENCH_HEADER)
+
+
+def test_measurement_aids_are_not_part_of_the_operator_header():
+    """Timing and probe entry points live in mm_amx_amd_bench.h; the operator ABI declares none of them."""
+    ops = declared_functions()
+    assert not [n for n in ops if "probe" in n or "time" in n]
 
 
 def test_sizes_and_argument_validation(lib):

@@ -564,6 +564,32 @@ def test_weight_compressed_matmul(po, M):
     assert np.array_equal(host_bits(Wq_gpu), Wq)
 
 
+@pytest.mark.parametrize("scale", [2.0, 0.7, 37.0])
+def test_scaled_truncating_quantiser(po, scale):
+    """mmx_quantize_weights_scaled = the quantising half of repackB_1xL<int8_t> (weight_compression/fc16m.cpp:80-81):
+    bit-exact against the oracle (itself pinned to the reference's bfloat16 class), including a strided source, the
+    saturating cases and NaN; then fc16m's own use: int8 weights made with quantize_i8_scale, per-tensor dequant
+    1 / scale after the K loop (:280, :444), through the decode kernel."""
+    rng = np.random.default_rng(int(scale * 10))
+    K, N = 512, 192
+    Wf = rng.uniform(-3.4, 3.4, (K, N + 8)).astype(np.float32)
+    Wf[0, :6] = [np.nan, 1e30, -1e30, 127.4 / scale, -128.6 / scale, 0.0]
+    W = wl.f32_to_bf16_bits(Wf)
+    W[0, 0] = 0x7FC0
+    want = po.quantize_scale_trunc(np.ascontiguousarray(W[:, :N]), scale)
+    Wd = dev_bf16(W)[:, :N]                                   # row stride of N + 8 elements
+    got = mx.quantize_weights_scaled(Wd, scale)
+    assert np.array_equal(host_bits(got), want)
+    for M in (1, 16):
+        x = rand_bf16(rng, (M, K), 1.0)
+        y_ref, _ = po.gemv_w8(x, want, np.full(N, np.float32(1.0) / np.float32(scale), np.float32), want_acc=True)
+        y = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+        mx.gemm(dev_bf16(x), mx.repack_b(got), N, mx.Epilogue(y, mx.PP_DEQUANT, deq_scale=float(np.float32(1.0) / np.float32(scale))),
+                b_dtype=mx.I8)
+        assert "skinny" in mx.last_kernel()
+        check_float_parity(bf16_to_f32(host_bits(y)), bf16_to_f32(y_ref), f"fc16m int8 weights M={M}")
+
+
 def _w8_case(po, M, K, N, seed, steps=None, **gemm_kw):
     """bf16 x int8-weight GEMM against the bf16 GEMM of the oracle on the (exactly representable) integers."""
     rng = np.random.default_rng(seed)
@@ -714,7 +740,7 @@ def _mlp_case(po, M, K, N, seed):
     e3 = np.linalg.norm(yf - rf) / np.linalg.norm(rf)
     print(f"mlp M={M}: h rel={e1:.2e} ({f1 * 100:.3f}% <=1ulp)  y|h rel={e2:.2e} ({f2 * 100:.3f}%)  end-to-end rel={e3:.2e}  "
           f"kernels={k_fused}, {k_down}")
-    assert e3 < 3e-3
+    assert e3 < 1e-3  # the stated bar (measured: 5.5e-5 at M = 1, 3.4e-4 at M = 256)
     return k_fused, k_down
 
 

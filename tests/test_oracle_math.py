@@ -212,3 +212,101 @@ def test_int4_non_finite_weights_are_defined(po):
     assert not q[:, 1].any() and np.isinf(deq[1])
     assert not q[:, 2].any() and deq[2] == 0.0
     assert list(q[:, 3]) == [7] * 8
+
+
+def test_ffn_up_gelu_against_a_better_rounded_sum_shows_the_same_shortfall(po):
+    """The 1-bf16-ulp bar on the FC + BIAS + GELU configuration (K = 4096, A ~ N(0,1), B ~ N(0,0.02), bias ~ N(0,0.1)),
+    measured between the reference's own arithmetic (AMX summation order, fp32) and the same product accumulated
+    in fp64 and rounded once: over ALL elements even this pair stays below 99.9 %, above a pre-activation of -3.5
+    it is met with room to spare.  So 99.9 % over all elements is not reachable by any implementation whose fp32
+    accumulators are not bit-identical to AMX's; the GPU tests therefore apply the bar where GELU is well
+    conditioned and check the fused epilogue bit for bit on the GPU's own accumulators."""
+    from mm_amx_amd import workloads as wl
+    w = wl.ffn_up_bias_gelu(M=192)  # 192 x 11008 = 2.1 M elements of the benchmark's own distribution
+    acc = po.gemm_bf16(w["A"], w["B"])
+    acc64 = po.gemm_bf16(w["A"], w["B"], f64=True)
+    steps = po.PP_BIAS | po.PP_GELU
+    a = po.bf16_to_f32(po.pp(acc, steps, po.BF16, bias=w["bias"])).astype(np.float64)
+    b = po.bf16_to_f32(po.pp(acc64, steps, po.BF16, bias=w["bias"])).astype(np.float64)
+    ulp = np.exp2(np.floor(np.log2(np.maximum(np.abs(a), 2.0 ** -126))) - 7)
+    within = np.abs(a - b) <= ulp
+    pre = acc + w["bias"][None, :]
+    good = pre > -3.5
+    assert a.size >= 2_000_000
+    assert within.mean() < 0.999, within.mean()            # measured 0.99886
+    assert within.mean() > 0.998
+    assert within[good].mean() >= 0.9999, within[good].mean()  # measured 0.999994
+    # the accumulators themselves agree far better than the bar asks: the shortfall is GELU's conditioning, not the sums
+    ulp_acc = np.exp2(np.floor(np.log2(np.maximum(np.abs(acc.astype(np.float64)), 2.0 ** -126))) - 7)
+    assert (np.abs(acc.astype(np.float64) - acc64) <= ulp_acc).mean() > 0.9999
+
+
+def test_scaled_truncating_quantiser_by_hand_and_by_brute_force(po):
+    """q = trunc(bf16_rne(w * scale)) (repackB_1xL<int8_t>, weight_compression/fc16m.cpp:80-81): answers worked out by
+    hand (the bf16 rounding of the product comes BEFORE the truncation and can carry a value across an integer),
+    an independent numpy restatement on random inputs, and the function's tile order by its index formula."""
+    def q1(x, scale):
+        return int(po.quantize_scale_trunc(po.f32_to_bf16(np.array([[x]], np.float32)), scale)[0, 0])
+    assert q1(1.296875, 2.0) == 2 and q1(-1.296875, 2.0) == -2          # 2.59375 -> toward zero
+    assert q1(0.99609375, 1.0) == 0 and q1(-0.99609375, 1.0) == 0       # just below one
+    assert q1(1.0, 1.0) == 1 and q1(63.5, 2.0) == 127 and q1(-64.0, 2.0) == -128
+    # 0.33203125 * 3 = 0.99609375 exactly (a bf16): 0; 1.9921875 * (1/3 in fp32) = 0.66406256 -> bf16 0.6640625 -> 0
+    assert q1(0.33203125, 3.0) == 0
+    # the product 85 * 1.0117188 = 85.996098 rounds to bf16 86.0 BEFORE the truncation: 86, where trunc(product) is 85
+    assert q1(85.0, 1.01171875) == 86
+    assert q1(100.0, 2.0) == 127 and q1(-100.0, 2.0) == -128 and q1(float("nan"), 2.0) == 0  # defined here: saturate, NaN -> 0
+    rng = np.random.default_rng(3)
+    W = po.f32_to_bf16(rng.uniform(-60, 60, (64, 48)).astype(np.float32))
+    for scale in (2.0, 0.7, 1.9):
+        prod = po.bf16_to_f32(W) * np.float32(scale)                     # fp32 product, correctly rounded
+        rb = po.bf16_to_f32(po.f32_to_bf16(prod))                        # ... to bf16, nearest even
+        want = np.clip(np.trunc(rb), -128, 127).astype(np.int8)
+        assert np.array_equal(po.quantize_scale_trunc(W, scale), want)
+    # tile order (fc16m.cpp:61-99): with scale 1 and small integer entries the bytes are the entries themselves
+    K, N, L = 64, 64, 2
+    k_idx, n_idx = np.meshgrid(np.arange(K), np.arange(N), indexing="ij")
+    for plane, vals in (("k", k_idx), ("n", n_idx)):
+        out = po.repack_1xL_s8(po.f32_to_bf16(vals.astype(np.float32)), L, 1.0)
+        i = 0
+        for n0 in range(0, N, 16 * L):
+            for k0 in range(0, K, 32):
+                for l in range(L):
+                    tile = out[i:i + 512].reshape(16, 16, 2)             # [k pair][column][k parity]
+                    i += 512
+                    kk = k0 + 2 * np.arange(16)[:, None, None] + np.arange(2)[None, None, :]
+                    nn = n0 + 16 * l + np.arange(16)[None, :, None]
+                    want = np.broadcast_to(kk if plane == "k" else nn, (16, 16, 2))
+                    assert np.array_equal(tile, want.astype(np.int8))
+
+
+def test_streamed_gemv_is_the_converted_gemv_bit_for_bit(po):
+    """orc_gemv_w8_stream (packed int8 weights read once, converted in registers: the form of matmul16m_Wint8B,
+    weight_compression/fc16m.cpp:451-502) against orc_gemv_w8 (weights converted to bf16 up front, then the pinned AMX-order
+    GEMM): same bits for every M it takes, any thread count; and its packing is the order of repackB_1xL<int8_t,2>."""
+    from mm_amx_amd import workloads as wl
+    for M, K, N in ((1, 256, 96), (4, 512, 64), (7, 96, 160), (16, 1024, 32)):
+        w = wl.decode_gemv_w8(M=M, K=K, N=N, seed=M)
+        want = po.gemv_w8(w["x"], w["W"], w["scale"])
+        packed = po.pack_1x2_s8(w["W"])
+        for nt in (1, 3):
+            assert np.array_equal(po.gemv_w8_stream(w["x"], packed, w["scale"], N, nthreads=nt), want), (M, K, N, nt)
+    rng = np.random.default_rng(0)
+    Wi = rng.integers(-100, 100, (64, 96)).astype(np.int8)
+    assert np.array_equal(po.pack_1x2_s8(Wi), po.repack_1xL_s8(po.f32_to_bf16(Wi.astype(np.float32)), 2, 1.0))
+
+
+def test_int8_gemm_fast_path_equals_the_generic_one_and_int64(po):
+    """orc_gemm_i8 takes a vpmaddwd path where the host has AVX-512BW (even K): the same int32 sums as the generic
+    loop and as an int64 product, including the extremes -128 x -128."""
+    rng = np.random.default_rng(1)
+    for M, K, N, t in ((37, 130, 75, False), (5, 64, 33, True), (64, 256, 48, False), (3, 65, 20, False)):
+        A = rng.integers(-128, 128, (M, K)).astype(np.int8)
+        B = rng.integers(-128, 128, ((N, K) if t else (K, N))).astype(np.int8)
+        A[0, :] = -128
+        if t:
+            B[0, :] = -128
+        else:
+            B[:, 0] = -128
+        want = A.astype(np.int64) @ (B.T if t else B).astype(np.int64)
+        assert np.array_equal(po.gemm_i8(A, B, transB=t), want)
+        assert np.array_equal(po.gemm_i8_generic(A, B, transB=t), want)

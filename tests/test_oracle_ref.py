@@ -142,3 +142,19 @@ def test_silu_is_the_stated_composition(po, ref):
     ref.ref_rcp14(p(one_plus), p(r14), one_plus.size)
     want = (g * r14).astype(np.float32)
     assert np.array_equal(bits(po.silu(g)), bits(want))
+
+
+def test_scaled_truncating_quantiser_is_the_reference_expression(po, ref):
+    """repackB_1xL<int8_t, L> (weight_compression/fc16m.cpp:80-81): "*dst++ = src0[n] * scale" evaluated by the
+    reference's own bfloat16 class (compiled in the shim) on every bf16 input and a set of scales, against the
+    oracle's trunc(bf16_rne(w * scale)).  Compared where the conversion to int8 is defined (|value| < 127.5)."""
+    allb = np.arange(65536, dtype=np.uint16)
+    for scale in (1.0, 2.0, 0.5, 3.0, 127.0 / 3.3, 0.37, -2.0, 1e-3, 1.0 / 3.0):
+        want = np.empty(65536, np.int8)
+        ref.ref_bf16_scale_to_s8(p(allb), C.c_float(scale), p(want), C.c_size_t(65536))
+        got = po.quantize_scale_trunc(allb.reshape(256, 256), scale).reshape(-1)
+        with np.errstate(invalid="ignore", over="ignore"):
+            v = po.bf16_to_f32(allb).astype(np.float64) * np.float64(np.float32(scale))
+        defined = np.isfinite(v) & (np.abs(v) < 127.5)
+        assert defined.sum() > 30000
+        assert np.array_equal(got[defined], want[defined]), scale
