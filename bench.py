@@ -760,6 +760,17 @@ def main():
         out["extra"] = extra
     elif cpu_other:
         out["extra"] = {"cpu_baselines": cpu_other}
+    # Which CPU figure stands as the baseline of a configuration: the faster of the two.  The port restates the
+    # reference's arithmetic (it is the parity oracle: AMX summation order in fp32 / integer FMAs, no VNNI, no bf16 dot
+    # products) and is the reference's own algorithm only for the decode GEMV (packed int8 weights streamed and converted in
+    # registers); torch's CPU matmul is the oneDNN path the reference compares itself with (benchmark/mmbench/dnnl.cpp).
+    def of_record(ent):
+        vals = {k: v.get("value") for k, v in ent.items() if isinstance(v, dict) and v.get("value") is not None}
+        return max(vals, key=vals.get) if vals else None
+    if "cpu_baseline" in out:
+        out["cpu_baseline"]["baseline_of_record"] = "onednn" if out["cpu_baseline"]["onednn"]["value"] > out["cpu_baseline"]["value"] else "port"
+    for ent in cpu_other.values():
+        ent["baseline_of_record"] = of_record(ent)
 
     print(json.dumps(out))
 

@@ -22,7 +22,8 @@ extern "C" {
 #endif
 
 /* element types */
-enum { MMX_F32 = 0, MMX_BF16 = 1, MMX_I8 = 2, MMX_I32 = 3, MMX_I4 = 4 /* packed weights only */ };
+enum { MMX_F32 = 0, MMX_BF16 = 1, MMX_I8 = 2, MMX_I32 = 3, MMX_I4 = 4 /* packed weights only */,
+       MMX_U8 = 5 /* unsigned bytes: mmx_repack_b, mmx_gemm_u8, mmx_matvec_u8 only */ };
 
 /* error codes */
 enum {
@@ -89,7 +90,9 @@ int mmx_init(int device);
  * row stride ldb_bytes, dtype MMX_BF16 or MMX_I8.  The result is in MFMA-fragment order:
  *     packed[panel = n/32][kstep = k/KS][lane 0..63][16 bytes],  KS = 16 (bf16) / 32 (int8),
  *     lane = n%32 + 32*((k%KS)/(KS/2)),  byte offset in the lane = (k%(KS/2))*sizeof(T),
- * zero padded in K up to a multiple of 128 bytes per column and in N up to a multiple of 32. */
+ * zero padded in K up to a multiple of 128 bytes per column and in N up to a multiple of 32.
+ * dtype MMX_U8 (unsigned weights, for mmx_gemm_u8): the int8 layout holding u - 128, i.e. every byte with its sign
+ * bit inverted (the padding stays zero). */
 size_t mmx_packed_b_bytes(int dtype, int K, int N);
 int mmx_repack_b(int dtype, const void* B, int64_t ldb_bytes, int K, int N, int transpose, void* packed,
                  void* stream);
@@ -170,7 +173,10 @@ int mmx_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const v
 int mmx_gemm_splitk(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* Bpacked, int M, int K,
                     int N, int n0, int n1, const mmx_epilogue* ep, int k_splits, void* workspace,
                     size_t workspace_bytes, void* stream);
-/* Workspace the call above would use for this shape (0 if it would not split).  steps = the post-op steps. */
+/* Workspace the call above would use for this shape (0 if it would not split).  steps = the post-op steps.  For decode
+ * shapes (M <= 32) the figure is an upper bound: it looks at the number of panels and the length of K only, and a launch
+ * whose x fits in LDS, or whose K or alignment takes another kernel, does not split after all.  The answer depends on the
+ * device's CU count: call mmx_init first. */
 size_t mmx_gemm_workspace_bytes(int a_dtype, int b_dtype, int M, int K, int N, int n0, int n1, uint32_t steps,
                                 int k_splits);
 
@@ -189,6 +195,25 @@ int mmx_gemm_splitk_static(int a_dtype, int b_dtype, const void* A, int64_t lda_
 /* ---- c[M] = A[M, K] · b[K]: amx_kernel::MatmulVector::operator() (include/kernels_amx.hpp:959)
  * and amx_kernel::GemAvB::operator() (:1534).  dtype MMX_BF16 (c fp32) or MMX_I8 (c int32). */
 int mmx_matvec(int dtype, const void* A, int64_t lda_bytes, const void* b, void* c, int M, int K, void* stream);
+
+/* ---- the unsigned 8-bit forms: amx_kernel::Matmul<uint8_t|int8_t, uint8_t|int8_t> (tdpbusd / tdpbsud / tdpbuud,
+ * include/kernels_amx.hpp:1057-1101, accumulator int32 :825) and amx_kernel::MatmulVector in the same forms
+ * (:839-850).  a_dtype / b_dtype are MMX_I8 or MMX_U8, at least one of them MMX_U8.  (In the reference only
+ * Matmul<uint8_t, int8_t> can be instantiated - its repackB_1x2 has no uint8_t form, :293, :393, :810 - and all three
+ * MatmulVector forms; here all combinations exist.)  The matrix cores multiply signed bytes, so an unsigned operand
+ * u is computed as (u - 128) + 128: Bpacked comes from mmx_repack_b with the dtype of B (MMX_U8 stores u - 128), A is
+ * shifted per call, the signed product runs through the int8 kernels of mmx_gemm into int32 scratch, and a last pass
+ * adds 128 x the column sums of the weights / row sums of the activations (+ 16384 K when both are unsigned), in
+ * int32 arithmetic modulo 2^32 like the AMX accumulators, and applies the post-op `ep` (as for mmx_gemm on int8
+ * inputs; MMX_I32 output = the raw sums).  Exact; three launches more than mmx_gemm.
+ * scratch: device memory, 256-byte aligned, mmx_gemm_u8_scratch_bytes() bytes, free to reuse once the call's work on
+ * `stream` has finished (0 from the query = arguments it does not take). */
+size_t mmx_gemm_u8_scratch_bytes(int a_dtype, int b_dtype, int M, int K, int N, int n0, int n1);
+int mmx_gemm_u8(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* Bpacked, int M, int K, int N,
+                int n0, int n1, const mmx_epilogue* ep, void* scratch, size_t scratch_bytes, void* stream);
+/* c[M] (int32) = A[M, K] . b[K] with A and b each signed or unsigned bytes (at least one MMX_U8). */
+int mmx_matvec_u8(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* b, void* c, int M, int K,
+                  void* stream);
 
 /* ---- fused Llama MLP: AMX_MLP::MLP::run (tests/amx-mlp.cpp:778-783) ---------------------------
  * x [M, K] bf16; w_gate_up from mmx_repack_gate_up (K x 2N); w_down from mmx_repack_b of the

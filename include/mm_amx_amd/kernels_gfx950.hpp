@@ -62,10 +62,12 @@ template <> struct dtype_of<float> { static constexpr int value = MMX_F32; };
 template <> struct dtype_of<bfloat16> { static constexpr int value = MMX_BF16; };
 template <> struct dtype_of<int8_t> { static constexpr int value = MMX_I8; };
 template <> struct dtype_of<int32_t> { static constexpr int value = MMX_I32; };
+template <> struct dtype_of<uint8_t> { static constexpr int value = MMX_U8; };
 
 // accumulator type of an input type (include/kernels_amx.hpp:818-828)
 template <typename T> struct acc_type { typedef float type; };
 template <> struct acc_type<int8_t> { typedef int32_t type; };
+template <> struct acc_type<uint8_t> { typedef int32_t type; };  // (:825)
 
 // ---- tensor2D<T> (include/tensor2D.hpp:30-329), resident in HBM -----------------------------------
 // dims = {rows, cols}; stride is in BYTES; rows are padded to 64 bytes unless force_compact;
@@ -358,9 +360,16 @@ struct Matmul {
     // 0 = the library chooses, 1 = never, 2 = the reference's two halves, up to 4
     int k_splits = 0;
 
-    static_assert(std::is_same<TA, TB>::value, "Matmul<TA,TB>: TA == TB except for the <bfloat16,int8_t,float> form");
-    constexpr static bool is_i8_mode = std::is_same<TA, int8_t>::value;
+    // is_s8u8 / is_u8s8 / is_u8u8 (include/kernels_amx.hpp:1057-1061): at least one operand of unsigned bytes
+    constexpr static bool is_u8_mode = (std::is_same<TA, uint8_t>::value || std::is_same<TB, uint8_t>::value) &&
+                                       (std::is_same<TA, uint8_t>::value || std::is_same<TA, int8_t>::value) &&
+                                       (std::is_same<TB, uint8_t>::value || std::is_same<TB, int8_t>::value);
+    static_assert(std::is_same<TA, TB>::value || is_u8_mode,
+                  "Matmul<TA,TB>: TA == TB except for the <bfloat16,int8_t,float> form and the unsigned byte forms");
+    constexpr static bool is_i8_mode = std::is_same<TA, int8_t>::value || is_u8_mode;
     constexpr static int kStep = is_i8_mode ? 64 : 32;
+    std::shared_ptr<void> u8_scratch;  // unsigned forms: the shifted activations, correction terms and int32 sums of a call
+    size_t u8_scratch_bytes = 0;
 
     Matmul(bool constB = false, bool transposeB = false) : constB(constB), transposeB(transposeB) {}
 
@@ -378,6 +387,20 @@ struct Matmul {
         require(ppkernel.out_rows() >= M && ppkernel.out_cols() >= n1, "Matmul: C is smaller than M x n1");
         if (!constB || !internalB) internalB = repackB_1x2(matB, transposeB, stream);
         const mmx_epilogue e = ppkernel.descriptor();
+        if (is_u8_mode) {  // tdpbusd / tdpbsud / tdpbuud: mmx_gemm_u8 (three passes, exact)
+            const size_t need = mmx_gemm_u8_scratch_bytes(dtype_of<TA>::value, dtype_of<TB>::value, M, K, N, n0, n1);
+            if (need > u8_scratch_bytes) {
+                void* p = nullptr;
+                check_hip(hipStreamSynchronize(stream), "Matmul: hipStreamSynchronize");  // an earlier call may still use the old one
+                check_hip(hipMalloc(&p, need), "Matmul: hipMalloc(u8 scratch)");
+                u8_scratch = std::shared_ptr<void>(p, [](void* q) { (void)hipFree(q); });
+                u8_scratch_bytes = need;
+            }
+            check(mmx_gemm_u8(dtype_of<TA>::value, dtype_of<TB>::value, matA.data, matA.stride, internalB.data, M, K, N, n0, n1, &e,
+                              u8_scratch.get(), u8_scratch_bytes, stream),
+                  "Matmul (unsigned bytes)");
+            return;
+        }
         // (decode launches, M <= 32, choose their own slices: they take the workspace with k_splits = 0 only)
         const Workspace ws = (k_splits == 1 || (M <= 32 && k_splits != 0))
                                  ? Workspace()
@@ -488,12 +511,20 @@ struct MatmulW4 {
 // takes any K >= 1, the same bounds are not enforced.
 template <typename TA, typename TB, typename TC = typename acc_type<TA>::type>
 struct MatmulVector {
-    static_assert(std::is_same<TA, TB>::value, "MatmulVector: TA == TB");
-    constexpr static int kStep = std::is_same<TA, int8_t>::value ? 64 : 32;
+    // is_s8u8 / is_u8s8 / is_u8u8 (include/kernels_amx.hpp:839-850)
+    constexpr static bool is_u8_mode = (std::is_same<TA, uint8_t>::value || std::is_same<TB, uint8_t>::value) &&
+                                       (std::is_same<TA, uint8_t>::value || std::is_same<TA, int8_t>::value) &&
+                                       (std::is_same<TB, uint8_t>::value || std::is_same<TB, int8_t>::value);
+    static_assert(std::is_same<TA, TB>::value || is_u8_mode, "MatmulVector: TA == TB, or bytes of either sign");
+    constexpr static int kStep = (std::is_same<TA, int8_t>::value || is_u8_mode) ? 64 : 32;
     MatmulVector() {}
     void operator()(tensor2D<TA>& matA, const TB* vB, TC* vC, hipStream_t stream = nullptr) {
-        check(mmx_matvec(dtype_of<TA>::value, matA.data, matA.stride, vB, vC, matA.dims[0], matA.dims[1], stream),
-              "MatmulVector");
+        if (is_u8_mode)
+            check(mmx_matvec_u8(dtype_of<TA>::value, dtype_of<TB>::value, matA.data, matA.stride, vB, vC, matA.dims[0], matA.dims[1], stream),
+                  "MatmulVector (unsigned bytes)");
+        else
+            check(mmx_matvec(dtype_of<TA>::value, matA.data, matA.stride, vB, vC, matA.dims[0], matA.dims[1], stream),
+                  "MatmulVector");
     }
 };
 

@@ -29,12 +29,15 @@ int mmx_time_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, co
  * scratch: 16 KiB of device memory.  Blocks until the loop has finished; not thread-safe. */
 int mmx_probe_mfma(int dtype, int random_operands, int iters, void* scratch, void* stream, float* rate_out, float* mhz_out);
 
-/* A kernel that does nothing but read: `workgroups` resident workgroups of eight wavefronts walk `bytes` bytes
- * (a multiple of 8 KiB) at `buf` in equal contiguous shares, every wavefront keeping kib_in_flight (8, 16 or 32)
- * KiB of nontemporal 16-byte loads outstanding as a rolling window.  What it takes is what a decode kernel
- * streaming the same number of weight bytes cannot beat.  sink: 4 bytes of device memory (never written in
- * practice; it keeps the loads alive).  Asynchronous on `stream`, allocates nothing, may be captured into a graph. */
-int mmx_probe_read(const void* buf, size_t bytes, int workgroups, int kib_in_flight, void* sink, void* stream);
+/* A kernel that does nothing but read: `workgroups` resident workgroups of waves_per_workgroup (4 or 8) wavefronts walk
+ * `bytes` bytes at `buf` in equal contiguous shares (bytes must divide into shares of whole waves_per_workgroup KiB),
+ * every wavefront keeping kib_in_flight (2, 4, 8, 16 or 32) KiB of nontemporal 16-byte loads outstanding as a rolling
+ * window; blocked = 1 gives each wavefront a contiguous run of its workgroup's share (the pattern of the decode
+ * kernels), 0 lets the wavefronts of a workgroup go side by side through it.  What the best of these takes is what a
+ * decode kernel streaming the same number of weight bytes cannot beat.  sink: 4 bytes of device memory (never written
+ * in practice; it keeps the loads alive).  Asynchronous on `stream`, allocates nothing, may be captured into a graph. */
+int mmx_probe_read(const void* buf, size_t bytes, int workgroups, int waves_per_workgroup, int blocked, int kib_in_flight,
+                   void* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -8,7 +8,7 @@ import os
 
 import torch
 
-F32, BF16, I8, I32, I4 = 0, 1, 2, 3, 4
+F32, BF16, I8, I32, I4, U8 = 0, 1, 2, 3, 4, 5
 PP_NONE, PP_DEQUANT, PP_BIAS, PP_GELU, PP_QUANT, PP_SILU_GATE = 0, 1, 2, 4, 8, 16
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -17,7 +17,7 @@ _LIB_PATH = os.environ.get("MMX_LIB_PATH") or os.path.join(_HERE, "libmm_amx_amd
 
 EXPORTS = ["mmx_last_error", "mmx_init", "mmx_packed_b_bytes", "mmx_repack_b", "mmx_repack_gate_up",
            "mmx_quantize_weights", "mmx_quantize_weights_scaled", "mmx_quantize_pack_int4", "mmx_dequant_packed", "mmx_gemm", "mmx_gemm_splitk",
-           "mmx_gemm_splitk_static", "mmx_gemm_workspace_bytes", "mmx_matvec", "mmx_mlp", "mmx_mlp_splitk", "mmx_set_tile",
+           "mmx_gemm_splitk_static", "mmx_gemm_workspace_bytes", "mmx_gemm_u8_scratch_bytes", "mmx_gemm_u8", "mmx_matvec_u8", "mmx_matvec", "mmx_mlp", "mmx_mlp_splitk", "mmx_set_tile",
            "mmx_set_option", "mmx_last_kernel"]
 # measurement aids (include/mm_amx_amd_bench.h)
 BENCH_EXPORTS = ["mmx_time_gemm", "mmx_probe_mfma", "mmx_probe_read"]
@@ -74,6 +74,11 @@ def lib():
                                              C.c_int, C.c_int, C.POINTER(_Epilogue), C.c_int, C.c_void_p]
         l.mmx_gemm_workspace_bytes.restype = C.c_size_t
         l.mmx_gemm_workspace_bytes.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_uint32, C.c_int]
+        l.mmx_gemm_u8_scratch_bytes.restype = C.c_size_t
+        l.mmx_gemm_u8_scratch_bytes.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+        l.mmx_gemm_u8.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+                                  C.POINTER(_Epilogue), C.c_void_p, C.c_size_t, C.c_void_p]
+        l.mmx_matvec_u8.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
         l.mmx_mlp_splitk.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p,
                                      C.c_int64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]
         l.mmx_matvec.argtypes = [C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
@@ -86,7 +91,7 @@ def lib():
                                     C.c_void_p, C.c_int, C.POINTER(C.c_float)]
         l.mmx_probe_mfma.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.POINTER(C.c_float),
                                      C.POINTER(C.c_float)]
-        l.mmx_probe_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+        l.mmx_probe_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
         _lib = l
     return _lib
 
@@ -113,7 +118,7 @@ def _dev(t, what):
     return t
 
 
-_DT = {torch.float32: F32, torch.bfloat16: BF16, torch.int8: I8, torch.int32: I32}
+_DT = {torch.float32: F32, torch.bfloat16: BF16, torch.int8: I8, torch.int32: I32, torch.uint8: U8}
 
 
 def dtype_code(t):
@@ -157,9 +162,12 @@ def packed_b_bytes(dtype, K, N):
 
 
 def repack_b(B, transpose=False):
-    """B [K,N] (or [N,K] with transpose) bf16/int8 on the GPU -> packed weights (uint8 tensor)."""
+    """B [K,N] (or [N,K] with transpose) bf16/int8/uint8 on the GPU -> packed weights (uint8 tensor).  uint8 weights
+    (for gemm_u8) are stored as u - 128 in the int8 layout."""
     _dev(B, "B")
     dt = dtype_code(B)
+    if dt not in (BF16, I8, U8):
+        raise MmxError("B must be bf16, int8 or uint8")
     K, N = (B.shape[1], B.shape[0]) if transpose else B.shape
     out = torch.empty(packed_b_bytes(dt, K, N), dtype=torch.uint8, device=B.device)
     _check(lib().mmx_repack_b(dt, B.data_ptr(), _row_stride_bytes(B), K, N, int(transpose), out.data_ptr(), _stream()))
@@ -291,7 +299,7 @@ def _packed_bytes_host(dtype, K, N):
         return 0
     if dtype == I4:
         return ((N + 31) // 32) * ((K + 255) // 256 * 4) * 1024
-    es = {BF16: 2, I8: 1}.get(dtype, 0)
+    es = {BF16: 2, I8: 1, U8: 1}.get(dtype, 0)
     return ((N + 31) // 32) * 32 * ((K * es + 127) // 128 * 128)
 
 
@@ -343,6 +351,51 @@ def gemm_static(A, Bpacked, N, ep, b_dtype=None, n0=0, n1=None, k_splits=0):
                                         C.byref(s), k_splits, _stream()))
 
 
+def gemm_u8(A, Bpacked, N, ep, b_unsigned, n0=0, n1=None, scratch=None):
+    """The int8 GEMM with unsigned bytes in A (a uint8 tensor) and/or in the weights (b_unsigned: Bpacked comes from
+    repack_b of a uint8 matrix): mmx_gemm_u8.  scratch: a uint8 tensor of gemm_u8_scratch_bytes() bytes (made here if
+    not given)."""
+    n1 = N if n1 is None else n1
+    _is_2d(A, "A")
+    if A.dtype not in (torch.int8, torch.uint8):
+        raise MmxError("A must be int8 or uint8")
+    a_dt, b_dt = dtype_code(A), (U8 if b_unsigned else I8)
+    if a_dt != U8 and b_dt != U8:
+        raise MmxError("gemm_u8 is for unsigned operands: use gemm for int8 x int8")
+    M, K = A.shape
+    view = A.view(torch.int8) if A.dtype == torch.uint8 else A
+    _check_gemm_args(view, Bpacked, N, ep, I8, n0, n1)
+    _dev(A, "A"), _dev(Bpacked, "Bpacked")
+    need = lib().mmx_gemm_u8_scratch_bytes(a_dt, b_dt, M, K, N, n0, n1)
+    if scratch is None:
+        scratch = torch.empty(need, dtype=torch.uint8, device=A.device)
+    if scratch.dtype != torch.uint8 or not scratch.is_cuda or not scratch.is_contiguous() or scratch.numel() < need:
+        raise MmxError(f"scratch must be a contiguous uint8 tensor of at least {need} bytes on the GPU")
+    s = ep.struct()
+    _check(lib().mmx_gemm_u8(a_dt, b_dt, A.data_ptr(), _row_stride_bytes(A), Bpacked.data_ptr(), M, K, N, n0, n1, C.byref(s),
+                             scratch.data_ptr(), scratch.numel(), _stream()))
+
+
+def matvec_u8(A, b, out=None):
+    """c[M] (int32) = A[M,K] . b[K], A and b each int8 or uint8, at least one uint8 (mmx_matvec_u8)."""
+    _is_2d(A, "A")
+    M, K = A.shape
+    if A.dtype not in (torch.int8, torch.uint8) or not isinstance(b, torch.Tensor) or b.dtype not in (torch.int8, torch.uint8):
+        raise MmxError("A and b must be int8 or uint8")
+    if A.dtype != torch.uint8 and b.dtype != torch.uint8:
+        raise MmxError("matvec_u8 is for unsigned operands: use matvec for int8 x int8")
+    if b.numel() != K or not b.is_contiguous():
+        raise MmxError(f"b must be a contiguous vector of K = {K} elements")
+    if out is not None and (out.dtype != torch.int32 or out.numel() < M or not out.is_contiguous()):
+        raise MmxError(f"out must be a contiguous int32 vector of at least M = {M} elements")
+    _dev(A, "A"), _dev(b, "b")
+    if out is None:
+        out = torch.empty(M, dtype=torch.int32, device=A.device)
+    _check(lib().mmx_matvec_u8(dtype_code(A), dtype_code(b), A.data_ptr(), _row_stride_bytes(A), b.data_ptr(), out.data_ptr(), M, K,
+                               _stream()))
+    return out
+
+
 def gemm_workspace_bytes(a_dtype, b_dtype, M, K, N, steps=PP_NONE, k_splits=0, n0=0, n1=None):
     return lib().mmx_gemm_workspace_bytes(a_dtype, b_dtype, M, K, N, n0, N if n1 is None else n1, int(steps), k_splits)
 
@@ -373,9 +426,10 @@ def probe_mfma(dtype, random_operands, iters=20000):
     return rate.value, mhz.value
 
 
-def probe_read(buf, workgroups, kib_in_flight, sink):
+def probe_read(buf, workgroups, kib_in_flight, sink, waves=8, blocked=False):
     """One launch of the read-only kernel over the uint8 tensor `buf` (asynchronous; see mm_amx_amd_bench.h)."""
-    _check(lib().mmx_probe_read(buf.data_ptr(), buf.numel(), int(workgroups), int(kib_in_flight), sink.data_ptr(), _stream()))
+    _check(lib().mmx_probe_read(buf.data_ptr(), buf.numel(), int(workgroups), int(waves), int(bool(blocked)), int(kib_in_flight),
+                                sink.data_ptr(), _stream()))
 
 
 def matvec(A, b, out=None):

@@ -73,7 +73,13 @@ size_t plan_workspace_bytes(int elesz, bool w8, int M, int K, int Ncols, uint32_
 bool skinny_i8_eligible(const void* x, int64_t ldx, int M, int K);
 int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int K, int N, int n0, int n1,
                   const Epilogue& ep, hipStream_t st, const SplitRequest* rq);
-int launch_repack(int elesz, const void* B, int64_t ldb, int K, int N, int transpose, void* out, hipStream_t st);
+int launch_repack(int elesz, const void* B, int64_t ldb, int K, int N, int transpose, void* out, hipStream_t st, int flip);
+size_t u8_scratch_bytes(bool a_unsigned, int M, int K, int n1);
+int launch_gemm_x8(bool a_unsigned, bool b_unsigned, const void* A, int64_t lda, const void* Bp, int M, int K, int N, int n0, int n1,
+                   const Epilogue& ep, char* scratch, hipStream_t st,
+                   int (*signed_gemm)(const void* A, int64_t lda, const void* Bp, int M, int K, int N, int n0, int n1, int32_t* acc,
+                                      int64_t ldacc_bytes, hipStream_t st));
+int launch_matvec_x8(bool a_unsigned, bool b_unsigned, const void* A, int64_t lda, const void* b, void* c, int M, int K, hipStream_t st);
 int launch_repack_gate_up(const void* wg, const void* wu, int64_t ldw, int K, int N, void* out, hipStream_t st);
 int launch_quantize(const void* W, int64_t ldw, int rows, int cols, void* Wq, int64_t ldq, float* scales_out,
                     uint32_t* scratch, hipStream_t st);
@@ -82,7 +88,7 @@ int launch_dequant_packed(const void* in, int K, int N, void* out, hipStream_t s
 int probe_mfma(bool i8, int random_operands, int iters, void* scratch, hipStream_t st, float* rate_out, float* mhz_out);
 int launch_quantize_pack_int4(const void* W, int64_t ldw, int K, int N, int transpose, void* packed, float* deq_out,
                               hipStream_t st);
-int probe_read(const void* buf, size_t bytes, int workgroups, int kib_in_flight, void* sink, hipStream_t st);
+int probe_read(const void* buf, size_t bytes, int workgroups, int waves, int blocked, int kib_in_flight, void* sink, hipStream_t st);
 int launch_matvec(bool i8, const void* A, int64_t lda, const void* b, void* c, int M, int K, hipStream_t st);
 
 struct TileCfg {
@@ -95,16 +101,14 @@ static thread_local int g_decode_halves = -1;
 static thread_local int g_decode_valu = -1;
 static thread_local int g_decode_resident = -1;
 static thread_local int g_waves = 8;
-static thread_local int g_a_kblocked = 0;
 TileCfg forced_tile() { return g_forced; }
 int load_mode() { return g_load_mode; }
 int decode_halves() { return g_decode_halves; }
 int decode_valu() { return g_decode_valu; }
 int decode_resident() { return g_decode_resident; }
 int wave_count() { return g_waves; }
-int a_kblocked() { return g_a_kblocked; }
 
-static int elesz_of(int dtype) { return dtype == MMX_BF16 ? 2 : dtype == MMX_I8 ? 1 : 0; }
+static int elesz_of(int dtype) { return dtype == MMX_BF16 ? 2 : (dtype == MMX_I8 || dtype == MMX_U8) ? 1 : 0; }
 
 static int out_size(int dtype) {
     switch (dtype) {
@@ -190,6 +194,19 @@ static int gemm_dispatch(int a_dtype, int b_dtype, const void* A, int64_t lda_by
               : launch_gemm_tiles_bf16(A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, rq, st);
 }
 
+// the signed int8 GEMM into raw int32 accumulators (the middle pass of mmx_gemm_u8)
+static int signed_gemm_i32(const void* A, int64_t lda, const void* Bp, int M, int K, int N, int n0, int n1, int32_t* acc,
+                           int64_t ldacc_bytes, hipStream_t st) {
+    mmx_epilogue e;
+    memset(&e, 0, sizeof e);
+    e.steps = MMX_PP_NONE;
+    e.out_dtype = MMX_I32;
+    e.C = acc;
+    e.ldc_bytes = ldacc_bytes;
+    const SplitRequest none = {1, nullptr, 0};
+    return gemm_dispatch(MMX_I8, MMX_I8, A, lda, Bp, M, K, N, n0, n1, &e, none, st);
+}
+
 }  // namespace mmx
 
 using namespace mmx;
@@ -234,13 +251,13 @@ size_t mmx_packed_b_bytes(int dtype, int K, int N) {
 
 int mmx_repack_b(int dtype, const void* B, int64_t ldb_bytes, int K, int N, int transpose, void* packed, void* stream) {
     const int es = elesz_of(dtype);
-    if (!es) return set_error(MMX_E_INVALID, "mmx_repack_b: dtype %d is neither bf16 nor int8", dtype);
+    if (!es) return set_error(MMX_E_INVALID, "mmx_repack_b: dtype %d is neither bf16 nor (u)int8", dtype);
     if (!B || !packed) return set_error(MMX_E_INVALID, "mmx_repack_b: NULL pointer");
     if (K <= 0 || N <= 0) return set_error(MMX_E_INVALID, "mmx_repack_b: K and N must be positive");
     const int64_t min_ld = (int64_t)(transpose ? K : N) * es;
     if (ldb_bytes < min_ld || ldb_bytes % es) return set_error(MMX_E_INVALID, "mmx_repack_b: ldb_bytes %lld too small or misaligned", (long long)ldb_bytes);
     if (reinterpret_cast<uintptr_t>(packed) & 15) return set_error(MMX_E_INVALID, "mmx_repack_b: packed buffer must be 16-byte aligned");
-    return launch_repack(es, B, ldb_bytes, K, N, transpose, packed, static_cast<hipStream_t>(stream));
+    return launch_repack(es, B, ldb_bytes, K, N, transpose, packed, static_cast<hipStream_t>(stream), dtype == MMX_U8 ? 1 : 0);
 }
 
 int mmx_repack_gate_up(const void* w_gate, const void* w_up, int64_t ldw_bytes, int K, int N, void* packed, void* stream) {
@@ -333,12 +350,51 @@ size_t mmx_gemm_workspace_bytes(int a_dtype, int b_dtype, int M, int K, int N, i
 
 int mmx_matvec(int dtype, const void* A, int64_t lda_bytes, const void* b, void* c, int M, int K, void* stream) {
     const int es = elesz_of(dtype);
+    if (dtype == MMX_U8) return set_error(MMX_E_INVALID, "mmx_matvec: unsigned operands go through mmx_matvec_u8");
     if (!es) return set_error(MMX_E_INVALID, "mmx_matvec: dtype %d is neither bf16 nor int8", dtype);
     if (!A || !b || !c || M <= 0 || K <= 0) return set_error(MMX_E_INVALID, "mmx_matvec: bad argument");
     if (lda_bytes < (int64_t)K * es) return set_error(MMX_E_INVALID, "mmx_matvec: lda_bytes smaller than a row of A");
     if (lda_bytes % es || (reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(b)) % es || reinterpret_cast<uintptr_t>(c) % 4)
         return set_error(MMX_E_INVALID, "mmx_matvec: A, b or c is not aligned to its element size");
     return launch_matvec(dtype == MMX_I8, A, lda_bytes, b, c, M, K, static_cast<hipStream_t>(stream));
+}
+
+size_t mmx_gemm_u8_scratch_bytes(int a_dtype, int b_dtype, int M, int K, int N, int n0, int n1) {
+    const bool au = a_dtype == MMX_U8, bu = b_dtype == MMX_U8;
+    if ((!au && a_dtype != MMX_I8) || (!bu && b_dtype != MMX_I8) || (!au && !bu)) return 0;
+    if (M <= 0 || K <= 0 || N <= 0 || n0 < 0 || n1 > N || n0 >= n1) return 0;
+    return u8_scratch_bytes(au, M, K, n1);
+}
+
+int mmx_gemm_u8(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* Bpacked, int M, int K, int N, int n0, int n1,
+                const mmx_epilogue* ep_in, void* scratch, size_t scratch_bytes, void* stream) {
+    const bool au = a_dtype == MMX_U8, bu = b_dtype == MMX_U8;
+    if ((!au && a_dtype != MMX_I8) || (!bu && b_dtype != MMX_I8) || (!au && !bu))
+        return set_error(MMX_E_INVALID, "mmx_gemm_u8: dtypes (%d, %d): each MMX_I8 or MMX_U8, at least one unsigned", a_dtype, b_dtype);
+    if (!A || !Bpacked || !scratch) return set_error(MMX_E_INVALID, "mmx_gemm_u8: NULL operand or scratch");
+    if (M <= 0 || K <= 0 || N <= 0) return set_error(MMX_E_INVALID, "mmx_gemm_u8: M, K, N must be positive");
+    if (n0 < 0 || n1 > N || n0 >= n1 || n0 % 32) return set_error(MMX_E_INVALID, "mmx_gemm_u8: column range [%d, %d) (n0 a multiple of 32) outside [0, %d)", n0, n1, N);
+    if (lda_bytes < K) return set_error(MMX_E_INVALID, "mmx_gemm_u8: lda_bytes smaller than a row of A");
+    if (reinterpret_cast<uintptr_t>(scratch) & 255) return set_error(MMX_E_INVALID, "mmx_gemm_u8: the scratch must be 256-byte aligned");
+    const size_t need = u8_scratch_bytes(au, M, K, n1);
+    if (scratch_bytes < need) return set_error(MMX_E_INVALID, "mmx_gemm_u8: %zu bytes of scratch, %zu needed", scratch_bytes, need);
+    Epilogue ep;
+    // the post-op is checked as for a signed int8 GEMM (raw int32 output only with steps == 0)
+    int rc = make_epilogue(ep_in, MMX_I8, MMX_I8, M, n0, n1, &ep);
+    if (rc) return rc;
+    if (ep.steps & MMX_PP_SILU_GATE) return set_error(MMX_E_INVALID, "mmx_gemm_u8: SILU_GATE needs bf16 activations");
+    return launch_gemm_x8(au, bu, A, lda_bytes, Bpacked, M, K, N, n0, n1, ep, static_cast<char*>(scratch), static_cast<hipStream_t>(stream),
+                          signed_gemm_i32);
+}
+
+int mmx_matvec_u8(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* b, void* c, int M, int K, void* stream) {
+    const bool au = a_dtype == MMX_U8, bu = b_dtype == MMX_U8;
+    if ((!au && a_dtype != MMX_I8) || (!bu && b_dtype != MMX_I8) || (!au && !bu))
+        return set_error(MMX_E_INVALID, "mmx_matvec_u8: dtypes (%d, %d): each MMX_I8 or MMX_U8, at least one unsigned", a_dtype, b_dtype);
+    if (!A || !b || !c || M <= 0 || K <= 0) return set_error(MMX_E_INVALID, "mmx_matvec_u8: bad argument");
+    if (lda_bytes < K) return set_error(MMX_E_INVALID, "mmx_matvec_u8: lda_bytes smaller than a row of A");
+    if (reinterpret_cast<uintptr_t>(c) % 4) return set_error(MMX_E_INVALID, "mmx_matvec_u8: c is not aligned to its element size");
+    return launch_matvec_x8(au, bu, A, lda_bytes, b, c, M, K, static_cast<hipStream_t>(stream));
 }
 
 int mmx_mlp(const void* x, int64_t ldx_bytes, const void* w_gate_up, const void* w_down, void* h, int64_t ldh_bytes, void* y,
@@ -404,11 +460,6 @@ int mmx_set_option(const char* name, int value) {
         g_decode_resident = value;
         return MMX_OK;
     }
-    if (name && !strcmp(name, "a_kblocked")) {
-        if (value != 0 && value != 1) return set_error(MMX_E_INVALID, "mmx_set_option: a_kblocked is 0 or 1");
-        g_a_kblocked = value;
-        return MMX_OK;
-    }
     if (name && !strcmp(name, "waves")) {
         if (value != 4 && value != 8) return set_error(MMX_E_INVALID, "mmx_set_option: waves is 4 or 8");
         g_waves = value;
@@ -423,10 +474,11 @@ int mmx_probe_mfma(int dtype, int random_operands, int iters, void* scratch, voi
     return probe_mfma(dtype == MMX_I8, random_operands, iters, scratch, static_cast<hipStream_t>(stream), rate_out, mhz_out);
 }
 
-int mmx_probe_read(const void* buf, size_t bytes, int workgroups, int kib_in_flight, void* sink, void* stream) {
+int mmx_probe_read(const void* buf, size_t bytes, int workgroups, int waves_per_workgroup, int blocked, int kib_in_flight, void* sink,
+                   void* stream) {
     if (!buf || !sink || workgroups <= 0 || workgroups > 65536 || (reinterpret_cast<uintptr_t>(buf) & 15))
         return set_error(MMX_E_INVALID, "mmx_probe_read: bad argument");
-    return probe_read(buf, bytes, workgroups, kib_in_flight, sink, static_cast<hipStream_t>(stream));
+    return probe_read(buf, bytes, workgroups, waves_per_workgroup, blocked, kib_in_flight, sink, static_cast<hipStream_t>(stream));
 }
 
 int mmx_time_gemm(int a_dtype, int b_dtype, const void* A, int64_t lda_bytes, const void* const* Bpacked_rot, int n_rot, int M,

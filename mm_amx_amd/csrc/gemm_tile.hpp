@@ -95,7 +95,6 @@ struct Mfma<int8_t> {
 struct GemmArgs {
     const char* A;
     int64_t lda;           // bytes
-    int64_t a_kstride;     // bytes from one 128-byte k-iteration of a row of A to the next (128: rows are contiguous)
     const char* Bp;        // packed weights
     int64_t panel_stride;  // bytes per 32-column panel = nk * 4096
     int M;
@@ -226,7 +225,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4,
         kt0 = slice * g.kq;
         nk = g.nk - kt0 < g.kq ? g.nk - kt0 : g.kq;
     }
-    const char* const a_base = g.A + (int64_t)kt0 * g.a_kstride;
+    const char* const a_base = g.A + (int64_t)kt0 * 128;
     const int tn = tile / g.tiles_m, tm = tile % g.tiles_m;
     MMX_STAMP(0);
     MMX_STAMP(1);
@@ -457,7 +456,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4,
             } else if constexpr (PART == 2) {
                 int st = (w + 1) >> 1;
                 st = st < last_st ? st : last_st;
-                n.srcA = a_base + (int64_t)st * g.a_kstride;
+                n.srcA = a_base + (int64_t)st * 128;
                 asm volatile("" : "+s"(n.srcA));
             } else {
                 // A operand of k-step s (0..3 within the stage): position (2 s + g32) ^ ((row >> 1) & 7) of the row
@@ -556,7 +555,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW / 4,
                 kp.m0B = lds_wave + B0 + W * BH;
                 kp.m0A = lds_wave + (((W + 1) >> 1) % RA) * A_ST + HALF * (BM / 2) * 128;
                 kp.srcB = b_base + (int64_t)hs * BP_HS;
-                kp.srcA = a_base + (int64_t)st * g.a_kstride;
+                kp.srcA = a_base + (int64_t)st * 128;
                 static_for<0, (W < R - 1 ? NL : H)>([&](auto q_c) { dma(q_c, integral_constant<int, HALF>{}, kp); });
             });
         }
@@ -979,7 +978,6 @@ struct TileCfg {
 TileCfg forced_tile();
 int load_mode();
 int wave_count();
-int a_kblocked();
 int ensure_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done_on_device);
 
 // Where the partial sums of a K split live: the first WS_COUNTER_BYTES hold one arrival counter per tile
@@ -1128,7 +1126,6 @@ static inline int prepare_gemm(GemmArgs& g, TileCfg& t, int& mode, int elesz, co
                                int M, int K, int N, int n0, int n1, const Epilogue& ep, const SplitRequest& rq, bool w8 = false) {
     g.A = static_cast<const char*>(A);
     g.lda = lda;
-    g.a_kstride = 128;
     g.Bp = static_cast<const char*>(Bp);
     g.M = M;
     g.kbytes = K * elesz;
@@ -1165,10 +1162,6 @@ static inline int prepare_gemm(GemmArgs& g, TileCfg& t, int& mode, int elesz, co
     g.ws_cnt = reinterpret_cast<uint32_t*>(use.ws);
     g.ws_part = use.ws ? use.ws + WS_COUNTER_BYTES : nullptr;
     g.stamps = nullptr;
-    if (a_kblocked() && mode == 2) {  // A as [K * elesz / 128][M][128 bytes]: a load instruction's 8 rows x 128 bytes are contiguous
-        g.lda = 128;
-        g.a_kstride = (int64_t)M * 128;
-    }
     g.tiles_m = (M + t.bm - 1) / t.bm;
     const int tiles_n = (n1 - n0 + t.bn - 1) / t.bn;
     g.total_tiles = g.tiles_m * tiles_n * g.ksplit;

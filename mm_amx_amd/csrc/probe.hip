@@ -86,26 +86,28 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(uint64_t* stamps, int ra
 }
 
 
-// A grid of resident workgroups that only reads: workgroup g walks the g-th of gridDim.x equal shares of the buffer,
-// its eight waves side by side (wave w takes the 1 KiB pieces w, w + 8, ... of the share), each wave with U pieces
-// in flight as a rolling window: piece i + U is requested as soon as piece i has been consumed (one XOR per dword).
-template <int U>
-__global__ __launch_bounds__(512) void read_stream_kernel(const char* buf, int pieces_per_wave, uint32_t* sink, uint32_t unlikely) {
+// A grid of resident workgroups that only reads: workgroup g walks the g-th of gridDim.x equal shares of the buffer with
+// NW waves, each wave with U pieces of 1 KiB in flight as a rolling window: piece i + U is requested as soon as piece i
+// has been consumed (one XOR per dword).  BLOCKED: wave w takes a contiguous run of the share (as the decode kernels'
+// waves take runs of a panel's fragments); otherwise the waves go side by side (wave w: pieces w, w + NW, ...).
+template <int U, int NW, bool BLOCKED>
+__global__ __launch_bounds__(NW * 64) void read_stream_kernel(const char* buf, int pieces_per_wave, uint32_t* sink, uint32_t unlikely) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
-    const char* p = buf + ((size_t)blockIdx.x * pieces_per_wave * 8 + wave) * 1024 + lane * 16;
+    constexpr size_t STEP = BLOCKED ? 1024 : (size_t)NW * 1024;
+    const char* p = buf + ((size_t)blockIdx.x * pieces_per_wave * NW + (BLOCKED ? (size_t)wave * pieces_per_wave : wave)) * 1024 + lane * 16;
     u32x4 w[U];
     uint32_t x = 0;
     const int last = pieces_per_wave - 1;
 #pragma unroll
-    for (int u = 0; u < U; u++) w[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + (size_t)(u < last ? u : last) * 8192));
+    for (int u = 0; u < U; u++) w[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + (size_t)(u < last ? u : last) * STEP));
     for (int i0 = 0; i0 < pieces_per_wave; i0 += U) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
             x ^= w[u][0] ^ w[u][1] ^ w[u][2] ^ w[u][3];
             int nx = i0 + U + u;  // past the end: the last piece once more (it stays in the window, unused)
             nx = nx < last ? nx : last;
-            w[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + (size_t)nx * 8192));
+            w[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + (size_t)nx * STEP));
         }
     }
 #pragma unroll
@@ -145,20 +147,30 @@ int probe_mfma(bool i8, int random_operands, int iters, void* scratch, hipStream
     return MMX_OK;
 }
 
-int probe_read(const void* buf, size_t bytes, int workgroups, int kib_in_flight, void* sink, hipStream_t st) {
-    const size_t per_wg = bytes / (size_t)workgroups;
-    if (per_wg * workgroups != bytes || per_wg % 8192 || per_wg == 0 || per_wg / 8192 > (size_t)1 << 20)
-        return set_error(MMX_E_INVALID, "mmx_probe_read: %zu bytes do not divide into %d shares of whole 8 KiB", bytes, workgroups);
-    const int ppw = (int)(per_wg / 8192);
-    const char* b = static_cast<const char*>(buf);
-    uint32_t* s = static_cast<uint32_t*>(sink);
-    switch (kib_in_flight) {
-    case 8: hipLaunchKernelGGL(read_stream_kernel<8>, dim3(workgroups), dim3(512), 0, st, b, ppw, s, 0x9e3779b9u); break;
-    case 16: hipLaunchKernelGGL(read_stream_kernel<16>, dim3(workgroups), dim3(512), 0, st, b, ppw, s, 0x9e3779b9u); break;
-    case 32: hipLaunchKernelGGL(read_stream_kernel<32>, dim3(workgroups), dim3(512), 0, st, b, ppw, s, 0x9e3779b9u); break;
-    default: return set_error(MMX_E_INVALID, "mmx_probe_read: kib_in_flight is 8, 16 or 32");
+template <int NW, bool BLOCKED>
+static int probe_read_launch(const char* b, int ppw, int workgroups, int kib, uint32_t* s, hipStream_t st) {
+    switch (kib) {
+    case 2: hipLaunchKernelGGL((read_stream_kernel<2, NW, BLOCKED>), dim3(workgroups), dim3(NW * 64), 0, st, b, ppw, s, 0x9e3779b9u); break;
+    case 4: hipLaunchKernelGGL((read_stream_kernel<4, NW, BLOCKED>), dim3(workgroups), dim3(NW * 64), 0, st, b, ppw, s, 0x9e3779b9u); break;
+    case 8: hipLaunchKernelGGL((read_stream_kernel<8, NW, BLOCKED>), dim3(workgroups), dim3(NW * 64), 0, st, b, ppw, s, 0x9e3779b9u); break;
+    case 16: hipLaunchKernelGGL((read_stream_kernel<16, NW, BLOCKED>), dim3(workgroups), dim3(NW * 64), 0, st, b, ppw, s, 0x9e3779b9u); break;
+    case 32: hipLaunchKernelGGL((read_stream_kernel<32, NW, BLOCKED>), dim3(workgroups), dim3(NW * 64), 0, st, b, ppw, s, 0x9e3779b9u); break;
+    default: return set_error(MMX_E_INVALID, "mmx_probe_read: kib_in_flight is 2, 4, 8, 16 or 32");
     }
     return check_hip(hipGetLastError(), "read_stream_kernel launch");
+}
+
+int probe_read(const void* buf, size_t bytes, int workgroups, int waves, int blocked, int kib_in_flight, void* sink, hipStream_t st) {
+    if (waves != 4 && waves != 8) return set_error(MMX_E_INVALID, "mmx_probe_read: waves_per_workgroup is 4 or 8");
+    const size_t unit = (size_t)waves * 1024;
+    const size_t per_wg = bytes / (size_t)workgroups;
+    if (per_wg * workgroups != bytes || per_wg % unit || per_wg == 0 || per_wg / unit > (size_t)1 << 20)
+        return set_error(MMX_E_INVALID, "mmx_probe_read: %zu bytes do not divide into %d shares of whole %zu KiB", bytes, workgroups, unit / 1024);
+    const int ppw = (int)(per_wg / unit);
+    const char* b = static_cast<const char*>(buf);
+    uint32_t* s = static_cast<uint32_t*>(sink);
+    if (waves == 8) return blocked ? probe_read_launch<8, true>(b, ppw, workgroups, kib_in_flight, s, st) : probe_read_launch<8, false>(b, ppw, workgroups, kib_in_flight, s, st);
+    return blocked ? probe_read_launch<4, true>(b, ppw, workgroups, kib_in_flight, s, st) : probe_read_launch<4, false>(b, ppw, workgroups, kib_in_flight, s, st);
 }
 
 }  // namespace mmx

@@ -11,9 +11,11 @@
 namespace mmx {
 
 // Packed layout: [panel = n/32][f = k/KS][lane][16 B], KS = 32/ES elements, lane = n%32 + 32*((k%KS)/(KS/2)).
+// flip: the sign bit of every byte is inverted on the way (unsigned 8-bit weights u -> u - 128 as a signed byte; the
+// zero padding is left at zero)
 template <int ES>
 __global__ void repack_kernel(const char* __restrict__ B, int64_t ldb, int K, int N, int transpose,
-                              char* __restrict__ out, int nfrag, int64_t total_slots) {
+                              char* __restrict__ out, int nfrag, int64_t total_slots, int flip) {
     constexpr int HALF = 16 / ES;  // elements per lane slot
     const int64_t slot = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (slot >= total_slots) return;
@@ -32,13 +34,13 @@ __global__ void repack_kernel(const char* __restrict__ B, int64_t ldb, int K, in
         if (ES == 2) {
             reinterpret_cast<uint16_t*>(buf)[e] = ok ? *reinterpret_cast<const uint16_t*>(src) : (uint16_t)0;
         } else {
-            buf[e] = ok ? *src : (char)0;
+            buf[e] = ok ? (char)(*src ^ (flip ? 0x80 : 0)) : (char)0;
         }
     }
     *reinterpret_cast<uint4*>(out + slot * 16) = *reinterpret_cast<const uint4*>(buf);
 }
 
-int launch_repack(int elesz, const void* B, int64_t ldb, int K, int N, int transpose, void* out, hipStream_t st) {
+int launch_repack(int elesz, const void* B, int64_t ldb, int K, int N, int transpose, void* out, hipStream_t st, int flip) {
     const int kpad_bytes = (K * elesz + 127) / 128 * 128;
     const int nfrag = kpad_bytes / 32;
     const int64_t npanels = (N + 31) / 32;
@@ -48,10 +50,10 @@ int launch_repack(int elesz, const void* B, int64_t ldb, int K, int N, int trans
     if (blocks > 0x7fffffff) return set_error(MMX_E_INVALID, "weight matrix too large to repack in one launch");
     if (elesz == 2)
         hipLaunchKernelGGL((repack_kernel<2>), dim3((unsigned)blocks), dim3(threads), 0, st,
-                           static_cast<const char*>(B), ldb, K, N, transpose, static_cast<char*>(out), nfrag, slots);
+                           static_cast<const char*>(B), ldb, K, N, transpose, static_cast<char*>(out), nfrag, slots, 0);
     else
         hipLaunchKernelGGL((repack_kernel<1>), dim3((unsigned)blocks), dim3(threads), 0, st,
-                           static_cast<const char*>(B), ldb, K, N, transpose, static_cast<char*>(out), nfrag, slots);
+                           static_cast<const char*>(B), ldb, K, N, transpose, static_cast<char*>(out), nfrag, slots, flip);
     return check_hip(hipGetLastError(), "repack_kernel launch");
 }
 

@@ -91,7 +91,7 @@ class Matmul:
         Kb, N = (matB.shape[1], matB.shape[0]) if self.transposeB else matB.shape
         if K != Kb:
             raise L.MmxError(f"Matmul: K of A ({K}) and B ({Kb}) differ")
-        kstep = 64 if matA.dtype == torch.int8 else 32
+        kstep = 64 if matA.dtype in (torch.int8, torch.uint8) else 32
         if K < kstep:  # include/kernels_amx.hpp:1183
             raise L.MmxError(f"Matmul: K = {K} must be at least {kstep}")
         n0 = 0 if n0 is None else n0
@@ -106,7 +106,10 @@ class Matmul:
                 self.internalB = L.repack_b(Wq, self.transposeB)
             else:
                 self.internalB = L.repack_b(matB, self.transposeB)
-        if self.weight_int8:
+        if matA.dtype == torch.uint8 or matB.dtype == torch.uint8:
+            # the uint8_t forms of Matmul (tdpbusd / tdpbsud / tdpbuud, include/kernels_amx.hpp:1057-1101)
+            L.gemm_u8(matA, self.internalB, N, ppkernel.descriptor(), b_unsigned=matB.dtype == torch.uint8, n0=n0, n1=n1)
+        elif self.weight_int8:
             ppkernel.set_deq_scale(self.dequant_scale_B)  # include/kernels_amx.hpp:1379
             # the int8 fragments are converted between LDS and the MFMA operand at every M (:1447-1497); no bf16 copy
             L.gemm(matA, self.internalB, N, ppkernel.descriptor(), b_dtype=L.I8, n0=n0, n1=n1)
@@ -118,6 +121,8 @@ class MatmulVector:
     """amx_kernel::MatmulVector (include/kernels_amx.hpp:833-1043): c[M] = A[M,K] · b[K]."""
 
     def __call__(self, matA, vB, vC=None):
+        if matA.dtype == torch.uint8 or vB.dtype == torch.uint8:  # is_s8u8 / is_u8s8 / is_u8u8 (:839-850)
+            return L.matvec_u8(matA, vB, vC)
         return L.matvec(matA, vB, vC)
 
 

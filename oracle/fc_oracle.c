@@ -225,6 +225,43 @@ void orc_repack_1xL_s8(const uint16_t* B, int64_t ldb, int K, int N, int L, floa
                     }
 }
 
+/* ------------------------------------------------------------------------------------ */
+/* The unsigned operand forms of the int8 GEMM and mat-vec (tdpbusd / tdpbsud / tdpbuud,
+ * include/kernels_amx.hpp:1057-1101, :839-850): exact integer products summed in int32 modulo 2^32 (the AMX
+ * accumulators wrap).  a_unsigned / b_unsigned say how the bytes of A / B are read. */
+void orc_gemm_x8(int a_unsigned, int b_unsigned, const void* A, int64_t lda, const void* B, int64_t ldb, int transB,
+                 int32_t* C, int64_t ldc, int M, int K, int N) {
+    const uint8_t* a8 = (const uint8_t*)A;
+    const uint8_t* b8 = (const uint8_t*)B;
+#pragma omp parallel for schedule(static)
+    for (int m = 0; m < M; m++)
+        for (int n = 0; n < N; n++) {
+            uint32_t acc = 0;
+            for (int k = 0; k < K; k++) {
+                const uint8_t ab = a8[(size_t)m * lda + k];
+                const uint8_t bb = transB ? b8[(size_t)n * ldb + k] : b8[(size_t)k * ldb + n];
+                const int av = a_unsigned ? (int)ab : (int)(int8_t)ab;
+                const int bv = b_unsigned ? (int)bb : (int)(int8_t)bb;
+                acc += (uint32_t)(av * bv);
+            }
+            C[(size_t)m * ldc + n] = (int32_t)acc;
+        }
+}
+
+void orc_matvec_x8(int a_unsigned, int b_unsigned, const void* A, int64_t lda, const void* b, int32_t* c, int M, int K) {
+    const uint8_t* a8 = (const uint8_t*)A;
+    const uint8_t* b8 = (const uint8_t*)b;
+    for (int m = 0; m < M; m++) {
+        uint32_t acc = 0;
+        for (int k = 0; k < K; k++) {
+            const int av = a_unsigned ? (int)a8[(size_t)m * lda + k] : (int)(int8_t)a8[(size_t)m * lda + k];
+            const int bv = b_unsigned ? (int)b8[k] : (int)(int8_t)b8[k];
+            acc += (uint32_t)(av * bv);
+        }
+        c[m] = (int32_t)acc;
+    }
+}
+
 /* int4 weight compression.  The reference has no algorithm to restate here: weight_compression/wcompress.hpp:90-134
  * and README.md:216-244 only time a stand-in that copies bytes ("we haven't found efficient instructions to
  * implement a fully-functional dequant() for INT4").  This is the definition the device code is held to:

@@ -32,6 +32,11 @@
  *                                    int8's range: beyond it the reference's conversion is undefined); the tile
  *                                    order by its index formula on matrices whose entries encode their position.
  *                                    fc16m.cpp itself needs xbyak (through test_bw.hpp) and cannot be compiled here.
+ *   orc_gemm_x8, orc_matvec_x8
+ *                          pinned  — integer arithmetic: against an int64 product everywhere, and against the
+ *                                    compiled reference where the reference has the form at all
+ *                                    (Matmul<uint8_t,int8_t> and the three MatmulVector forms; the reference's
+ *                                    Matmul with unsigned B does not compile: its repackB_1x2 has no uint8_t form)
  *   orc_quantize_int4,     spec    — PARITY UNPINNED against the reference, which has no int4 algorithm (it
  *   orc_pack_int4                    only times a byte-copying stand-in): these define what the device code
  *                                    must produce; checked by what the mathematics fixes (|w - q deq| <=
@@ -96,6 +101,11 @@ void orc_gemm_bf16_f64(const uint16_t* A, int64_t lda, const uint16_t* B, int64_
 void orc_gemm_i8(const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb, int transB,
                  int32_t* C, int64_t ldc, int M, int K, int N, int nthreads);
 
+/* C[M,N] (int32, modulo 2^32) = A x B with the bytes of A and/or B read as unsigned (tdpbusd / tdpbsud / tdpbuud,
+ * include/kernels_amx.hpp:1057-1101); lda/ldb/ldc in elements */
+void orc_gemm_x8(int a_unsigned, int b_unsigned, const void* A, int64_t lda, const void* B, int64_t ldb, int transB,
+                 int32_t* C, int64_t ldc, int M, int K, int N);
+void orc_matvec_x8(int a_unsigned, int b_unsigned, const void* A, int64_t lda, const void* b, int32_t* c, int M, int K);
 /* the same without the AVX-512BW path (scalar-order check of the fast one) */
 void orc_gemm_i8_generic(const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb, int transB,
                          int32_t* C, int64_t ldc, int M, int K, int N);

@@ -100,6 +100,23 @@ def gemm_i8(A, B, transB=False, nthreads=0):
     return Cm
 
 
+def gemm_x8(A, B, transB=False):
+    """int32 product of int8 / uint8 matrices (the dtype of each array says how its bytes are read)."""
+    M, K = A.shape
+    N = B.shape[0] if transB else B.shape[1]
+    Cm = np.empty((M, N), np.int32)
+    lib().orc_gemm_x8(int(A.dtype == np.uint8), int(B.dtype == np.uint8), _p(A), C.c_int64(_ld(A)), _p(B), C.c_int64(_ld(B)),
+                      int(transB), _p(Cm), C.c_int64(N), M, K, N)
+    return Cm
+
+
+def matvec_x8(A, b):
+    M, K = A.shape
+    c = np.empty(M, np.int32)
+    lib().orc_matvec_x8(int(A.dtype == np.uint8), int(b.dtype == np.uint8), _p(A), C.c_int64(_ld(A)), _p(b), _p(c), M, K)
+    return c
+
+
 def gemm_i8_generic(A, B, transB=False):
     M, K = A.shape
     N = B.shape[0] if transB else B.shape[1]

@@ -241,6 +241,35 @@ long long ref_rcp14_check_all(float (*fn)(float), unsigned* first_bad) {
     return bad;
 }
 
+/* The unsigned operand combinations of the int8 GEMM and mat-vec (tdpbusd / tdpbsud / tdpbuud,
+ * include/kernels_amx.hpp:1057-1101 and :839-850).  Of the GEMM only <uint8_t, int8_t> can be instantiated: with
+ * TB = uint8_t the reference's own repackB_1x2<uint8_t> does not compile (kpack_tile_B0B1 has no uint8_t overload,
+ * :293, :393, :810), so the s8 x u8 and u8 x u8 GEMMs exist as branches of TILE_DP only.  The mat-vec takes its
+ * vector as a plain pointer and instantiates in all three forms. */
+void ref_gemm_u8s8_acc(const void* A, int64_t lda_bytes, const void* B, int64_t ldb_bytes, int transB, int32_t* C,
+                       int64_t ldc, int M, int K, int N, int nthreads) {
+    RawStore<int32_t> pp{C, ldc};
+    auto tA = view<uint8_t>(A, M, K, lda_bytes);
+    auto tB = transB ? view<int8_t>(B, N, K, ldb_bytes) : view<int8_t>(B, K, N, ldb_bytes);
+    run_nsplit<amx_kernel::Matmul<uint8_t, int8_t>>(nthreads, transB, tA, tB, N, pp);
+}
+
+void ref_matvec_x8(int a_unsigned, int b_unsigned, const void* A, int64_t lda_bytes, const void* b, int32_t* c, int M, int K) {
+    if (a_unsigned && b_unsigned) {
+        auto tA = view<uint8_t>(A, M, K, lda_bytes);
+        amx_kernel::MatmulVector<uint8_t, uint8_t> mv;
+        mv(tA, reinterpret_cast<const uint8_t*>(b), c);
+    } else if (a_unsigned) {
+        auto tA = view<uint8_t>(A, M, K, lda_bytes);
+        amx_kernel::MatmulVector<uint8_t, int8_t> mv;
+        mv(tA, reinterpret_cast<const int8_t*>(b), c);
+    } else {
+        auto tA = view<int8_t>(A, M, K, lda_bytes);
+        amx_kernel::MatmulVector<int8_t, uint8_t> mv;
+        mv(tA, reinterpret_cast<const uint8_t*>(b), c);
+    }
+}
+
 /* The element expression of repackB_1xL<int8_t, L> (weight_compression/fc16m.cpp:80-81: "*dst++ = src0[n] * scale"
  * with src0 an ov::bfloat16* and dst an int8_t*), evaluated by the reference's own bfloat16 class.  The function
  * around it cannot be compiled here (its file needs xbyak); this is the part of it that has arithmetic. */

@@ -274,6 +274,32 @@ static void test_matvec(int M, int K) {
     EXPECT(ci.to_host() == refi, "MatmulVector int8 differs");
 }
 
+// ---- the unsigned byte forms (include/kernels_amx.hpp:839-850, 1057-1101) ----
+template <typename TA, typename TB>
+static void test_unsigned_bytes(int M, int K, int N) {
+    std::printf("  Matmul / MatmulVector <%s8,%s8> M=%d K=%d N=%d\n", std::is_same<TA, uint8_t>::value ? "u" : "s",
+                std::is_same<TB, uint8_t>::value ? "u" : "s", M, K, N);
+    auto rA = rand_i8(static_cast<size_t>(M) * K), rB = rand_i8(static_cast<size_t>(K) * N);  // any byte pattern
+    tensor2D<TA> A(M, K);
+    tensor2D<TB> B(K, N);
+    tensor2D<int32_t> C(M, N);
+    A.upload(reinterpret_cast<const TA*>(rA.data()));
+    B.upload(reinterpret_cast<const TB*>(rB.data()));
+    Matmul<TA, TB> mm(true, false);
+    mm(A, B, PP::StoreI32(C));
+    check_hip(hipDeviceSynchronize(), "sync");
+    std::vector<int32_t> got(static_cast<size_t>(M) * N), ref(got.size());
+    C.download(got.data());
+    orc_gemm_x8(std::is_same<TA, uint8_t>::value, std::is_same<TB, uint8_t>::value, rA.data(), K, rB.data(), N, 0, ref.data(), N, M, K, N);
+    EXPECT(got == ref, "unsigned-byte Matmul differs from the integer product");
+    device_vector<TB> b(std::vector<TB>(reinterpret_cast<const TB*>(rB.data()), reinterpret_cast<const TB*>(rB.data()) + K));
+    device_vector<int32_t> c(M);
+    MatmulVector<TA, TB>()(A, b.data, c.data);
+    std::vector<int32_t> refv(M);
+    orc_matvec_x8(std::is_same<TA, uint8_t>::value, std::is_same<TB, uint8_t>::value, rA.data(), K, rB.data(), refv.data(), M, K);
+    EXPECT(c.to_host() == refv, "unsigned-byte MatmulVector differs from the integer product");
+}
+
 // ---- LinearNxN call shape (torch-ext/test.py:35-37, 108-119) ----
 static void test_linear_nxn(int M, int K, int N) {
     std::printf("  LinearNxN M=%d K=%d N=%d\n", M, K, N);
@@ -419,6 +445,9 @@ int main() {
         test_matmul_weight_int4(7, 300, 77);
         test_matvec(901, 80);  // main.cpp:884
         test_matvec(901, 96);  // main.cpp:885
+        test_unsigned_bytes<uint8_t, int8_t>(77, 200, 95);
+        test_unsigned_bytes<int8_t, uint8_t>(160, 512, 96);
+        test_unsigned_bytes<uint8_t, uint8_t>(16, 4096, 64);
         test_linear_nxn(32, 32, 32);  // torch-ext/test.py:35
         test_linear_nxn(512, 128, 4096);  // torch-ext/test.py:37
         test_mlp(1, 512, 1024);

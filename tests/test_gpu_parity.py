@@ -590,6 +590,52 @@ def test_scaled_truncating_quantiser(po, scale):
         check_float_parity(bf16_to_f32(host_bits(y)), bf16_to_f32(y_ref), f"fc16m int8 weights M={M}")
 
 
+@pytest.mark.parametrize("a_unsigned,b_unsigned", [(True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("shape", [(5, 70, 40), (40, 256, 96), (200, 1024, 320), (16, 4096, 512)])
+def test_unsigned_byte_gemm(po, a_unsigned, b_unsigned, shape):
+    """The uint8_t forms of Matmul (tdpbusd / tdpbsud / tdpbuud, include/kernels_amx.hpp:1057-1101) through mmx_gemm_u8:
+    raw int32 sums bit-exact against the oracle (pinned to the reference's Matmul<uint8_t,int8_t> and to int64
+    products), then the requantising post-op on them, a column range, and a strided A."""
+    M, K, N = shape
+    rng = np.random.default_rng(M + K + N + 2 * a_unsigned + b_unsigned)
+    A = rng.integers(0, 256, (M, K + 16)).astype(np.uint8) if a_unsigned else rng.integers(-128, 128, (M, K + 16)).astype(np.int8)
+    B = rng.integers(0, 256, (K, N)).astype(np.uint8) if b_unsigned else rng.integers(-128, 128, (K, N)).astype(np.int8)
+    A[0, :K] = 255 if a_unsigned else -128
+    B[:, 0] = 255 if b_unsigned else -128
+    want = po.gemm_x8(np.ascontiguousarray(A[:, :K]), B)
+    Ad = dev(A)[:, :K]                                         # rows K + 16 bytes apart
+    packed = mx.repack_b(dev(B))
+    acc = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    mx.gemm_u8(Ad, packed, N, mx.Epilogue(acc, mx.PP_NONE), b_unsigned)
+    assert np.array_equal(host_bits(acc), want)
+    # the operator surface: Matmul with uint8 tensors
+    acc2 = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    if K >= 64:
+        mx.Matmul(True, False)(Ad, dev(B), ppkernel=mx.BiasGeluStore(acc2, mx.Steps.NONE))
+        assert np.array_equal(host_bits(acc2), want.astype(np.float32))
+    # post-op + column range
+    bias = rng.standard_normal(N).astype(np.float32)
+    deq = rng.uniform(1e-4, 1e-3, N).astype(np.float32)
+    steps = po.PP_DEQUANT | po.PP_BIAS | po.PP_QUANT
+    ref = po.pp(want, steps, po.I8, bias=bias, deq_per_oc=deq, q=8.0)
+    out = torch.zeros((M, N), dtype=torch.int8, device="cuda")
+    n0 = 32 if N > 64 else 0
+    mx.gemm_u8(Ad, packed, N, mx.Epilogue(out, steps, bias=dev(bias), deq_scale_per_oc=dev(deq), q_scale=8.0), b_unsigned, n0=n0, n1=N)
+    got = host_bits(out)
+    assert np.array_equal(got[:, n0:], ref[:, n0:]) and not got[:, :n0].any()
+
+
+@pytest.mark.parametrize("a_unsigned,b_unsigned", [(True, False), (False, True), (True, True)])
+def test_unsigned_byte_matvec(po, a_unsigned, b_unsigned):
+    """MatmulVector in its s8u8 / u8s8 / u8u8 forms (include/kernels_amx.hpp:839-850)."""
+    rng = np.random.default_rng(3 + 2 * a_unsigned + b_unsigned)
+    for (M, K) in ((7, 100), (40, 256), (901, 96), (33, 4096)):
+        A = rng.integers(0, 256, (M, K)).astype(np.uint8) if a_unsigned else rng.integers(-128, 128, (M, K)).astype(np.int8)
+        b = rng.integers(0, 256, K).astype(np.uint8) if b_unsigned else rng.integers(-128, 128, K).astype(np.int8)
+        got = mx.MatmulVector()(dev(A), dev(b))
+        assert np.array_equal(host_bits(got), po.matvec_x8(A, b)), (M, K)
+
+
 def _w8_case(po, M, K, N, seed, steps=None, **gemm_kw):
     """bf16 x int8-weight GEMM against the bf16 GEMM of the oracle on the (exactly representable) integers."""
     rng = np.random.default_rng(seed)

@@ -310,3 +310,23 @@ def test_int8_gemm_fast_path_equals_the_generic_one_and_int64(po):
         want = A.astype(np.int64) @ (B.T if t else B).astype(np.int64)
         assert np.array_equal(po.gemm_i8(A, B, transB=t), want)
         assert np.array_equal(po.gemm_i8_generic(A, B, transB=t), want)
+
+
+def test_unsigned_byte_products_against_int64(po):
+    """orc_gemm_x8 / orc_matvec_x8 in all four signedness combinations against an int64 product, extremes included,
+    and the identity the GPU path rests on: u = (u ^ 0x80 as a signed byte) + 128."""
+    rng = np.random.default_rng(8)
+    def draw(unsigned, shape):
+        a = rng.integers(0, 256, shape).astype(np.uint8) if unsigned else rng.integers(-128, 128, shape).astype(np.int8)
+        a.flat[0] = 255 if unsigned else -128
+        return a
+    for au in (False, True):
+        for bu in (False, True):
+            for (M, K, N, t) in ((9, 130, 21, False), (3, 64, 40, True)):
+                A, B = draw(au, (M, K)), draw(bu, (N, K) if t else (K, N))
+                want = (A.astype(np.int64) @ (B.T if t else B).astype(np.int64)).astype(np.int32)
+                assert np.array_equal(po.gemm_x8(A, B, transB=t), want)
+                b = np.ascontiguousarray((B[0] if t else B[:, 0]))
+                assert np.array_equal(po.matvec_x8(A, b), (A.astype(np.int64) @ b.astype(np.int64)).astype(np.int32))
+    u = np.arange(256, dtype=np.uint8)
+    assert np.array_equal((u ^ 0x80).view(np.int8).astype(np.int32) + 128, u.astype(np.int32))

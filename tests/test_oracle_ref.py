@@ -158,3 +158,22 @@ def test_scaled_truncating_quantiser_is_the_reference_expression(po, ref):
         defined = np.isfinite(v) & (np.abs(v) < 127.5)
         assert defined.sum() > 30000
         assert np.array_equal(got[defined], want[defined]), scale
+
+
+def test_unsigned_byte_forms_against_the_reference(po, ref):
+    """Matmul<uint8_t,int8_t> (the one unsigned GEMM the reference can instantiate) and the three unsigned forms of
+    MatmulVector (include/kernels_amx.hpp:839-850, 1057-1101) against the oracle's integer products."""
+    rng = np.random.default_rng(6)
+    for (M, K, N) in ((16, 64, 32), (37, 128, 75), (64, 256, 96), (5, 70, 40), (2, 2560, 64)):
+        A = rng.integers(0, 256, (M, K)).astype(np.uint8)
+        B = rng.integers(-128, 128, (K, N)).astype(np.int8)
+        want = np.empty((M, N), np.int32)
+        ref.ref_gemm_u8s8_acc(p(A), C.c_int64(A.strides[0]), p(B), C.c_int64(B.strides[0]), 0, p(want), C.c_int64(N), M, K, N, 1)
+        assert np.array_equal(po.gemm_x8(A, B), want)
+    for au, bu in ((1, 0), (0, 1), (1, 1)):
+        for (M, K) in ((16, 64), (33, 128), (40, 256), (7, 100)):
+            A = rng.integers(0, 256, (M, K)).astype(np.uint8) if au else rng.integers(-128, 128, (M, K)).astype(np.int8)
+            b = rng.integers(0, 256, K).astype(np.uint8) if bu else rng.integers(-128, 128, K).astype(np.int8)
+            want = np.empty(M, np.int32)
+            ref.ref_matvec_x8(au, bu, p(A), C.c_int64(A.strides[0]), p(b), p(want), M, K)
+            assert np.array_equal(po.matvec_x8(A, b), want), (au, bu, M, K)
