@@ -252,7 +252,10 @@ const char* mmx_last_kernel(void);
  * most two 32-column panels per CU; x within a CU's LDS) runs as one workgroup per CU that keeps x in LDS and walks
  * its one or two panels — -1 (default) where x is too large for the streaming kernel's two workgroups per CU and,
  * over int8 weights, wherever no workgroup gets a second panel (and only while decode_halves and decode_valu are
- * left at -1); 0 never; 1 wherever the shape allows (same bits as the streaming kernel). */
+ * left at -1); 0 never; 1 wherever the shape allows (same bits as the streaming kernel).  "decode_pair": how that
+ * kernel walks a workgroup's second panel over int8-compressed weights — 1 (default) a second group of eight waves walks
+ * it at the same time as the first panel, against the same copy of x; 0 the same eight waves walk it after the first
+ * (same bits either way). */
 int mmx_set_option(const char* name, int value);  /* like mmx_set_tile: affects the calling thread's later calls only */
 #ifdef __cplusplus
 }

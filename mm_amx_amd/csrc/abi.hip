@@ -101,12 +101,14 @@ static thread_local int g_decode_halves = -1;
 static thread_local int g_decode_valu = -1;
 static thread_local int g_decode_resident = -1;
 static thread_local int g_waves = 8;
+static thread_local int g_decode_pair = 1;
 TileCfg forced_tile() { return g_forced; }
 int load_mode() { return g_load_mode; }
 int decode_halves() { return g_decode_halves; }
 int decode_valu() { return g_decode_valu; }
 int decode_resident() { return g_decode_resident; }
 int wave_count() { return g_waves; }
+int decode_pair() { return g_decode_pair; }
 
 static int elesz_of(int dtype) { return dtype == MMX_BF16 ? 2 : (dtype == MMX_I8 || dtype == MMX_U8) ? 1 : 0; }
 
@@ -458,6 +460,11 @@ int mmx_set_option(const char* name, int value) {
     if (name && !strcmp(name, "decode_resident")) {
         if (value < -1 || value > 1) return set_error(MMX_E_INVALID, "mmx_set_option: decode_resident is -1, 0 or 1");
         g_decode_resident = value;
+        return MMX_OK;
+    }
+    if (name && !strcmp(name, "decode_pair")) {
+        if (value != 0 && value != 1) return set_error(MMX_E_INVALID, "mmx_set_option: decode_pair is 0 or 1");
+        g_decode_pair = value;
         return MMX_OK;
     }
     if (name && !strcmp(name, "waves")) {

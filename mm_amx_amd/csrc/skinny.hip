@@ -962,6 +962,151 @@ __global__ __launch_bounds__(512) void skinny_resident_kernel(const SkinnyArgs s
 #undef MMX_REQUEST
 }
 
+// ---- resident-x variant, two panels side by side -----------------------------------------------------------
+// With more panels than CUs (344 on 256) the kernel above gives some workgroups a second panel to walk after the
+// first, alone on the machine and at the rate one small window allows.  Here a workgroup has SIXTEEN waves: waves 0-7
+// multiply panel blockIdx.x, waves 8-15 panel blockIdx.x + gridDim.x at the same time (where there is none they only
+// keep the barriers company), wave w and wave w + 8 the same share of K against the same slice of x, which wave w fetched: one copy
+// of x per CU, two weight streams, as two workgroups per CU would have if x fitted twice.  Same split of K over the
+// waves and same order of the sums as the kernels above: the same bits.  One barrier publishes x (a wave of the
+// second group reads what a wave of the first fetched), one ends the multiplies, after which the LDS of x becomes
+// the reduction scratch of both groups.
+template <bool W8, int U>  // U: fragments per panel and wave (K = 8 waves x U fragments)
+__global__ __launch_bounds__(1024) void skinny_resident_pair_kernel(const SkinnyArgs s, int region, int oc_off, int mr_log2) {
+    constexpr int D = U >= 32 ? 8 : 4;  // fragments (KiB) a wave keeps in flight, as above
+    constexpr int XB = W8 ? 64 : 32;    // bytes of a row of x that one fragment covers
+    extern __shared__ __attribute__((aligned(1024))) char xs[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kw = wave & 7, grp = wave >> 3;  // share of K, panel of the pair
+    const int l32 = lane & 31, g32 = lane >> 5;
+    const int row_bytes = s.K * 2;
+    const int G = gridDim.x;
+    const int panels = ((s.n1 + 31) >> 5) - (s.n0 >> 5);
+    // (a group without a panel only takes part in the barriers: every wave of the workgroup reaches each of them)
+    const bool active = !(grp == 1 && (int)blockIdx.x + G >= panels);
+    const int panel = (s.n0 >> 5) + (int)blockIdx.x + (active ? grp * G : 0);
+    const Epilogue& ep = s.ep;
+    const bool deq_oc = (ep.steps & MMX_PP_DEQUANT) && ep.deq_oc, bias_oc = (ep.steps & MMX_PP_BIAS) != 0,
+               q_oc = (ep.steps & MMX_PP_QUANT) && ep.q_oc;
+    const int MR = 1 << mr_log2;
+    float* const red = reinterpret_cast<float*>(xs) + grp * (256 << mr_log2);           // [8 waves][16][2][MR], over x once it is spent
+    const float* const oc = reinterpret_cast<const float*>(xs + oc_off) + grp * 192;     // [3][64] per group
+
+    constexpr int per_wave = U;  // the launcher checks: nfrag = 8 * U
+    const int f_begin = kw * per_wave;
+    const int SB = per_wave * XB;
+    const int rowp = SB + 16;
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)xs);
+    if (grp == 0) {  // slice kw of x -> region kw (pieces of 16 bytes, row-major over [M][SB / 16 + 1]; see the kernel above)
+        const uint32_t lds_w = lds_base + (uint32_t)(kw * region);
+        const int cpr1 = SB / 16 + 1;
+        const int npieces = s.M * cpr1;
+        const int slice0 = f_begin * XB;
+        int r = lane / cpr1, c = lane - r * cpr1;
+        for (int i0 = 0; i0 < npieces; i0 += 64) {
+            const int rr = r < s.M ? r : s.M - 1;
+            int cb = slice0 + (c < cpr1 - 1 ? c : cpr1 - 2) * 16;
+            cb = cb < row_bytes - 16 ? cb : row_bytes - 16;
+            const char* src = s.x + (int64_t)rr * s.ldx + cb;
+            const uint32_t m0v = lds_w + (uint32_t)(i0 * 16);
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0v), "v"(src) : "memory");
+            c += 64;
+            while (c >= cpr1) {
+                c -= cpr1;
+                r++;
+            }
+        }
+    }
+    if (kw == 0 && active) {  // the group's per-column post-op operands -> oc (lanes 32-63 repeat the 32 columns)
+        int n = (panel << 5) + l32;
+        n = n < s.n1 ? n : s.n1 - 1;
+        const uint32_t dst = lds_base + (uint32_t)(oc_off + grp * 768);
+        if (deq_oc) {
+            const float* src = ep.deq_oc + n;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(dst), "v"(src) : "memory");
+        }
+        if (bias_oc) {
+            const float* src = ep.bias + n;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(dst + 256), "v"(src) : "memory");
+        }
+        if (q_oc) {
+            const float* src = ep.q_oc + n;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(dst + 512), "v"(src) : "memory");
+        }
+    }
+
+    const int mrow = l32 < s.M ? l32 : 0;
+    const char* const xrow = xs + kw * region + mrow * rowp + g32 * (XB / 2);
+    const char* const wcur = s.Wp + (int64_t)panel * s.panel_stride + (int64_t)f_begin * 1024 + lane * 16;
+
+    u32x4 w[D];
+    f32x16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+
+    // the first fragments behind x; "at most these outstanding" = this wave's loads of x and operands have landed;
+    // the barrier then publishes every slice to both groups
+    constexpr int U0 = D < 4 ? D : 4;
+    if (active) {
+#pragma unroll
+        for (int g = 0; g < U0; g++) {
+            w[g % D] = MMX_WLOAD(wcur + g * 1024);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "n"(U0) : "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    if (active) {
+#pragma unroll
+        for (int g = U0; g < D; g++) {
+            w[g % D] = MMX_WLOAD(wcur + g * 1024);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int g = 0; g < U; g++) {
+            const bf16x8 xa = *reinterpret_cast<const bf16x8*>(xrow + g * XB);
+            if constexpr (W8) {
+                const bf16x8 xc = *reinterpret_cast<const bf16x8*>(xrow + g * XB + 16);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(w[g % D].x, w[g % D].y), xa, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s8x8_to_bf16(w[g % D].z, w[g % D].w), xc, acc, 0, 0, 0);
+            } else {
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, w[g % D]), xa, acc, 0, 0, 0);
+            }
+            if (g + D < U) {
+                w[g % D] = MMX_WLOAD(wcur + (g + D < U ? g + D : 0) * 1024);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+    // every wave has read its last x: the regions become the reduction scratch
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory");
+    if (l32 < MR && active) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) red[((((kw * 16 + v) * 2) + g32) << mr_log2) + l32] = acc[v];
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory");
+    if (!active) return;
+    const int gtid = tid & 511;  // thread of the group
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int idx = gtid + 512 * t;
+        const int v = idx >> (mr_log2 + 1), g = (idx >> mr_log2) & 1, m = idx & (MR - 1);
+        const int nloc = 8 * (v >> 2) + 4 * g + (v & 3);
+        const int n = (panel << 5) + nloc;
+        if (v >= 16 || m >= s.M || n >= s.n1) continue;
+        float r = 0.0f;
+#pragma unroll
+        for (int w8 = 0; w8 < 8; w8++) r += red[((((w8 * 16 + v) * 2) + g) << mr_log2) + m];
+        if (ep.steps & MMX_PP_DEQUANT) r = r * (deq_oc ? oc[nloc] : ep.deq);
+        if (ep.steps & MMX_PP_BIAS) r = r + oc[64 + nloc];
+        if (ep.steps & MMX_PP_GELU) r = gelu_erf_minimax(r);
+        if (ep.steps & MMX_PP_QUANT) r = r * (q_oc ? oc[128 + nloc] : ep.q);
+        store_out(ep, m, n, r);
+    }
+}
+
 // Half-panel variant of the streaming kernel for 1-4 rows of x.  A list of 32-column panels that is only 1-2
 // per CU long leaves some CUs with twice the work of others (or idle), and how fast one CU can pull
 // weights in is what bounds this kernel.  Here a workgroup (four waves) multiplies HALF a panel
@@ -1155,6 +1300,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 int decode_halves();
 int decode_valu();
 int decode_resident();
+int decode_pair();
 
 // int8 x int8 at M <= 32 can use the decode kernels if x is 16-byte aligned and K fills whole 128-byte groups of
 // the packed weights: the streaming form if x fits in LDS, else the chunked one, which walks K in chunks of 256
@@ -1410,8 +1556,20 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
         // (two panels on some CUs: ahead of the chunked form while a good part of the CUs has one, 344 or 432 panels on 256
         // CUs; with two on every CU, 8192 x 16384 at M = 8, the chunked form's two workgroups per CU win, 24.5 against 26.0 us)
         const bool some_two = !one_each && panels * 4 <= 7 * num_cus();
+        // Second panels over int8 weights are walked side by side by a second group of eight waves
+        // (skinny_resident_pair_kernel: one copy of x, two weight streams; 4096 x 11008 at M = 12 / 16 12.5 / 13.0 -> 12.1 /
+        // 12.5 us, 4096 x 13824 at M = 1 / 8 / 16 12.0 / 12.8 / 14.0 -> 11.8 / 12.3 / 13.2, 4096 x 16384 13.8 / 14.4 / 15.5 ->
+        // 13.4 / 14.1 / 15.0).  Over bf16 weights the pair is behind the one-after-the-other form (4096 x 11008 at M = 1
+        // 18.9 against 18.5 us, 4096 x 16384 27.1 against 23.8) and is not used.  With few rows and fewer than 1.5 panels
+        // per CU the streaming form stays ahead (11008 columns, M = 1 / 4: 10.7 / 11.0 against 11.0 / 11.4).
+        const int pair_red = 2 * (1024 << mr_log2);
+        const int pair_oc_off = 8 * region > pair_red ? 8 * region : pair_red;
+        const int pair_lds = pair_oc_off + 2 * 768;
+        const bool pair_ok = w8 && !one_each && (s.nfrag == 128 || s.nfrag == 256) && decode_pair() != 0 && pair_lds <= 160 * 1024;
+        const bool pair_rule = pair_ok && s.nfrag == 128 && decode_valu() == -1 && decode_halves() == -1 &&
+                               (xbytes > 80 * 1024 || panels * 2 >= 3 * num_cus());
         const bool by_rule = (xbytes > 80 * 1024 && (one_each || (w8 && some_two))) ||
-                             (w8 && one_each && decode_valu() == -1 && decode_halves() == -1);
+                             (w8 && one_each && decode_valu() == -1 && decode_halves() == -1) || pair_rule;
         if (shape_ok && rforce != 0 && (rforce == 1 || by_rule)) {
             typedef void (*ResidentKernel)(const SkinnyArgs, int, int, int);
             static std::atomic<uint64_t> attr_done[6];
@@ -1422,8 +1580,20 @@ int launch_skinny(int wk, const void* x, int64_t ldx, const void* Wp, int M, int
             const ResidentKernel kern = kerns[ki];
             const int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, attr_done[ki]);
             if (rc) return rc;
-            note_kernel(w8 ? "skinny_resident_w8" : "skinny_resident_bf16");
             const int grid = panels < num_cus() ? panels : num_cus();
+            if (pair_ok) {
+                // second panels: sixteen waves walk both panels of a workgroup at the same time over one copy of x
+                typedef void (*PairKernel)(const SkinnyArgs, int, int, int);
+                static std::atomic<uint64_t> pair_done[2];
+                const PairKernel pkerns[2] = {skinny_resident_pair_kernel<true, 16>, skinny_resident_pair_kernel<true, 32>};
+                const int pi = s.nfrag == 256 ? 1 : 0;
+                const int rc2 = ensure_dynamic_lds(reinterpret_cast<const void*>(pkerns[pi]), 160 * 1024, pair_done[pi]);
+                if (rc2) return rc2;
+                note_kernel("skinny_resident_w8_pair");
+                hipLaunchKernelGGL(pkerns[pi], dim3(grid), dim3(1024), pair_lds, st, s, region, pair_oc_off, mr_log2);
+                return check_hip(hipGetLastError(), "skinny_resident_pair_kernel launch");
+            }
+            note_kernel(w8 ? "skinny_resident_w8" : "skinny_resident_bf16");
             hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, st, s, region, red_off, mr_log2);
             return check_hip(hipGetLastError(), "skinny_resident_kernel launch");
         }

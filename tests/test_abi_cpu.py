@@ -63,7 +63,8 @@ def test_sizes_and_argument_validation(lib):
     assert lib.mmx_set_option(b"nonsense", 1) != 0
     # every documented option takes its documented values and nothing else
     for name, good, bad in ((b"load_mode", (0, 2), (1, 3)), (b"waves", (4, 8), (2, 16)), (b"decode_halves", (-1, 0, 1), (-2, 2)),
-                            (b"decode_valu", (-1, 0, 1), (-2, 2)), (b"decode_resident", (-1, 0, 1), (-2, 2))):
+                            (b"decode_valu", (-1, 0, 1), (-2, 2)), (b"decode_resident", (-1, 0, 1), (-2, 2)),
+                            (b"decode_pair", (0, 1), (-1, 2))):
         for v in bad:
             assert lib.mmx_set_option(name, v) != 0, (name, v)
         for v in good:
@@ -74,7 +75,11 @@ def test_sizes_and_argument_validation(lib):
     # NULL operands are rejected by validation, before any HIP call
     assert lib.mmx_gemm(1, 1, None, C.c_int64(0), None, 1, 64, 64, 0, 64, None, None) == -1
     assert b"NULL" in lib.mmx_last_error()
-    assert lib.mmx_repack_b(5, None, C.c_int64(0), 1, 1, 0, None, None) == -1
+    assert lib.mmx_repack_b(7, None, C.c_int64(0), 1, 1, 0, None, None) == -1   # no such dtype
+    assert lib.mmx_repack_b(5, None, C.c_int64(0), 1, 1, 0, None, None) == -1   # unsigned bytes, NULL pointers
+    assert lib.mmx_gemm_u8(2, 2, None, C.c_int64(0), None, 1, 64, 64, 0, 64, None, None, C.c_size_t(0), None) == -1  # nothing unsigned
+    lib.mmx_gemm_u8_scratch_bytes.restype = C.c_size_t
+    assert lib.mmx_gemm_u8_scratch_bytes(2, 2, 4, 64, 64, 0, 64) == 0 and lib.mmx_gemm_u8_scratch_bytes(5, 2, 4, 64, 64, 0, 64) > 0
 
 
 def test_package_fails_loudly_without_the_library(monkeypatch):

@@ -408,6 +408,7 @@ def test_decode_valu_form(po, shape, out):
 # the GPU's own sums, and the same bits as the streaming kernel wherever both run (same split of K over the waves,
 # same order of the cross-wave sum).
 @pytest.mark.parametrize("case", [(True, 1, 4096, 352), (True, 16, 4096, 4096), (True, 10, 4096, 11008), (True, 16, 4096, 16384),
+                                  (True, 3, 4096, 8200), (True, 13, 4096, 9000), (True, 7, 8192, 8500),
                                   (True, 5, 8192, 1000), (True, 4, 4096, 8200), (True, 6, 11008, 1000), (True, 1, 11008, 4096),
                                   (True, 12, 5120, 704), (False, 12, 4096, 2000), (False, 16, 2048, 9000), (False, 3, 4096, 96),
                                   (False, 24, 2048, 1000), (False, 19, 2048, 8300)])   # (more than 16 rows: the wider reduction scratch)
@@ -435,9 +436,13 @@ def test_decode_resident_form(po, case, out):
     tdt, odt = {"f32": (torch.float32, po.F32), "bf16": (torch.bfloat16, po.BF16), "i8": (torch.int8, po.I8)}[out]
     n0, n1 = (64, N - 5) if N > 160 else (0, N)   # a column range that starts on a panel and ends inside one
     res = {}
+    # forms: the resident-x kernel with second panels side by side (sixteen waves) or one after the other, and whatever
+    # else the library has for the shape
+    forms = (("resident", 1, 1), ("resident_seq", 1, 0), ("other", 0, 1))
     try:
-        for resident in (1, 0):
+        for form, resident, pair in forms:
             mx.set_option("decode_resident", resident)
+            mx.set_option("decode_pair", pair)
             mx.set_option("decode_halves", 0)
             mx.set_option("decode_valu", 0)
             y = torch.full((M, N), 7, dtype=tdt, device="cuda")
@@ -447,20 +452,29 @@ def test_decode_resident_form(po, case, out):
             acc = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
             mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(acc, mx.PP_NONE), **kw)
             assert ("resident" in k1) == (resident == 1) and ("resident" in mx.last_kernel()) == (resident == 1), (k1, mx.last_kernel())
-            res[resident] = (host_bits(y), host_bits(acc), mx.last_kernel())
+            if resident and not pair:
+                assert "pair" not in mx.last_kernel()
+            res[form] = (host_bits(y), host_bits(acc), mx.last_kernel())
     finally:
         mx.set_option("decode_resident", -1)
+        mx.set_option("decode_pair", 1)
         mx.set_option("decode_halves", -1)
         mx.set_option("decode_valu", -1)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    if w8 and K in (4096, 8192) and N > 32 * cus:   # second panels over int8 weights: the sixteen-wave form
+        assert res["resident"][2] == "skinny_resident_w8_pair", res["resident"][2]
     fill = host_bits(torch.full((1, 1), 7, dtype=tdt, device="cuda"))[0, 0]
-    for resident, (got, acc, kernel) in res.items():
+    for form, (got, acc, kernel) in res.items():
         check_float_parity(acc, acc_ref, f"accumulators {case} {kernel}")
         again = po.pp(acc, posteps, odt, bias=bias, deq_per_oc=scale, q_per_oc=qs)
         assert np.array_equal(got[:, n0:n1], again[:, n0:n1]), kernel
         assert np.all(got[:, :n0] == fill) and np.all(got[:, n1:] == fill), kernel   # nothing outside the range is written
-    if "stream" in res[0][2]:
-        assert np.array_equal(res[1][1].view(np.uint32), res[0][1].view(np.uint32)), res[0][2]
-        assert np.array_equal(res[1][0], res[0][0])
+    # the two resident forms split K over the waves and add the shares alike: the same bits; so does the streaming kernel
+    assert np.array_equal(res["resident"][1].view(np.uint32), res["resident_seq"][1].view(np.uint32))
+    assert np.array_equal(res["resident"][0], res["resident_seq"][0])
+    if "stream" in res["other"][2]:
+        assert np.array_equal(res["resident"][1].view(np.uint32), res["other"][1].view(np.uint32)), res["other"][2]
+        assert np.array_equal(res["resident"][0], res["other"][0])
 
 
 # The chunked kernel (x too large for LDS, or a K the resident-x kernel does not exist for) with at most one workgroup per CU
@@ -500,9 +514,11 @@ def test_decode_resident_rule(po):
         mx.gemm(x, packed, N, mx.Epilogue(y, mx.PP_NONE), k_splits=1, **kw)
         return mx.last_kernel()
 
-    assert kernel_for(True, 16, 4096, 11008) == "skinny_resident_w8"
+    assert kernel_for(True, 16, 4096, 11008) == "skinny_resident_w8_pair"  # second panels side by side
     assert kernel_for(True, 1, 4096, 4096) == "skinny_resident_w8"
-    assert kernel_for(True, 1, 4096, 11008) == "skinny_stream_w8"          # two panels on some CUs, few rows
+    assert kernel_for(True, 1, 4096, 11008) == "skinny_stream_w8"          # fewer than 1.5 panels per CU, few rows
+    assert kernel_for(True, 4, 4096, 13824) == "skinny_resident_w8_pair"   # 1.7 panels per CU
+    assert kernel_for(True, 16, 4096, 16384) == "skinny_resident_w8_pair"  # two panels on every CU, x too large to stream
     assert kernel_for(True, 16, 4096, 16416) == "skinny_chunk_w8"          # more than two panels per CU
     assert kernel_for(True, 16, 4160 - 64, 512) == "skinny_resident_w8"    # K = 4096
     assert kernel_for(True, 12, 5120, 512) == "skinny_resident_w8"         # K = 8 x 20 fragments
