@@ -32,9 +32,10 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # when the kernel that ran is the one profiled AND its source is the one that was profiled (first 16 hex digits of
 # the SHA-256 of the kernel's source file): after a change of the kernel the figure reads null until it is re-measured.
 MEASURED_TRAFFIC = {
-    "gemm_bf16_256x192_ring8w_out_bf16": {"bytes": (81702.5 * 2.000 + 27474.0 * 1.000) * 1024, "source": "mm_amx_amd/csrc/gemm_tile.hpp",
-                                          "sha": "6f92c557e1ef21c0"},
-    "skinny_stream_w8": {"bytes": (22154.3 * 2.000 + 39.7 * 1.000) * 1024, "source": "mm_amx_amd/csrc/skinny.hip", "sha": "c4f3a25ae1d3b1c9"},
+    "gemm_bf16_256x192_ring8w_out_bf16": {"bytes": (81718.2 * 2.000 + 27580.4 * 1.000) * 1024, "source": "mm_amx_amd/csrc/gemm_tile.hpp",
+                                          "sha": "497af55a19cd666b"},
+    "skinny_stream_w8": {"bytes": (22154.3 * 2.000 + 21.5 * 1.000) * 1024, "source": "mm_amx_amd/csrc/skinny.hip", "sha": "b5f086f849d23a5a"},
+    "skinny_resident_w8_pair": {"bytes": (22617.9 * 2.000 + 344.0 * 1.000) * 1024, "source": "mm_amx_amd/csrc/skinny.hip", "sha": "b5f086f849d23a5a"},
 }
 
 
@@ -77,6 +78,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU time budget of the headline baseline (the others get a third each)")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
+    ap.add_argument("--progress", action="store_true", help="name each section on stderr before it starts")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 256 MiB device-to-device copy: a kernel of known traffic to scale profiler byte counters by")
     args = ap.parse_args()
@@ -94,6 +96,11 @@ def main():
     torch.cuda.set_device(0)
     mx.init(0)
 
+    def progress(name):
+        if args.progress:
+            print(f"bench.py: {name}", file=sys.stderr, flush=True)
+
+    progress("headline")
     # ---- headline: bf16 FC + BIAS_GELU, M=1024 ------------------------------------------------------
     w = wl.ffn_up_bias_gelu(M=1024)
     M, K, N = w["M"], w["K"], w["N"]
@@ -159,6 +166,7 @@ def main():
     }
 
     if args.calibrate_copy:
+        progress("calibrate_copy")
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
         dst = torch.empty_like(src)
         for _ in range(5):
@@ -318,6 +326,7 @@ def main():
             n = max(10, len(packs))
             return round(sorted(mx.time_gemm(Ain, packs, Nn, epi, n, **kw) for _ in range(11))[5] * 1e3, 2)
 
+        progress("bf16_gemm_256x256x256")
         # bf16 256^3, fp32 out, no post-op (launch-latency bound; reported, not a roofline case)
         w1 = wl.gemm_bf16_256()
         A1, B1 = dev_bf16(w1["A"]), mx.repack_b(dev_bf16(w1["B"]))
@@ -326,6 +335,7 @@ def main():
         extra["bf16_gemm_256x256x256"] = {"us": round(ms * 1e3, 2), "tflops": round(2.0 * 256 ** 3 / ms / 1e9, 2),
                                           "kernel": mx.last_kernel()}
 
+        progress("bf16_fc_bias_gelu_sweep_M")
         # bf16 FC sweep over M
         sweep = {}
         for Ms in (128, 512, 2048):
@@ -339,6 +349,7 @@ def main():
             del As, Cs
         extra["bf16_fc_bias_gelu_sweep_M"] = sweep
 
+        progress("bf16_fc_bias_gelu_M1024_two_streams")
         # The headline FC launched alternately on two streams (independent requests, separate outputs): a launch of
         # 232 workgroups leaves 24 CUs idle and successive launches on one stream are ~5 us apart; two streams let the
         # next launch start on the idle CUs.  Throughput only - a launch on its own is not faster this way.
@@ -364,6 +375,7 @@ def main():
                                                         "frac_of_bf16_peak": round(flops / us2 / 1e6 / PEAK_BF16_TFLOPS, 4)}
         del C2
 
+        progress("int8_fc_requant_M512_K4096_N4096")
         # int8 FC with dequant/bias/requant
         wi = wl.int8_fc()
         Ai, Bi = dev(wi["A"]), mx.repack_b(dev(wi["B"]))
@@ -397,6 +409,7 @@ def main():
             "kernel": mx.last_kernel()}
         del Ai, Bi, Ci
 
+        progress("decode_gemv_int8w_K4096_N11008")
         # decode GEMV over int8 weights, rotating over 12 weight copies (540 MB > 256 MB of cache)
         gemv = {}
         for Mg in (1, 4, 16):
@@ -410,7 +423,7 @@ def main():
             gemv[str(Mg)] = {"us": round(ms * 1e3, 2), "median_us": med_us(xg, packs, wg["N"], epg, b_dtype=mx.I8),
                              "weight_GBps": round(wbytes / ms / 1e6, 0),
                              "frac_of_hbm_peak": round(wbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "kernel": mx.last_kernel(),
-                             "traffic": measured_traffic(mx.last_kernel()) if Mg == 1 else None, "algorithmic_bytes": wbytes}
+                             "traffic": measured_traffic(mx.last_kernel()) if Mg in (1, 16) else None, "algorithmic_bytes": wbytes}
             if Mg == 1:
                 # the same launch in its other form (matrix cores <-> v_dot2_f32_bf16 per lane), for the record
                 auto_valu = "valu" in mx.last_kernel()
@@ -423,6 +436,7 @@ def main():
             del packs, Wg
         extra["decode_gemv_int8w_K4096_N11008"] = gemv
 
+        progress("decode_gemv_int8w_K4096_M1_sweep_N")
         # The same GEMV (M=1) over the number of output columns, in each of its forms: per-launch cost and rate, and
         # what the balance of 32-column panels over 256 CUs is worth (N = 8192 and 16384 are exactly 1 and 2 panels per CU)
         sweepn = {}
@@ -452,6 +466,7 @@ def main():
             del packs, Wn
         extra["decode_gemv_int8w_K4096_M1_sweep_N"] = sweepn
 
+        progress("decode_k_split")
         # Decode shapes with a panel for at most every second CU: the chunked kernel whole (k_splits = 1) and with K cut
         # into slices over several workgroups (k_splits = 0 with a workspace), weights rotated over 540 MB
         ksp = {}
@@ -474,6 +489,7 @@ def main():
             del packs, Wk
         extra["decode_k_split"] = ksp
 
+        progress("decode_chain_int8w_24_layers_K4096_N11008")
         # Steady state of a chain of decode layers (the topology of main.cpp:660-711: A1 x B1 -> A2, A2 x B2 -> A1, ...,
         # one set of weights per layer): 12 pairs of [1,4096] x [4096,11008] and [1,11008] x [11008,4096] over int8
         # weights (1.08 GB, nothing repeats within the cache), every layer reading the previous layer's output,
@@ -514,6 +530,7 @@ def main():
             "note": "graph replay, M=1, each layer reads the previous layer's output; median of 10 replays"}
         del gr, W1, W2
 
+        progress("decode_gemv_int8x_int8w_K4096_N11008")
         # int8 activations x int8 weights at M=1 (int32 sums), same weights and rotation
         w8b = wl.decode_gemv_w8(M=1)
         Wi = mx.repack_b(dev(w8b["W"]))
@@ -526,6 +543,7 @@ def main():
             "frac_of_hbm_peak": round(float(w8b["K"]) * w8b["N"] / ms / 1e6 / PEAK_HBM_GBS, 4), "kernel": mx.last_kernel()}}
         del packs, Wi
 
+        progress("decode_gemv_int4w_K4096_N11008")
         # the same GEMV over int4-compressed weights (22.5 MB), rotating over 24 copies (541 MB)
         gemv4 = {}
         wg = wl.decode_gemv_w8(M=4)
@@ -543,6 +561,7 @@ def main():
         del packs, P4, W4
         extra["decode_gemv_int4w_K4096_N11008"] = gemv4
 
+        progress("bf16_x_int8w_gemm_M896_K2560_N10240")
         # bf16 activations on int8-compressed weights at large M: the shape the reference publishes its
         # weight-compressed figure on (perf.log:36: M=896, K=2560, N=10240); the int8 fragments are converted on the fly
         Mw, Kw, Nw = 896, 2560, 10240
@@ -557,6 +576,7 @@ def main():
             "weight_bytes_resident": int(Ww.numel())}
         del Aw, Ww, Cw
 
+        progress("bf16_down_proj_K11008_N4096_ksplit")
         # shapes with few output tiles, where K is split over several workgroups per tile (the MLP's down
         # projection at prefill sizes below a full machine): with and without the split
         ksp = {}
@@ -573,6 +593,7 @@ def main():
         extra["bf16_down_proj_K11008_N4096_ksplit"] = ksp
         del Wdn
 
+        progress("llama7b_mlp_fused")
         # fused Llama-7B MLP
         mlp = {}
         wm = wl.llama_mlp(M=2048)
@@ -596,6 +617,7 @@ def main():
                             "weight_GBps": round(3.0 * wm["K"] * wm["N"] * 2 / ms / 1e6, 0)}
         extra["llama7b_mlp_fused"] = mlp
 
+        progress("llama7b_mlp_stages")
         # the MLP's two GEMMs on their own, with their roofline fractions; at M=1 the weights are rotated
         # (3 copies of gate/up = 541 MB, 6 of down) so that nothing is served from the 256 MB cache
         from mm_amx_amd import _lib as L
@@ -622,6 +644,7 @@ def main():
         del gu, dn
         extra["llama7b_mlp_stages"] = stages
 
+        progress("llama7b_mlp_stack_32_layers")
         # The reference's end-to-end demo at its size (torch-ext/test.py:176-218): a stack of 32 Llama-7B MLPs (RMSNorm +
         # fused MLP, every layer its own 270 MB of weights: 8.7 GB packed + the same again for torch's layers), per-layer
         # time through torch's bf16 linear layers and through this library; at M=1 also replayed from a HIP graph,
@@ -639,6 +662,7 @@ def main():
             torch.cuda.empty_cache()
         extra["llama7b_mlp_stack_32_layers"] = demo
 
+        progress("qk_matvec_bf16_T2097152_D128")
         # q against a cache of keys (the mat-vec of test_qk.cpp): 2^21 tokens x head size 128, bf16, 537 MB
         # (more than the 256 MB last-level cache holds)
         T, D = 1 << 21, 128
@@ -660,6 +684,7 @@ def main():
                                                  "frac_of_hbm_peak": round(T * D * 2 / ms / 1e6 / PEAK_HBM_GBS, 4)}
         del keys, sc
 
+        progress("streaming_read_floor")
         # What a kernel that only streams the same number of bytes takes, launch after launch, replayed from a HIP graph
         # so that no host time is in the figure, buffers rotated over 541 MB+ (more than the last-level cache holds).
         # The decode kernels are judged against the best of these:
@@ -717,6 +742,7 @@ def main():
             del ks, flat, scf, dst
         extra["streaming_read_floor"] = floor
 
+        progress("torch_hipblaslt_same_shapes")
         # The vendor library on the same shapes, same box (torch.matmul / torch._int_mm -> hipBLASLt; the bare product,
         # no bias, no GELU, no requantisation), for context only
         vend = {}
@@ -746,6 +772,7 @@ def main():
             vend["note"] = f"{type(e).__name__}: {e}"[:160]
         extra["torch_hipblaslt_same_shapes"] = vend
 
+        progress("mfma_issue_loop")
         # what the matrix pipes deliver with nothing else going on: an issue-bound loop of independent MFMAs,
         # all-zero operands vs operands like the benchmark's (the clock under matrix load depends on the data)
         ceil = {}
