@@ -21,7 +21,8 @@ SOURCES = ["abi.hip", "gemm_bf16.hip", "gemm_i8.hip", "gemm_w8.hip",
            "gemm_bf16_out_bf16.hip", "gemm_bf16_out_f32.hip", "gemm_bf16_out_i8.hip",
            "gemm_i8_out_i8.hip", "gemm_i8_out_i32.hip", "gemm_i8_out_f32.hip", "gemm_i8_out_bf16.hip",
            "skinny.hip", "repack.hip", "probe.hip", "u8.hip"]
-HEADERS = ["common.hpp", "gemm_tile.hpp", os.path.join("..", "..", "include", "mm_amx_amd.h")]
+HEADERS = ["common.hpp", "gemm_tile.hpp", os.path.join("..", "..", "include", "mm_amx_amd.h"),
+           os.path.join("..", "..", "include", "mm_amx_amd_bench.h")]
 # -ffp-contract=off: the epilogues reproduce the reference's separately rounded mul/add sequence;
 # fused operations are spelled fmaf().  Packed fp32 VALU instructions stay disabled.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-Wall", "-Wno-unused-function",

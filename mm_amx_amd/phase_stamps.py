@@ -1,10 +1,12 @@
-"""Per-workgroup phase timings of the MFMA tile kernels, from the instrumented build.
+"""Per-workgroup phase timings of the MFMA tile kernels and of the streaming decode kernel, from the instrumented build.
 
-    python -m mm_amx_amd.build --stamps
-    python -m mm_amx_amd.phase_stamps bf16,1024,4096,11008,256x192,1,8 i8,512,4096,4096,128x64,1
+    python -m mm_amx_amd.phase_stamps bf16,1024,4096,11008,256x192,1,8 i8,512,4096,4096,128x64,1 gemv8,1,4096,11008
 
 Each argument is  dtype,M,K,N,tile,k_splits[,waves]  (dtype bf16: the FC with BIAS+GELU and a bf16 store; i8: the int8 FC
-with DEQUANT+BIAS+QUANT and an int8 store; w8: bf16 activations on int8-compressed weights, DEQUANT, fp32 store; tile as for mmx_set_tile, empty = the library's choice; waves 4 or 8).
+with DEQUANT+BIAS+QUANT and an int8 store; w8: bf16 activations on int8-compressed weights, DEQUANT, fp32 store; tile as for
+mmx_set_tile, empty = the library's choice; waves 4 or 8), or  gemv8,M,K,N  (decode: bf16 activations on int8 weights
+through the streaming kernel, weights rotated over 540 MB).  The instrumented library is built on first use (several
+minutes) and whenever a kernel source is newer than it.
 The instrumented library (libmm_amx_amd_stamps.so, -DMMX_STAMPS) makes thread 0 of every workgroup write the shader
 clock at its phase boundaries behind the K-split workspace; this module launches the shape, reads the stamps back and
 prints medians over the workgroups: cycles from start to the first data in LDS, of the main loop, of parking and
@@ -21,8 +23,9 @@ import mm_amx_amd as mx
 from mm_amx_amd import _lib
 
 # the library is loaded on first use: point the binding at the instrumented build before that
+STAMPS_LIB = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmm_amx_amd_stamps.so")
 if "MMX_LIB_PATH" not in os.environ:
-    _lib._LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmm_amx_amd_stamps.so")
+    _lib._LIB_PATH = STAMPS_LIB
 
 STAMP_OFFSET = 96 << 20          # the kernels write at workspace partials + 96 MiB + 64 * unit index
 COUNTER_BYTES = 16 << 10
@@ -92,13 +95,70 @@ def run(ws, dt, M, K, N, tile, S, waves=8, out=sys.stdout):
     print(line, file=out, flush=True)
 
 
+def run_decode(ws, M, K, N, out=sys.stdout):
+    """The streaming decode kernel's stamps: 0/7 wall clock at start/end, 1 start, 2 x in LDS, 3 end of the weight stream,
+    4 after the barrier, 5 after the reduction and the store (shader clock)."""
+    W = mx.repack_b(torch.randint(-127, 128, (K, N), dtype=torch.int8, device="cuda"))
+    packs = [W] + [W.clone() for _ in range(max(2, int(540e6 // (K * N))) - 1)]
+    x = torch.randn((M, K), device="cuda").to(torch.bfloat16)
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    ep = mx.Epilogue(y, mx.PP_DEQUANT, deq_scale=1e-3)
+    stamp_off = COUNTER_BYTES + STAMP_OFFSET
+    mx.set_option("decode_resident", 0)
+    mx.set_option("decode_valu", 0)
+    try:
+        mx.time_gemm(x, packs, N, ep, 200, b_dtype=mx.I8, ws=ws)
+        ms = mx.time_gemm(x, packs, N, ep, 200, b_dtype=mx.I8, ws=ws)
+        kern = mx.last_kernel()
+        torch.cuda.synchronize()
+        for rep in range(4):                      # four launches in a row, the last one's stamps are read
+            ws[stamp_off:].zero_()
+            for i in range(4):
+                mx.gemm(x, packs[(rep * 4 + i) % len(packs)], N, ep, b_dtype=mx.I8, ws=ws)
+            torch.cuda.synchronize()
+    finally:
+        mx.set_option("decode_resident", -1)
+        mx.set_option("decode_valu", -1)
+    st = ws[stamp_off:].view(torch.int64).cpu().numpy().reshape(-1, 8)
+    st = st[st[:, 0] != 0]
+    if not len(st):
+        print(f"== gemv8 {M}x{K}x{N} {kern}: {ms * 1e3:.2f} us/launch, no stamps (this kernel is not instrumented)", file=out)
+        return
+    t0 = st[:, 0].min()
+    start, end = (st[:, 0] - t0) / 100.0, (st[:, 7] - t0) / 100.0
+    ghz = np.median((st[:, 5] - st[:, 1]) / np.maximum(end - start, 1e-3)) / 1e3
+
+    def d(a, b):
+        return np.median(st[:, b] - st[:, a])
+    print(f"== gemv8 {M}x{K}x{N} {kern}: {ms * 1e3:.2f} us/launch, {len(st)} workgroups, clock ~{ghz:.2f} GHz", file=out)
+    print(f"   workgroup start after the first: median {np.median(start):.2f} max {start.max():.2f} us; life median "
+          f"{np.median(end - start):.2f} max {(end - start).max():.2f} us; last end {end.max():.2f} us", file=out)
+    print(f"   cycles, median: start->x in LDS {d(1, 2):.0f}   weight stream + products {d(2, 3):.0f}   barrier {d(3, 4):.0f}   "
+          f"reduction + store {d(4, 5):.0f}", file=out, flush=True)
+
+
+def ensure_library():
+    """Build the instrumented library if it is missing or older than a kernel source (the shipped tree holds none)."""
+    if "MMX_LIB_PATH" in os.environ:
+        return
+    from mm_amx_amd import build as B
+    srcs = [os.path.join(B.CSRC, f) for f in list(B.SOURCES) + list(B.HEADERS)]
+    if not os.path.exists(STAMPS_LIB) or os.path.getmtime(STAMPS_LIB) < max(os.path.getmtime(f) for f in srcs):
+        print("phase_stamps: building the instrumented library (several minutes)", file=sys.stderr, flush=True)
+        B.build(incremental=True, stamps=True)
+
+
 def main(argv):
+    ensure_library()
     if "stamps" not in os.path.basename(mx.lib_path()):
-        sys.exit("phase_stamps: the instrumented library is needed (python -m mm_amx_amd.build --stamps)")
+        sys.exit("phase_stamps: MMX_LIB_PATH does not name an instrumented library (python -m mm_amx_amd.build --stamps)")
     mx.init(0)
     ws = torch.zeros(COUNTER_BYTES + STAMP_OFFSET + STAMP_BYTES, dtype=torch.uint8, device="cuda")
     for a in argv:
         parts = a.split(",")
+        if parts[0] == "gemv8":
+            run_decode(ws, int(parts[1]), int(parts[2]), int(parts[3]))
+            continue
         dt, M, K, N, tile, S = parts[:6]
         run(ws, dt, int(M), int(K), int(N), tile, int(S), waves=int(parts[6]) if len(parts) > 6 else 8)
 
