@@ -1,5 +1,7 @@
 """The entry point that allocates nothing (mmx_gemm_splitk_static): same results as mmx_gemm_splitk with a caller's
 workspace of the same size, on two calls in a row, the second with a smaller input."""
+import contextlib
+
 import numpy as np
 import pytest
 import torch
@@ -11,6 +13,19 @@ pytestmark = pytest.mark.gpu
 import mm_amx_amd as mx  # noqa: E402
 from mm_amx_amd import _lib as L  # noqa: E402
 from mm_amx_amd import workloads as wl  # noqa: E402
+
+
+@contextlib.contextmanager
+def _no_device_allocation():
+    """The free device memory as the driver reports it (hipMemGetInfo: it sees every hipMalloc and hipFree of the process,
+    also those that do not go through torch's caching allocator) and torch's own counter must both be unchanged by the
+    calls inside; the queue is drained on either side so that nothing in flight holds memory."""
+    torch.cuda.synchronize()
+    free0, torch0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
+    yield
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == torch0
+    assert torch.cuda.mem_get_info()[0] == free0, (free0, torch.cuda.mem_get_info()[0])
 
 
 def _int8_case(po, M, K, N, seed, k_splits, ws):
@@ -25,11 +40,10 @@ def _int8_case(po, M, K, N, seed, k_splits, ws):
     want = torch.zeros((M, N), dtype=torch.int8, device="cuda")
     mx.gemm(Ad, packed, N, mx.Epilogue(want, steps, **kw), k_splits=k_splits, ws=ws)
     k_want = mx.last_kernel()
-    before = torch.cuda.memory_allocated()
     got = torch.full((M, N), 77, dtype=torch.int8, device="cuda")
-    after_out = torch.cuda.memory_allocated()
-    mx.gemm_static(Ad, packed, N, mx.Epilogue(got, steps, **kw), k_splits=k_splits)
-    assert torch.cuda.memory_allocated() == after_out and after_out >= before
+    ep_got = mx.Epilogue(got, steps, **kw)
+    with _no_device_allocation():
+        mx.gemm_static(Ad, packed, N, ep_got, k_splits=k_splits)
     assert mx.last_kernel() == k_want
     assert np.array_equal(host_bits(got), host_bits(want)), (M, K, N, k_want)
     assert np.array_equal(host_bits(got), po.pp(po.gemm_i8(A, B), steps, po.I8, bias=bias, deq_per_oc=deq, q=20.0))
@@ -46,7 +60,9 @@ def _bf16_case(po, M, K, N, seed, k_splits, ws):
     mx.gemm(Ad, packed, N, mx.Epilogue(want, mx.PP_BIAS | mx.PP_GELU, bias=bd), k_splits=k_splits, ws=ws)
     k_want = mx.last_kernel()
     got = torch.full((M, N), 3.0, dtype=torch.bfloat16, device="cuda")
-    mx.gemm_static(Ad, packed, N, mx.Epilogue(got, mx.PP_BIAS | mx.PP_GELU, bias=bd), k_splits=k_splits)
+    ep_got = mx.Epilogue(got, mx.PP_BIAS | mx.PP_GELU, bias=bd)
+    with _no_device_allocation():
+        mx.gemm_static(Ad, packed, N, ep_got, k_splits=k_splits)
     assert mx.last_kernel() == k_want
     # the same plan adds the same partial sums in the same order: the bits agree, not just the values
     assert np.array_equal(host_bits(got), host_bits(want)), (M, K, N, k_want)
@@ -74,6 +90,46 @@ def test_static_workspace_entry_point_matches_the_workspace_one(po):
     assert k7.startswith("skinny_chunk_bf16_ksplit") and k8.startswith("skinny_chunk_i8_ksplit") and "skinny" in k9, (k7, k8, k9)
     torch.cuda.synchronize()
     assert not ws[:16 << 10].any().item()
+
+
+def test_static_workspace_entry_point_replays_from_a_hip_graph(po):
+    """One call of the entry point captured into a HIP graph after a warm-up call (capture forbids allocation, so a
+    capture that succeeds is itself the check) and replayed with new inputs: every replay gives the bits of an eager
+    call with a caller's workspace."""
+    mx.init(0)
+    M, K, N, S = 200, 4096, 640, 2
+    rng = np.random.default_rng(77)
+    B = wl.f32_to_bf16_bits((rng.standard_normal((K, N)) * 0.05).astype(np.float32))
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    packed, bd = mx.repack_b(dev_bf16(B)), dev(bias)
+    x = dev_bf16(wl.f32_to_bf16_bits(rng.standard_normal((M, K)).astype(np.float32))).clone()
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    ep = mx.Epilogue(y, mx.PP_BIAS | mx.PP_GELU, bias=bd)
+    ws = torch.zeros(L.WORKSPACE_BYTES, dtype=torch.uint8, device="cuda")
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        mx.gemm_static(x, packed, N, ep, k_splits=S)   # warm-up on the capture stream
+        side.synchronize()
+        with torch.cuda.graph(g, stream=side):
+            mx.gemm_static(x, packed, N, ep, k_splits=S)
+    assert f"ksplit{S}" in mx.last_kernel()
+    torch.cuda.synchronize()
+    for rep in range(3):
+        x.copy_(dev_bf16(wl.f32_to_bf16_bits(rng.standard_normal((M, K)).astype(np.float32))))
+        y.zero_()
+        if rep == 0:
+            g.replay()              # (the runtime may set a graph up on its first launch)
+            torch.cuda.synchronize()
+        else:
+            with _no_device_allocation():
+                g.replay()
+        got = host_bits(y).copy()
+        y2 = torch.zeros_like(y)
+        mx.gemm(x, packed, N, mx.Epilogue(y2, mx.PP_BIAS | mx.PP_GELU, bias=bd), k_splits=S, ws=ws)
+        torch.cuda.synchronize()
+        assert np.array_equal(got, host_bits(y2)), rep
 
 
 def test_static_workspace_rejects_what_does_not_fit():
