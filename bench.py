@@ -689,7 +689,8 @@ def main():
         # so that no host time is in the figure, buffers rotated over 541 MB+ (more than the last-level cache holds).
         # The decode kernels are judged against the best of these:
         #   matvec:      the mat-vec kernel over key caches of the size of the decode weights (many short workgroups)
-        #   persistent:  a resident grid of 256 / 512 workgroups, each wave a rolling window of 8 / 16 / 32 KiB of loads
+        #   persistent:  a resident grid of 256 / 512 workgroups, each wave a rolling window of 8 / 16 / 32 KiB of loads, and
+        #                the two best grids of a wider sweep (688 x 4 waves and 344 x 8 waves, 2 KiB per wave)
         #   device_copy: the runtime's own device-to-device copy of as many bytes (reads AND writes them)
         def graph_us(launch, nl):
             for i in range(nl):
@@ -733,6 +734,13 @@ def main():
                     us = graph_us(lambda i: mx.probe_read(flat[i % ncopy][:share * grid], grid, kib, sink), ncopy * 10)
                     ent[f"persistent_{grid}wg_{kib}KiB"] = {"us": round(us, 2), "bytes": share * grid, "GBps": round(share * grid / us / 1e3),
                                                             "us_scaled_to_all_bytes": round(us * nbytes / (share * grid), 2)}
+            # the best grids of a sweep over workgroups x waves x bytes in flight: many small workgroups, little in flight each
+            for grid, waves, kib in ((688, 4, 2), (344, 8, 2)):
+                unit = waves * kib * 1024
+                share = nbytes // grid // unit * unit
+                us = graph_us(lambda i: mx.probe_read(flat[i % ncopy][:share * grid], grid, kib, sink, waves=waves), ncopy * 10)
+                ent[f"persistent_{grid}wg_{waves}waves_{kib}KiB"] = {"us": round(us, 2), "bytes": share * grid, "GBps": round(share * grid / us / 1e3),
+                                                                    "us_scaled_to_all_bytes": round(us * nbytes / (share * grid), 2)}
             dst = torch.empty_like(flat[0])
             us = graph_us(lambda i: dst.copy_(flat[i % ncopy]), ncopy * 10)
             ent["device_copy"] = {"us": round(us, 2), "GBps_read_plus_written": round(2 * nbytes / us / 1e3)}
