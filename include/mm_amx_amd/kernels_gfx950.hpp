@@ -289,6 +289,35 @@ inline PackedB<T> repackB_1x2(const tensor2D<T>& Bi, bool transpose = false, hip
     return p;
 }
 
+// repackB_1xL<T, L>(Bi, scale) (weight_compression/fc16m.cpp:61-99): the packed weights of the M <= 16 kernels from a
+// bf16 [K, N] matrix, as bf16 (scale 1, as everywhere in the reference) or compressed to int8 on the way: every weight
+// becomes int8_t(w * scale), the bf16 product rounded to nearest even and then truncated toward zero (:80-81; saturated
+// here where the reference's conversion is undefined).  L = 1..4 tiles of 16 columns side by side only orders the
+// reference's cache layout: its preconditions are kept (K a multiple of 32, N of 16 L), the result is this library's
+// fragment order.
+template <typename T, int L>
+inline PackedB<T> repackB_1xL(const tensor2D<bfloat16>& Bi, float scale = 1.0f, hipStream_t stream = nullptr) {
+    static_assert(L >= 1 && L <= 4, "L = 1 ... 4");
+    static_assert(std::is_same<T, bfloat16>::value || std::is_same<T, int8_t>::value, "T is bfloat16 or int8_t");
+    const int K = Bi.dims[0], N = Bi.dims[1];
+    require(K % 32 == 0, "repackB_1xL: K must be a multiple of 32");
+    require(N % (L * 16) == 0, "repackB_1xL: N must be a multiple of 16 L");
+    PackedB<T> p = alloc_packed<T>(K, N);
+    if (std::is_same<T, bfloat16>::value) {
+        require(scale == 1.0f, "repackB_1xL: a scale is for the int8 form only");
+        check(mmx_repack_b(MMX_BF16, Bi.data, Bi.stride, K, N, 0, p.data, stream), "repackB_1xL");
+        return p;
+    }
+    void* q = nullptr;  // the quantised matrix in source order, between the two kernels only
+    const size_t qbytes = static_cast<size_t>(K) * static_cast<size_t>(N);
+    check_hip(hipMalloc(&q, qbytes > 0 ? qbytes : 1), "repackB_1xL: hipMalloc");
+    std::shared_ptr<void> hold(q, [](void* x) { (void)hipFree(x); });
+    check(mmx_quantize_weights_scaled(Bi.data, Bi.stride, K, N, scale, q, N, stream), "repackB_1xL: quantise");
+    check(mmx_repack_b(MMX_I8, q, N, K, N, 0, p.data, stream), "repackB_1xL: pack");
+    check_hip(hipStreamSynchronize(stream), "repackB_1xL");  // (the temporary is freed on return)
+    return p;
+}
+
 // ---- workspace of the K split -------------------------------------------------------------------------
 // AMX_MLP::Linear keeps the partial results of its two K halves in per-thread buffers (work.C,
 // tests/amx-mlp.cpp:648-682); here the partial tiles of mmx_gemm_splitk live in one zero-initialised device

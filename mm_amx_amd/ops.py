@@ -71,6 +71,29 @@ def repackB_1x2(Bi, transpose=False):
     return L.repack_b(Bi, transpose)
 
 
+def repackB_1xL(Bi, dtype=torch.bfloat16, L_=2, scale=1.0):
+    """repackB_1xL<T, L>(Bi, scale) of weight_compression/fc16m.cpp:61-99: the packed form of the bf16 matrix Bi [K, N]
+    for the M <= 16 kernels, as bf16 (T = bfloat16, the scale must be 1 as everywhere in the reference) or compressed to
+    int8 on the way (T = int8_t: every weight becomes int8_t(w * scale), i.e. the bf16 product rounded to nearest even,
+    then truncated toward zero, :80-81; saturated here where the reference's conversion is undefined).  L (1..4 tiles of
+    16 columns side by side) only orders the reference's cache layout; the preconditions are kept (K a multiple of 32,
+    N of 16 L) and the result is this library's fragment order, which mmx_gemm takes as b_dtype bf16 or int8."""
+    if Bi.dtype != torch.bfloat16 or Bi.dim() != 2:
+        raise L.MmxError("repackB_1xL: Bi must be a bf16 [K, N] matrix")
+    if L_ not in (1, 2, 3, 4):
+        raise L.MmxError("repackB_1xL: L must be 1..4")
+    K, N = Bi.shape
+    if K % 32 or N % (L_ * 16):
+        raise L.MmxError(f"repackB_1xL: K = {K} must be a multiple of 32 and N = {N} of {L_ * 16} (fc16m.cpp:66-67)")
+    if dtype == torch.bfloat16:
+        if scale != 1.0:
+            raise L.MmxError("repackB_1xL: a scale is for the int8 form only")
+        return L.repack_b(Bi)
+    if dtype == torch.int8:
+        return L.repack_b(L.quantize_weights_scaled(Bi, float(scale)))
+    raise L.MmxError("repackB_1xL: T is bfloat16 or int8")
+
+
 class Matmul:
     """amx_kernel::Matmul<TA,TB,TC> (include/kernels_amx.hpp:1045-1315) and its dispatcher in
     main.cpp:32-80.  ``weight_int8=True`` gives Matmul<bf16,int8,float> (:1319-1516): the bf16 B is

@@ -3,6 +3,7 @@
 // naive product, :517-525 whole-N vs N-split, :884-885 MatmulVector shapes, :929 BiasGelu shape;
 // weight_compression/fc16m.cpp:749-759 decode shapes; torch-ext/test.py:35-37 LinearNxN shapes).
 // Needs one MI355X.  Exit status 0 = every case passed.  The oracle is linked here as the checker.
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -17,6 +18,7 @@
 using namespace gfx950_kernel;
 
 static int g_failed = 0;
+static bool throws(const std::function<void()>& f);
 #define EXPECT(cond, ...)                                    \
     do {                                                     \
         if (!(cond)) {                                       \
@@ -217,6 +219,42 @@ static void test_matmul_weight_int8(int M, int K, int N) {
     for (size_t i = 0; i < ref.size(); i++) ref[i] = acc[i] * dq;
     const Err e = compare(got, ref);
     EXPECT(e.fro <= 1e-3 && e.within >= 0.999, "rel Frobenius %.3e, %.3f%% within 1 bf16 ulp", e.fro, e.within * 100);
+}
+
+// ---- repackB_1xL<int8_t, 2>(B, scale): fc16m's own way to its int8 weights (weight_compression/fc16m.cpp:61-99, 123) ----
+static void test_repack_1xL(int M, int K, int N) {
+    std::printf("  repackB_1xL<int8_t,2>(B, 127/max|B|) + decode GEMM M=%d K=%d N=%d\n", M, K, N);
+    auto hA = rand_bf16(static_cast<size_t>(M) * K, 1.0f), hB = rand_bf16(static_cast<size_t>(K) * N, 0.05f);
+    float amax = 0.0f;
+    for (const auto& b : hB) amax = std::max(amax, std::fabs(static_cast<float>(b)));
+    const float scale = 127.0f / amax;  // quantize_i8_scale (fc16m.cpp:113-118)
+    tensor2D<bfloat16> A(M, K), B(K, N);
+    tensor2D<float> C(M, N);
+    A.upload(hA.data());
+    B.upload(hB.data());
+    PackedB<int8_t> Wp = repackB_1xL<int8_t, 2>(B, scale);
+    PP::BiasGeluStore<float, PP::DEQUANT> pp(C);
+    pp.set_deq_scale(1.0f / scale);
+    const mmx_epilogue e = pp.descriptor();
+    check(mmx_gemm(MMX_BF16, MMX_I8, A.data, A.stride, Wp.data, M, K, N, 0, N, &e, nullptr), "mmx_gemm");
+    check_hip(hipDeviceSynchronize(), "sync");
+    std::vector<float> got(static_cast<size_t>(M) * N);
+    C.download(got.data());
+
+    std::vector<int8_t> Wq(static_cast<size_t>(K) * N);
+    orc_quantize_scale_trunc(bits(hB), N, K, N, scale, Wq.data(), N);
+    std::vector<float> acc(got.size()), ref(got.size()), ones(N, 1.0f);
+    std::vector<uint16_t> ydummy(got.size());
+    orc_gemv_w8(bits(hA), K, Wq.data(), N, 0, ones.data(), ydummy.data(), N, acc.data(), M, K, N, 0);
+    const float dq = 1.0f / scale;
+    for (size_t i = 0; i < ref.size(); i++) ref[i] = acc[i] * dq;
+    const Err er = compare(got, ref);
+    EXPECT(er.fro <= 1e-3 && er.within >= 0.999, "rel Frobenius %.3e, %.3f%% within 1 bf16 ulp", er.fro, er.within * 100);
+    // the bf16 form is the plain pack; the preconditions are the reference's
+    PackedB<bfloat16> Wb = repackB_1xL<bfloat16, 4>(B);
+    EXPECT(Wb.bytes == mmx_packed_b_bytes(MMX_BF16, K, N), "bf16 form: %zu bytes", Wb.bytes);
+    tensor2D<bfloat16> Bodd(K, N + 16);
+    EXPECT(throws([&] { repackB_1xL<int8_t, 2>(Bodd, scale); }), "N = %d is not a multiple of 32: no error", N + 16);
 }
 
 // ---- MatmulW4: int4 weight compression inside the op (no reference counterpart beyond a timing stand-in) ----
@@ -441,6 +479,8 @@ int main() {
         test_matmul_weight_int8(160, 512, 256);   // large M: int8 fragments converted between LDS and the MFMA operand
         test_matmul_weight_int8(300, 200, 96);    // ... with a K tail (masked loads)
         test_matmul_weight_int8(24, 8192, 256);   // decode with few panels: K walked in slices through the stream's workspace
+        test_repack_1xL(2, 2560, 192);            // fc16m.cpp:749
+        test_repack_1xL(16, 512, 352);
         test_matmul_weight_int4(1, 4096, 352);
         test_matmul_weight_int4(7, 300, 77);
         test_matvec(901, 80);  // main.cpp:884

@@ -261,3 +261,20 @@ def test_bench_traffic_figures_belong_to_the_current_kernel_sources():
     spec.loader.exec_module(bench)
     for kernel in bench.MEASURED_TRAFFIC:
         assert bench.measured_traffic(kernel) is not None, f"{kernel}: its source changed after the traffic was measured"
+
+
+def test_repackB_1xL_checks_the_reference_preconditions():
+    """repackB_1xL asserts K % 32 == 0 and N % (16 L) == 0 (weight_compression/fc16m.cpp:66-67); here they raise, as do
+    a source that is not bf16, an L outside 1..4 and a scale on the bf16 form - all before anything reaches the library."""
+    import torch
+
+    import mm_amx_amd as mx
+    good = torch.zeros((64, 64), dtype=torch.bfloat16)
+    for bad_call in (lambda: mx.repackB_1xL(torch.zeros((48, 64), dtype=torch.bfloat16), torch.int8, 2, 2.0),
+                     lambda: mx.repackB_1xL(torch.zeros((64, 48), dtype=torch.bfloat16), torch.int8, 2, 2.0),
+                     lambda: mx.repackB_1xL(torch.zeros((64, 64), dtype=torch.float32), torch.int8, 2, 2.0),
+                     lambda: mx.repackB_1xL(good, torch.int8, 5, 2.0),
+                     lambda: mx.repackB_1xL(good, torch.bfloat16, 2, 2.0),
+                     lambda: mx.repackB_1xL(good, torch.float32, 2, 1.0)):
+        with pytest.raises(mx.MmxError):
+            bad_call()

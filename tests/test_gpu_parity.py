@@ -615,6 +615,29 @@ def test_scaled_truncating_quantiser(po, scale):
         check_float_parity(bf16_to_f32(host_bits(y)), bf16_to_f32(y_ref), f"fc16m int8 weights M={M}")
 
 
+def test_repackB_1xL_operator(po):
+    """repackB_1xL<T, L>(Bi, scale) of the operator surface (weight_compression/fc16m.cpp:61-99) on fc16m's own shape
+    (M = 2, K = 2560, N = 192, :749) and scale (127 / max|B|, :113-118): the int8 form is the oracle's quantiser followed
+    by the pack, bit for bit, and runs through the decode kernel with the per-tensor dequant 1 / scale; the bf16 form is
+    the plain pack."""
+    M, K, N = 2, 2560, 192
+    rng = np.random.default_rng(749)
+    B = rand_bf16(rng, (K, N), 0.05)
+    scale = float(np.float32(127.0) / np.abs(bf16_to_f32(B)).max())
+    Bd = dev_bf16(B)
+    Wq = po.quantize_scale_trunc(B, scale)
+    packed = mx.repackB_1xL(Bd, torch.int8, 2, scale)
+    assert np.array_equal(host_bits(packed), host_bits(mx.repack_b(dev(Wq))))
+    assert np.array_equal(host_bits(mx.repackB_1xL(Bd, torch.bfloat16, 4)), host_bits(mx.repack_b(Bd)))
+    x = rand_bf16(rng, (M, K), 1.0)
+    dq = np.float32(1.0) / np.float32(scale)
+    y_ref, _ = po.gemv_w8(x, Wq, np.full(N, dq, np.float32), want_acc=True)
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    mx.gemm(dev_bf16(x), packed, N, mx.Epilogue(y, mx.PP_DEQUANT, deq_scale=float(dq)), b_dtype=mx.I8)
+    assert "skinny" in mx.last_kernel()
+    check_float_parity(bf16_to_f32(host_bits(y)), bf16_to_f32(y_ref), "repackB_1xL<int8_t,2> + decode GEMM")
+
+
 @pytest.mark.parametrize("a_unsigned,b_unsigned", [(True, False), (False, True), (True, True)])
 @pytest.mark.parametrize("shape", [(5, 70, 40), (40, 256, 96), (200, 1024, 320), (16, 4096, 512)])
 def test_unsigned_byte_gemm(po, a_unsigned, b_unsigned, shape):
