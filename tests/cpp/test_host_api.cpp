@@ -251,7 +251,7 @@ static void test_repack_1xL(int M, int K, int N) {
     const Err er = compare(got, ref);
     EXPECT(er.fro <= 1e-3 && er.within >= 0.999, "rel Frobenius %.3e, %.3f%% within 1 bf16 ulp", er.fro, er.within * 100);
     // the bf16 form is the plain pack; the preconditions are the reference's
-    PackedB<bfloat16> Wb = repackB_1xL<bfloat16, 4>(B);
+    PackedB<bfloat16> Wb = repackB_1xL<bfloat16, 2>(B);
     EXPECT(Wb.bytes == mmx_packed_b_bytes(MMX_BF16, K, N), "bf16 form: %zu bytes", Wb.bytes);
     tensor2D<bfloat16> Bodd(K, N + 16);
     EXPECT(throws([&] { repackB_1xL<int8_t, 2>(Bodd, scale); }), "N = %d is not a multiple of 32: no error", N + 16);
