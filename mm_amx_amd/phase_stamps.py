@@ -4,8 +4,8 @@
 
 Each argument is  dtype,M,K,N,tile,k_splits[,waves]  (dtype bf16: the FC with BIAS+GELU and a bf16 store; i8: the int8 FC
 with DEQUANT+BIAS+QUANT and an int8 store; w8: bf16 activations on int8-compressed weights, DEQUANT, fp32 store; tile as for
-mmx_set_tile, empty = the library's choice; waves 4 or 8), or  gemv8,M,K,N  (decode: bf16 activations on int8 weights
-through the streaming kernel, weights rotated over 540 MB).  The instrumented library is built on first use (several
+mmx_set_tile, empty = the library's choice; waves 4 or 8), or  gemv8,M,K,N / gemv4,M,K,N  (decode: bf16 activations on
+int8 / int4 weights through the streaming kernel, weights rotated over 540 MB).  The instrumented library is built on first use (several
 minutes) and whenever a kernel source is newer than it.
 The instrumented library (libmm_amx_amd_stamps.so, -DMMX_STAMPS) makes thread 0 of every workgroup write the shader
 clock at its phase boundaries behind the K-split workspace; this module launches the shape, reads the stamps back and
@@ -95,26 +95,31 @@ def run(ws, dt, M, K, N, tile, S, waves=8, out=sys.stdout):
     print(line, file=out, flush=True)
 
 
-def run_decode(ws, M, K, N, out=sys.stdout):
+def run_decode(ws, M, K, N, out=sys.stdout, int4=False):
     """The streaming decode kernel's stamps: 0/7 wall clock at start/end, 1 start, 2 x in LDS, 3 end of the weight stream,
     4 after the barrier, 5 after the reduction and the store (shader clock)."""
-    W = mx.repack_b(torch.randint(-127, 128, (K, N), dtype=torch.int8, device="cuda"))
-    packs = [W] + [W.clone() for _ in range(max(2, int(540e6 // (K * N))) - 1)]
+    if int4:
+        W, deq = mx.quantize_pack_int4((torch.randn((K, N), device="cuda") * 0.05).to(torch.bfloat16))
+        wdt, wbytes = mx.I4, K * N // 2
+    else:
+        W = mx.repack_b(torch.randint(-127, 128, (K, N), dtype=torch.int8, device="cuda"))
+        wdt, wbytes = mx.I8, K * N
+    packs = [W] + [W.clone() for _ in range(max(2, int(540e6 // wbytes)) - 1)]
     x = torch.randn((M, K), device="cuda").to(torch.bfloat16)
     y = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
-    ep = mx.Epilogue(y, mx.PP_DEQUANT, deq_scale=1e-3)
+    ep = mx.Epilogue(y, mx.PP_DEQUANT, deq_scale_per_oc=deq) if int4 else mx.Epilogue(y, mx.PP_DEQUANT, deq_scale=1e-3)
     stamp_off = COUNTER_BYTES + STAMP_OFFSET
     mx.set_option("decode_resident", 0)
     mx.set_option("decode_valu", 0)
     try:
-        mx.time_gemm(x, packs, N, ep, 200, b_dtype=mx.I8, ws=ws)
-        ms = mx.time_gemm(x, packs, N, ep, 200, b_dtype=mx.I8, ws=ws)
+        mx.time_gemm(x, packs, N, ep, 200, b_dtype=wdt, ws=ws)
+        ms = mx.time_gemm(x, packs, N, ep, 200, b_dtype=wdt, ws=ws)
         kern = mx.last_kernel()
         torch.cuda.synchronize()
         for rep in range(4):                      # four launches in a row, the last one's stamps are read
             ws[stamp_off:].zero_()
             for i in range(4):
-                mx.gemm(x, packs[(rep * 4 + i) % len(packs)], N, ep, b_dtype=mx.I8, ws=ws)
+                mx.gemm(x, packs[(rep * 4 + i) % len(packs)], N, ep, b_dtype=wdt, ws=ws)
             torch.cuda.synchronize()
     finally:
         mx.set_option("decode_resident", -1)
@@ -122,7 +127,7 @@ def run_decode(ws, M, K, N, out=sys.stdout):
     st = ws[stamp_off:].view(torch.int64).cpu().numpy().reshape(-1, 8)
     st = st[st[:, 0] != 0]
     if not len(st):
-        print(f"== gemv8 {M}x{K}x{N} {kern}: {ms * 1e3:.2f} us/launch, no stamps (this kernel is not instrumented)", file=out)
+        print(f"== {'gemv4' if int4 else 'gemv8'} {M}x{K}x{N} {kern}: {ms * 1e3:.2f} us/launch, no stamps (this kernel is not instrumented)", file=out)
         return
     t0 = st[:, 0].min()
     start, end = (st[:, 0] - t0) / 100.0, (st[:, 7] - t0) / 100.0
@@ -130,7 +135,7 @@ def run_decode(ws, M, K, N, out=sys.stdout):
 
     def d(a, b):
         return np.median(st[:, b] - st[:, a])
-    print(f"== gemv8 {M}x{K}x{N} {kern}: {ms * 1e3:.2f} us/launch, {len(st)} workgroups, clock ~{ghz:.2f} GHz", file=out)
+    print(f"== {'gemv4' if int4 else 'gemv8'} {M}x{K}x{N} {kern}: {ms * 1e3:.2f} us/launch, {len(st)} workgroups, clock ~{ghz:.2f} GHz", file=out)
     print(f"   workgroup start after the first: median {np.median(start):.2f} max {start.max():.2f} us; life median "
           f"{np.median(end - start):.2f} max {(end - start).max():.2f} us; last end {end.max():.2f} us", file=out)
     print(f"   cycles, median: start->x in LDS {d(1, 2):.0f}   weight stream + products {d(2, 3):.0f}   barrier {d(3, 4):.0f}   "
@@ -156,8 +161,8 @@ def main(argv):
     ws = torch.zeros(COUNTER_BYTES + STAMP_OFFSET + STAMP_BYTES, dtype=torch.uint8, device="cuda")
     for a in argv:
         parts = a.split(",")
-        if parts[0] == "gemv8":
-            run_decode(ws, int(parts[1]), int(parts[2]), int(parts[3]))
+        if parts[0] in ("gemv8", "gemv4"):
+            run_decode(ws, int(parts[1]), int(parts[2]), int(parts[3]), int4=parts[0] == "gemv4")
             continue
         dt, M, K, N, tile, S = parts[:6]
         run(ws, dt, int(M), int(K), int(N), tile, int(S), waves=int(parts[6]) if len(parts) > 6 else 8)
