@@ -49,12 +49,9 @@ __global__ __launch_bounds__(256) void u8_colsum_kernel(const char* __restrict__
     colsum[n - n0] = sum;
 }
 
-// acc (int32 [M, ld]) + correction terms -> post-op -> C: the steps and order of the tile kernels' store
-__global__ __launch_bounds__(256) void u8_finish_kernel(const int32_t* __restrict__ acc, int64_t ldacc, const int32_t* rowsum,
-                                                        const int32_t* colsum, int32_t both_term, int M, int n0, int n1,
-                                                        const Epilogue ep) {
-    const int n = n0 + blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
-    if (n >= n1 || m >= M) return;
+// one element of the result: int32 sum + correction terms -> post-op -> C
+__device__ __forceinline__ void u8_finish_one(const int32_t* __restrict__ acc, int64_t ldacc, const int32_t* rowsum, const int32_t* colsum,
+                                              int32_t both_term, int m, int n, int n0, const Epilogue& ep) {
     uint32_t v = (uint32_t)acc[(int64_t)m * ldacc + n];
     if (colsum) v += 128u * (uint32_t)colsum[n - n0];
     if (rowsum) v += 128u * (uint32_t)rowsum[m];
@@ -75,6 +72,16 @@ __global__ __launch_bounds__(256) void u8_finish_kernel(const int32_t* __restric
     case MMX_I8: reinterpret_cast<int8_t*>(row)[n] = to_s8_sat(r); break;
     default: reinterpret_cast<float*>(row)[n] = r; break;
     }
+}
+
+// acc (int32 [M, ld]) + correction terms -> post-op -> C: the steps and order of the tile kernels' store; a thread per
+// column, rows blockIdx.y, blockIdx.y + gridDim.y, ... (the grid's second dimension holds 65535 at most)
+__global__ __launch_bounds__(256) void u8_finish_kernel(const int32_t* __restrict__ acc, int64_t ldacc, const int32_t* rowsum,
+                                                        const int32_t* colsum, int32_t both_term, int M, int n0, int n1,
+                                                        const Epilogue ep) {
+    const int n = n0 + blockIdx.x * 256 + threadIdx.x;
+    if (n >= n1) return;
+    for (int m = blockIdx.y; m < M; m += gridDim.y) u8_finish_one(acc, ldacc, rowsum, colsum, both_term, m, n, n0, ep);
 }
 
 // c[m] = sum_k A[m, k] b[k] with either operand signed or unsigned: one wave per row
@@ -123,7 +130,7 @@ int launch_gemm_x8(bool a_unsigned, bool b_unsigned, const void* A, int64_t lda,
     rc = signed_gemm(a_unsigned ? static_cast<const void*>(As) : A, a_unsigned ? lds_ : lda, Bp, M, K, N, n0, n1, acc, (int64_t)n1 * 4, st);
     if (rc) return rc;
     const int32_t both = (a_unsigned && b_unsigned) ? (int32_t)(16384u * (uint32_t)K) : 0;
-    hipLaunchKernelGGL(u8_finish_kernel, dim3((n1 - n0 + 255) / 256, M), dim3(256), 0, st, acc, (int64_t)n1, b_unsigned ? rowsum : nullptr,
+    hipLaunchKernelGGL(u8_finish_kernel, dim3((n1 - n0 + 255) / 256, M < 65535 ? M : 65535), dim3(256), 0, st, acc, (int64_t)n1, b_unsigned ? rowsum : nullptr,
                        a_unsigned ? colsum : nullptr, both, M, n0, n1, ep);
     return check_hip(hipGetLastError(), "u8_finish_kernel launch");
 }

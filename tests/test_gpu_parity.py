@@ -639,7 +639,7 @@ def test_repackB_1xL_operator(po):
 
 
 @pytest.mark.parametrize("a_unsigned,b_unsigned", [(True, False), (False, True), (True, True)])
-@pytest.mark.parametrize("shape", [(5, 70, 40), (40, 256, 96), (200, 1024, 320), (16, 4096, 512)])
+@pytest.mark.parametrize("shape", [(5, 70, 40), (40, 256, 96), (200, 1024, 320), (16, 4096, 512), (66000, 64, 32)])  # (more rows than a grid dimension holds)
 def test_unsigned_byte_gemm(po, a_unsigned, b_unsigned, shape):
     """The uint8_t forms of Matmul (tdpbusd / tdpbsud / tdpbuud, include/kernels_amx.hpp:1057-1101) through mmx_gemm_u8:
     raw int32 sums bit-exact against the oracle (pinned to the reference's Matmul<uint8_t,int8_t> and to int64
