@@ -278,3 +278,13 @@ def test_repackB_1xL_checks_the_reference_preconditions():
                      lambda: mx.repackB_1xL(good, torch.float32, 2, 1.0)):
         with pytest.raises(mx.MmxError):
             bad_call()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU: --gpus above 1 exits with a message that says so, before anything touches a device."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in r.stderr and "--gpus must be 1" in r.stderr
+    assert not r.stdout.strip()
