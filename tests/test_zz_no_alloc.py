@@ -25,7 +25,7 @@ def _no_device_allocation():
     yield
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == torch0
-    assert torch.cuda.mem_get_info()[0] == free0, (free0, torch.cuda.mem_get_info()[0])
+    assert torch.cuda.mem_get_info()[0] >= free0, (free0, torch.cuda.mem_get_info()[0])   # (an allocation would lower it)
 
 
 def _int8_case(po, M, K, N, seed, k_splits, ws):
